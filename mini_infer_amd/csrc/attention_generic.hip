@@ -1,0 +1,244 @@
+// Paged causal attention, plain-FMA version: the float32 path of the engine and
+// the fallback for sizes the matrix-core kernels refuse.  One 64-lane wave per
+// (query token, key/value head, up to 4 query heads of its group, key split).
+// Lanes own keys while scores are computed (one key row per lane, q broadcast
+// from LDS) and own output dims while values are accumulated.  Scores, softmax
+// and the value sum are float32 with an online (running max) softmax.
+//
+// Semantics follow the reference's oracle (cache/packed_attention.py:296-338):
+// query head h reads key/value head h / (Hq/Hkv); a query at absolute position p
+// sees keys 0..p, or p-window+1..p with a window.
+//
+// Layout: q rows [token][head][head_dim] with a row stride; pages
+// [num_pages][kv_heads][page_size][head_dim]; block_table[request][i] is the page
+// of that request's keys i*page_size .. (i+1)*page_size-1.
+#include "common.h"
+
+#include <math.h>
+
+#define GT 4  // query heads handled together by one wave
+
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Pack {
+  T v[N];
+};
+
+template <typename T, int VPL>
+__global__ __launch_bounds__(64) void attn_generic_kernel(
+    const T* __restrict__ q, int64_t q_row_stride, const T* __restrict__ k_pages,
+    const T* __restrict__ v_pages, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ token_request, const int* __restrict__ positions, T* __restrict__ out,
+    int64_t out_row_stride, float* __restrict__ part_acc, float* __restrict__ part_ml, int q_heads,
+    int kv_heads, int head_dim, int page_size, float scale, int window, int num_splits) {
+  extern __shared__ float q_lds[];  // [GT][head_dim], pre-multiplied by the scale
+  constexpr int KV = 16 / sizeof(T);  // elements in a 16-byte load
+
+  const int t = blockIdx.x;
+  const int group = q_heads / kv_heads;
+  const int head_blocks = (group + GT - 1) / GT;
+  const int kvh = blockIdx.y / head_blocks;
+  const int g0 = (blockIdx.y % head_blocks) * GT;
+  const int nh = min(GT, group - g0);
+  const int head0 = kvh * group + g0;
+  const int split = blockIdx.z;
+  const int lane = threadIdx.x;
+
+  const T* q_row = q + (int64_t)t * q_row_stride + (int64_t)head0 * head_dim;
+  for (int i = lane; i < GT * head_dim; i += MI_WAVE)
+    q_lds[i] = (i < nh * head_dim) ? to_f32(q_row[i]) * scale : 0.f;
+  __syncthreads();
+
+  const int pos = positions[t];
+  const int req = token_request[t];
+  const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
+  const int hi = pos + 1;
+  int chunk = (hi - lo + num_splits - 1) / num_splits;
+  chunk = (chunk + MI_WAVE - 1) / MI_WAVE * MI_WAVE;
+  const int a = lo + split * chunk;
+  const int b = min(a + chunk, hi);
+  const int* bt = block_table + (int64_t)req * max_blocks;
+
+  float m[GT], l[GT], acc[GT][VPL];
+#pragma unroll
+  for (int g = 0; g < GT; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.f;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) acc[g][v] = 0.f;
+  }
+  const bool owns_dims = lane * VPL < head_dim;
+
+  for (int base = a; base < b; base += MI_WAVE) {
+    const int key = base + lane;
+    const bool valid = key < b;
+    int row_idx = 0;
+    float s[GT];
+#pragma unroll
+    for (int g = 0; g < GT; ++g) s[g] = -INFINITY;
+    if (valid) {
+      const int page = bt[key / page_size];
+      row_idx = (page * kv_heads + kvh) * page_size + key % page_size;
+      const T* k_row = k_pages + (int64_t)row_idx * head_dim;
+#pragma unroll
+      for (int g = 0; g < GT; ++g) s[g] = 0.f;
+      for (int d = 0; d < head_dim; d += KV) {
+        const Pack<T, KV> kk = *reinterpret_cast<const Pack<T, KV>*>(k_row + d);
+#pragma unroll
+        for (int e = 0; e < KV; ++e) {
+          const float kf = to_f32(kk.v[e]);
+#pragma unroll
+          for (int g = 0; g < GT; ++g) s[g] += q_lds[g * head_dim + d + e] * kf;
+        }
+      }
+    }
+    float p[GT];
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      const float m_new = fmaxf(m[g], wave_max(s[g]));
+      const float alpha = expf(m[g] - m_new);
+      p[g] = valid ? expf(s[g] - m_new) : 0.f;
+      l[g] = l[g] * alpha + wave_sum(p[g]);
+#pragma unroll
+      for (int v = 0; v < VPL; ++v) acc[g][v] *= alpha;
+      m[g] = m_new;
+    }
+    const int n_valid = min(MI_WAVE, b - base);
+    for (int j = 0; j < n_valid; ++j) {
+      const int rj = __shfl(row_idx, j, MI_WAVE);
+      float vv[VPL];
+#pragma unroll
+      for (int v = 0; v < VPL; ++v) vv[v] = 0.f;
+      if (owns_dims) {
+        const Pack<T, VPL> pk =
+            *reinterpret_cast<const Pack<T, VPL>*>(v_pages + (int64_t)rj * head_dim + lane * VPL);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) vv[v] = to_f32(pk.v[v]);
+      }
+#pragma unroll
+      for (int g = 0; g < GT; ++g) {
+        const float pj = __shfl(p[g], j, MI_WAVE);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) acc[g][v] += pj * vv[v];
+      }
+    }
+  }
+
+  if (num_splits == 1) {
+    if (owns_dims) {
+#pragma unroll
+      for (int g = 0; g < GT; ++g) {
+        if (g < nh) {
+          T* o = out + (int64_t)t * out_row_stride + (int64_t)(head0 + g) * head_dim + lane * VPL;
+          const float inv = 1.f / l[g];
+#pragma unroll
+          for (int v = 0; v < VPL; ++v) o[v] = from_f32<T>(acc[g][v] * inv);
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      if (g < nh) {
+        const int64_t slot = ((int64_t)t * q_heads + head0 + g) * num_splits + split;
+        if (owns_dims) {
+#pragma unroll
+          for (int v = 0; v < VPL; ++v) part_acc[slot * head_dim + lane * VPL + v] = acc[g][v];
+        }
+        if (lane == 0) {
+          part_ml[slot * 2] = m[g];
+          part_ml[slot * 2 + 1] = l[g];
+        }
+      }
+    }
+  }
+}
+
+// Combine the splits of one (token, head) in a fixed order.
+template <typename T>
+__global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict__ part_acc,
+                                                         const float* __restrict__ part_ml,
+                                                         T* __restrict__ out, int64_t out_row_stride,
+                                                         int q_heads, int head_dim, int num_splits) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int64_t base = ((int64_t)t * q_heads + h) * num_splits;
+  float m_all = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) m_all = fmaxf(m_all, part_ml[(base + s) * 2]);
+  float l_all = 0.f;
+  for (int s = 0; s < num_splits; ++s)
+    l_all += part_ml[(base + s) * 2 + 1] * expf(part_ml[(base + s) * 2] - m_all);
+  const float inv = 1.f / l_all;
+  for (int d = threadIdx.x; d < head_dim; d += MI_WAVE) {
+    float o = 0.f;
+    for (int s = 0; s < num_splits; ++s)
+      o += part_acc[(base + s) * head_dim + d] * expf(part_ml[(base + s) * 2] - m_all);
+    out[(int64_t)t * out_row_stride + (int64_t)h * head_dim + d] = from_f32<T>(o * inv);
+  }
+}
+
+template <typename T>
+static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* k_pages,
+                               const void* v_pages, const int* block_table, int max_blocks,
+                               const int* token_request, const int* positions, void* out,
+                               int64_t out_row_stride, float* part_acc, float* part_ml,
+                               int num_tokens, int q_heads, int kv_heads, int head_dim,
+                               int page_size, float scale, int window, int num_splits,
+                               hipStream_t stream) {
+  const int group = q_heads / kv_heads;
+  dim3 grid(num_tokens, kv_heads * ceil_div(group, GT), num_splits);
+  const size_t lds = sizeof(float) * GT * head_dim;
+#define MI_ATTN_LAUNCH(VPL)                                                                       \
+  attn_generic_kernel<T, VPL><<<grid, MI_WAVE, lds, stream>>>(                                    \
+      (const T*)q, q_row_stride, (const T*)k_pages, (const T*)v_pages, block_table, max_blocks,   \
+      token_request, positions, (T*)out, out_row_stride, part_acc, part_ml, q_heads, kv_heads,    \
+      head_dim, page_size, scale, window, num_splits)
+  if (head_dim <= 64) MI_ATTN_LAUNCH(1);
+  else if (head_dim <= 128) MI_ATTN_LAUNCH(2);
+  else MI_ATTN_LAUNCH(4);
+#undef MI_ATTN_LAUNCH
+  MI_CHECK_LAUNCH("attn_generic");
+  if (num_splits > 1) {
+    dim3 rgrid(num_tokens, q_heads);
+    attn_reduce_kernel<T><<<rgrid, MI_WAVE, 0, stream>>>(part_acc, part_ml, (T*)out, out_row_stride,
+                                                         q_heads, head_dim, num_splits);
+    MI_CHECK_LAUNCH("attn_reduce");
+  }
+  return MI_OK;
+}
+
+// part_acc holds num_tokens*q_heads*num_splits*head_dim floats and part_ml
+// num_tokens*q_heads*num_splits*2 floats; both may be null when num_splits == 1.
+extern "C" int mi_attn_generic(int dtype, const void* q, int64_t q_row_stride, const void* k_pages,
+                               const void* v_pages, const int* block_table, int max_blocks,
+                               const int* token_request, const int* positions, void* out,
+                               int64_t out_row_stride, float* part_acc, float* part_ml,
+                               int num_tokens, int q_heads, int kv_heads, int head_dim,
+                               int page_size, int num_pages, float scale, int window,
+                               int num_splits, hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && q_heads > 0 && kv_heads > 0, "attn_generic: bad sizes tokens=%d q_heads=%d kv_heads=%d",
+             num_tokens, q_heads, kv_heads);
+  MI_REQUIRE(q_heads % kv_heads == 0, "attn_generic: q_heads=%d is not a multiple of kv_heads=%d",
+             q_heads, kv_heads);
+  MI_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
+             "attn_generic: head_dim=%d must be a multiple of 16 and at most 256", head_dim);
+  MI_REQUIRE(page_size > 0 && num_pages > 0 && max_blocks > 0, "attn_generic: bad page sizes page_size=%d num_pages=%d max_blocks=%d",
+             page_size, num_pages, max_blocks);
+  MI_REQUIRE((int64_t)num_pages * kv_heads * page_size < (int64_t)1 << 31,
+             "attn_generic: the cache has too many key rows for 32-bit row indices");
+  MI_REQUIRE(window >= 0, "attn_generic: window=%d must be 0 (none) or positive", window);
+  MI_REQUIRE(num_splits >= 1 && num_splits <= 65535, "attn_generic: num_splits=%d out of range", num_splits);
+  MI_REQUIRE(num_splits == 1 || (part_acc && part_ml), "attn_generic: split keys need partial buffers");
+  MI_REQUIRE(q_row_stride >= (int64_t)q_heads * head_dim && out_row_stride >= (int64_t)q_heads * head_dim,
+             "attn_generic: row strides shorter than q_heads*head_dim");
+  MI_REQUIRE(kv_heads * ceil_div(q_heads / kv_heads, GT) <= 65535, "attn_generic: too many heads");
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "attn_generic: unknown dtype %d", dtype);
+  if (num_tokens == 0) return MI_OK;
+  if (dtype == MI_F32)
+    return attn_generic_launch<float>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
+                                      token_request, positions, out, out_row_stride, part_acc, part_ml,
+                                      num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
+                                      num_splits, stream);
+  return attn_generic_launch<bf16_t>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
+                                     token_request, positions, out, out_row_stride, part_acc, part_ml,
+                                     num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
+                                     num_splits, stream);
+}

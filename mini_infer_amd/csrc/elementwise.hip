@@ -1,0 +1,335 @@
+// Per-token kernels: embedding lookup, residual add + RMSNorm, rotation tables,
+// rotary position encoding fused with the write of keys and values into cache
+// pages, and SiLU(gate) * up.  All arithmetic is float32; storage is float32 or
+// bfloat16.  The residual stream is float32 in both modes.
+//
+// Formulas follow the reference (JonathanBerhe/mini-infer, src/mini_infer/):
+//   RMSNorm           models/blocks/rmsnorm.py:81-93, rms_norm_kernel.py:98-144
+//   rotation          models/blocks/rope.py:392-431, rope_write_kernel.py:119-152
+//   SiLU * up         models/blocks/silu_mul_kernel.py:86-90
+// but round once at the end instead of after every operation.
+#include "common.h"
+
+#include <math.h>
+
+typedef bf16_t bf16x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void load4(const float* p, float v[4]) {
+  const float4 x = *reinterpret_cast<const float4*>(p);
+  v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float v[4]) {
+  const bf16x4_t x = *reinterpret_cast<const bf16x4_t*>(p);
+  v[0] = (float)x[0]; v[1] = (float)x[1]; v[2] = (float)x[2]; v[3] = (float)x[3];
+}
+__device__ __forceinline__ void store4(float* p, const float v[4]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float v[4]) {
+  bf16x4_t x;
+  x[0] = (bf16_t)v[0]; x[1] = (bf16_t)v[1]; x[2] = (bf16_t)v[2]; x[3] = (bf16_t)v[3];
+  *reinterpret_cast<bf16x4_t*>(p) = x;
+}
+
+// ---------------------------------------------------------------------------
+// embedding: residual[t, :] = float(table[ids[t], :])
+// ---------------------------------------------------------------------------
+
+template <typename T, int VEC>
+__global__ void embed_gather_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                    float* __restrict__ residual, int hidden) {
+  const int t = blockIdx.x;
+  const T* row = table + (int64_t)ids[t] * hidden;
+  float* out = residual + (int64_t)t * hidden;
+  if (VEC == 4) {
+    for (int i = threadIdx.x * 4; i < hidden; i += blockDim.x * 4) {
+      float v[4];
+      load4(row + i, v);
+      store4(out + i, v);
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = to_f32(row[i]);
+  }
+}
+
+template <typename T>
+static int embed_gather_launch(const void* table, const int* ids, float* residual, int num_tokens,
+                               int hidden, hipStream_t stream) {
+  if (num_tokens == 0) return MI_OK;
+  if (hidden % 4 == 0) {
+    embed_gather_kernel<T, 4><<<num_tokens, 256, 0, stream>>>((const T*)table, ids, residual, hidden);
+  } else {
+    embed_gather_kernel<T, 1><<<num_tokens, 256, 0, stream>>>((const T*)table, ids, residual, hidden);
+  }
+  MI_CHECK_LAUNCH("embed_gather");
+  return MI_OK;
+}
+
+extern "C" int mi_embed_gather(int dtype, const void* table, const int* ids, float* residual,
+                               int num_tokens, int hidden, int vocab, hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && hidden > 0 && vocab > 0,
+             "embed_gather: bad sizes tokens=%d hidden=%d vocab=%d", num_tokens, hidden, vocab);
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "embed_gather: unknown dtype %d", dtype);
+  if (dtype == MI_F32) return embed_gather_launch<float>(table, ids, residual, num_tokens, hidden, stream);
+  return embed_gather_launch<bf16_t>(table, ids, residual, num_tokens, hidden, stream);
+}
+
+// ---------------------------------------------------------------------------
+// residual add + RMSNorm
+//   s = residual[r] + delta[r]           (float32; stored back unless `rows` is given)
+//   out[b] = weight * s * rsqrt(mean(s^2) + eps)
+// One block per output row; with `rows`, output row b reads input row rows[b].
+// ---------------------------------------------------------------------------
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(
+    const T* __restrict__ delta, float* __restrict__ residual, const T* __restrict__ weight,
+    T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
+  __shared__ float scratch[4];
+  const int b = blockIdx.x;
+  const int64_t r = rows ? rows[b] : b;
+  float* res = residual + r * hidden;
+  const T* dl = delta ? delta + r * hidden : nullptr;
+  T* o = out + (int64_t)b * hidden;
+  const bool store_sum = (rows == nullptr) && (delta != nullptr);
+
+  float sumsq = 0.f;
+  if (VEC == 4) {
+    for (int i = threadIdx.x * 4; i < hidden; i += blockDim.x * 4) {
+      float s[4];
+      load4(res + i, s);
+      if (dl) {
+        float d[4];
+        load4(dl + i, d);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) s[k] += d[k];
+        if (store_sum) store4(res + i, s);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) sumsq += s[k] * s[k];
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      float s = res[i];
+      if (dl) {
+        s += to_f32(dl[i]);
+        if (store_sum) res[i] = s;
+      }
+      sumsq += s * s;
+    }
+  }
+  const float total = block_sum(sumsq, scratch);
+  const float inv = rsqrtf(total / (float)hidden + eps);
+  const bool re_add = (dl != nullptr) && !store_sum;
+
+  if (VEC == 4) {
+    for (int i = threadIdx.x * 4; i < hidden; i += blockDim.x * 4) {
+      float s[4], w[4];
+      load4(res + i, s);
+      if (re_add) {
+        float d[4];
+        load4(dl + i, d);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) s[k] += d[k];
+      }
+      load4(weight + i, w);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) s[k] = w[k] * (s[k] * inv);
+      store4(o + i, s);
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      float s = res[i];
+      if (re_add) s += to_f32(dl[i]);
+      o[i] = from_f32<T>(to_f32(weight[i]) * (s * inv));
+    }
+  }
+}
+
+template <typename T>
+static int add_rmsnorm_launch(const void* delta, float* residual, const void* weight, void* out,
+                              const int* rows, int num_out_rows, int hidden, float eps,
+                              hipStream_t stream) {
+  if (num_out_rows == 0) return MI_OK;
+  if (hidden % 4 == 0) {
+    add_rmsnorm_kernel<T, 4><<<num_out_rows, 256, 0, stream>>>(
+        (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps);
+  } else {
+    add_rmsnorm_kernel<T, 1><<<num_out_rows, 256, 0, stream>>>(
+        (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps);
+  }
+  MI_CHECK_LAUNCH("add_rmsnorm");
+  return MI_OK;
+}
+
+extern "C" int mi_add_rmsnorm(int dtype, const void* delta, float* residual, const void* weight,
+                              void* out, const int* rows, int num_out_rows, int hidden, float eps,
+                              hipStream_t stream) {
+  MI_REQUIRE(num_out_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d hidden=%d",
+             num_out_rows, hidden);
+  MI_REQUIRE(eps > 0.f, "add_rmsnorm: eps must be positive, got %g", (double)eps);
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "add_rmsnorm: unknown dtype %d", dtype);
+  if (dtype == MI_F32)
+    return add_rmsnorm_launch<float>(delta, residual, weight, out, rows, num_out_rows, hidden, eps, stream);
+  return add_rmsnorm_launch<bf16_t>(delta, residual, weight, out, rows, num_out_rows, hidden, eps, stream);
+}
+
+// ---------------------------------------------------------------------------
+// rotation tables: angle = float(position) * inv_freq[j]; cos and sin in float32
+// ---------------------------------------------------------------------------
+
+__global__ void rope_table_kernel(const int* __restrict__ positions,
+                                  const float* __restrict__ inv_freq, float* __restrict__ cos_t,
+                                  float* __restrict__ sin_t, int half) {
+  const int t = blockIdx.x;
+  const float pos = (float)positions[t];
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    const float angle = pos * inv_freq[j];
+    float s, c;
+    sincosf(angle, &s, &c);
+    cos_t[(int64_t)t * half + j] = c;
+    sin_t[(int64_t)t * half + j] = s;
+  }
+}
+
+extern "C" int mi_rope_table(const int* positions, const float* inv_freq, float* cos_t,
+                             float* sin_t, int num_tokens, int half, hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && half > 0, "rope_table: bad sizes tokens=%d half=%d", num_tokens, half);
+  if (num_tokens == 0) return MI_OK;
+  rope_table_kernel<<<num_tokens, 64, 0, stream>>>(positions, inv_freq, cos_t, sin_t, half);
+  MI_CHECK_LAUNCH("rope_table");
+  return MI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// rotary encoding of q (in place) and k, and the write of k and v into pages.
+//   row layout of qkv: [q heads | k heads | v heads], each head `head_dim` wide.
+//   pairing: half rotation pairs dim j with j + rotary_dim/2; interleaved pairs
+//   2j with 2j+1.  Dims at and beyond rotary_dim pass through.
+//   pages: [num_pages, kv_heads, page_size, head_dim]; slot = page*page_size + offset;
+//   a negative slot writes nothing.
+// ---------------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(
+    T* __restrict__ qkv, int64_t row_stride, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, const int* __restrict__ slot_mapping, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int q_heads, int kv_heads, int head_dim, int rotary_dim,
+    int interleaved, int page_size) {
+  const int t = blockIdx.x;
+  const int half = rotary_dim / 2;
+  T* row = qkv + (int64_t)t * row_stride;
+  const float* c = cos_t + (int64_t)t * half;
+  const float* s = sin_t + (int64_t)t * half;
+
+  for (int e = threadIdx.x; e < q_heads * half; e += blockDim.x) {
+    const int h = e / half, j = e % half;
+    const int i0 = interleaved ? 2 * j : j;
+    const int i1 = interleaved ? 2 * j + 1 : j + half;
+    T* x = row + h * head_dim;
+    const float x0 = to_f32(x[i0]), x1 = to_f32(x[i1]);
+    x[i0] = from_f32<T>(x0 * c[j] - x1 * s[j]);
+    x[i1] = from_f32<T>(x1 * c[j] + x0 * s[j]);
+  }
+
+  if (kv_heads == 0 || slot_mapping == nullptr) return;
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;
+  const int page = slot / page_size, off = slot % page_size;
+  const T* k_row = row + (int64_t)q_heads * head_dim;
+  const T* v_row = k_row + (int64_t)kv_heads * head_dim;
+
+  for (int e = threadIdx.x; e < kv_heads * half; e += blockDim.x) {
+    const int h = e / half, j = e % half;
+    const int i0 = interleaved ? 2 * j : j;
+    const int i1 = interleaved ? 2 * j + 1 : j + half;
+    const T* x = k_row + h * head_dim;
+    T* dst = k_pages + (((int64_t)page * kv_heads + h) * page_size + off) * head_dim;
+    const float x0 = to_f32(x[i0]), x1 = to_f32(x[i1]);
+    dst[i0] = from_f32<T>(x0 * c[j] - x1 * s[j]);
+    dst[i1] = from_f32<T>(x1 * c[j] + x0 * s[j]);
+  }
+  const int pass = head_dim - rotary_dim;
+  for (int e = threadIdx.x; e < kv_heads * pass; e += blockDim.x) {
+    const int h = e / pass, d = rotary_dim + e % pass;
+    k_pages[(((int64_t)page * kv_heads + h) * page_size + off) * head_dim + d] = k_row[h * head_dim + d];
+  }
+  for (int e = threadIdx.x; e < kv_heads * head_dim; e += blockDim.x) {
+    const int h = e / head_dim, d = e % head_dim;
+    v_pages[(((int64_t)page * kv_heads + h) * page_size + off) * head_dim + d] = v_row[h * head_dim + d];
+  }
+}
+
+extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const float* cos_t,
+                                const float* sin_t, const int* slot_mapping, void* k_pages,
+                                void* v_pages, int num_tokens, int q_heads, int kv_heads,
+                                int head_dim, int rotary_dim, int interleaved, int page_size,
+                                int num_pages, hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && q_heads >= 0 && kv_heads >= 0 && head_dim > 0,
+             "rope_kv_write: bad sizes tokens=%d q_heads=%d kv_heads=%d head_dim=%d", num_tokens,
+             q_heads, kv_heads, head_dim);
+  MI_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
+             "rope_kv_write: rotary_dim=%d must be even and at most head_dim=%d", rotary_dim, head_dim);
+  MI_REQUIRE(row_stride >= (int64_t)(q_heads + 2 * kv_heads) * head_dim,
+             "rope_kv_write: row stride %lld is shorter than (q+2kv)*head_dim", (long long)row_stride);
+  MI_REQUIRE(kv_heads == 0 || slot_mapping == nullptr || (page_size > 0 && num_pages > 0 && k_pages && v_pages),
+             "rope_kv_write: pages are needed to write keys and values");
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "rope_kv_write: unknown dtype %d", dtype);
+  if (num_tokens == 0) return MI_OK;
+  if (dtype == MI_F32) {
+    rope_kv_write_kernel<float><<<num_tokens, 256, 0, stream>>>(
+        (float*)qkv, row_stride, cos_t, sin_t, slot_mapping, (float*)k_pages, (float*)v_pages,
+        q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size);
+  } else {
+    rope_kv_write_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
+        (bf16_t*)qkv, row_stride, cos_t, sin_t, slot_mapping, (bf16_t*)k_pages, (bf16_t*)v_pages,
+        q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size);
+  }
+  MI_CHECK_LAUNCH("rope_kv_write");
+  return MI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i],  silu(g) = g / (1 + exp(-g))
+// ---------------------------------------------------------------------------
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ gate_up,
+                                                       T* __restrict__ out, int inter) {
+  const int t = blockIdx.x;
+  const T* g = gate_up + (int64_t)t * 2 * inter;
+  const T* u = g + inter;
+  T* o = out + (int64_t)t * inter;
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
+  if (i >= inter) return;
+  if (VEC == 4) {
+    float gv[4], uv[4];
+    load4(g + i, gv);
+    load4(u + i, uv);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) gv[k] = gv[k] / (1.f + expf(-gv[k])) * uv[k];
+    store4(o + i, gv);
+  } else {
+    const float gv = to_f32(g[i]);
+    o[i] = from_f32<T>(gv / (1.f + expf(-gv)) * to_f32(u[i]));
+  }
+}
+
+extern "C" int mi_silu_mul(int dtype, const void* gate_up, void* out, int num_tokens, int inter,
+                           hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && inter > 0, "silu_mul: bad sizes tokens=%d inter=%d", num_tokens, inter);
+  MI_REQUIRE(ceil_div(inter, 256) <= 65535, "silu_mul: intermediate size %d is too large", inter);
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "silu_mul: unknown dtype %d", dtype);
+  if (num_tokens == 0) return MI_OK;
+  const int vec = (inter % 4 == 0) ? 4 : 1;
+  dim3 grid(num_tokens, ceil_div(inter, 256 * vec));
+  if (dtype == MI_F32) {
+    if (vec == 4) silu_mul_kernel<float, 4><<<grid, 256, 0, stream>>>((const float*)gate_up, (float*)out, inter);
+    else silu_mul_kernel<float, 1><<<grid, 256, 0, stream>>>((const float*)gate_up, (float*)out, inter);
+  } else {
+    if (vec == 4) silu_mul_kernel<bf16_t, 4><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, inter);
+    else silu_mul_kernel<bf16_t, 1><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, inter);
+  }
+  MI_CHECK_LAUNCH("silu_mul");
+  return MI_OK;
+}

@@ -1,0 +1,89 @@
+// True float32 matrix product for the 32-bit path: C[M,N] = A[M,K] * W[N,K]^T.
+// Plain FMA, no reduced-precision matrix mode.  Each output element is summed by
+// one thread over k = 0..K-1 in order, so a row's result does not depend on how
+// many other rows are in the batch or on where its tile lies.
+//
+// 64x64 output tile per 256-thread block, 16-deep K slices staged in LDS, 4x4
+// outputs per thread.  Any M, N, K; rows of A and W may have strides.
+#include "common.h"
+
+#define BM 64
+#define BN 64
+#define BK 16
+
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ a, int64_t lda,
+                                                       const float* __restrict__ w, int64_t ldw,
+                                                       float* __restrict__ c, int64_t ldc, int m,
+                                                       int n, int k) {
+  __shared__ float a_s[BK][BM + 4];
+  __shared__ float w_s[BK][BN + 4];
+
+  const int tid = threadIdx.x;
+  const int row0 = blockIdx.y * BM;
+  const int col0 = blockIdx.x * BN;
+  const int ty = tid / 16, tx = tid % 16;
+
+  // loader mapping: thread loads 4 consecutive k of one row
+  const int l_row = tid / 4;
+  const int l_k = (tid % 4) * 4;
+
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  for (int k0 = 0; k0 < k; k0 += BK) {
+    {
+      const int r = row0 + l_row;
+      const float* src = a + (int64_t)r * lda + k0 + l_k;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        a_s[l_k + i][l_row] = (r < m && k0 + l_k + i < k) ? src[i] : 0.f;
+    }
+    {
+      const int r = col0 + l_row;
+      const float* src = w + (int64_t)r * ldw + k0 + l_k;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        w_s[l_k + i][l_row] = (r < n && k0 + l_k + i < k) ? src[i] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float av[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = a_s[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wv[j] = w_s[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = row0 + ty * 4 + i;
+    if (r >= m) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = col0 + tx * 4 + j;
+      if (col < n) c[(int64_t)r * ldc + col] = acc[i][j];
+    }
+  }
+}
+
+extern "C" int mi_gemm_f32(const float* a, int64_t lda, const float* w, int64_t ldw, float* c,
+                           int64_t ldc, int m, int n, int k, hipStream_t stream) {
+  MI_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_f32: bad sizes m=%d n=%d k=%d", m, n, k);
+  MI_REQUIRE(lda >= k && ldw >= k && ldc >= n, "gemm_f32: a row stride is shorter than its row");
+  MI_REQUIRE(ceil_div(m, BM) <= 65535, "gemm_f32: m=%d is too large for one call", m);
+  if (m == 0) return MI_OK;
+  dim3 grid(ceil_div(n, BN), ceil_div(m, BM));
+  gemm_f32_kernel<<<grid, 256, 0, stream>>>(a, lda, w, ldw, c, ldc, m, n, k);
+  MI_CHECK_LAUNCH("gemm_f32");
+  return MI_OK;
+}

@@ -1,0 +1,258 @@
+// Next-token choice on the device: one 1024-thread block per row of logits.
+//
+// Meaning of the options follows the reference (engine/sampler.py:24-110):
+//   temperature 0      first index of the maximum
+//   temperature > 0    logits / temperature, then
+//   top_k in (0, V)    values below the k-th largest value are dropped (ties stay)
+//   top_p < 1          a token is dropped when the probability mass of the tokens
+//                      above it exceeds top_p (the boundary token stays)
+//   draw               argmax of p_i / q_i with q_i ~ Exp(1), here in log form
+//                      x_i - log(q_i)
+// Unlike the reference's global generator, the random numbers come from a
+// counter-based generator (Philox 4x32-10) keyed by the request's seed and the
+// index of the draw, so a request's tokens do not depend on what else is in the
+// batch.  Thresholds are found without sorting, by descending over the bytes of
+// an order-preserving integer image of the values; probability mass is summed in
+// 64-bit fixed point so the result does not depend on the order of the sum.
+#include "common.h"
+
+#include <math.h>
+
+#define SAMPLE_THREADS 1024
+#define SAMPLE_WAVES (SAMPLE_THREADS / MI_WAVE)
+#define MASS_ONE 1099511627776.0f  // 2^40
+
+__device__ __forceinline__ uint32_t order_key(float x) {
+  const uint32_t u = __float_as_uint(x);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__device__ __forceinline__ void philox4x32_10(uint32_t c[4], uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
+    const uint32_t n1 = (uint32_t)p1;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
+    const uint32_t n3 = (uint32_t)p0;
+    c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+}
+
+// -log(-log(u)) for u uniform in (0, 1), from 24 random bits
+__device__ __forceinline__ float gumbel_from_bits(uint32_t bits) {
+  const float u = ((float)(bits >> 8) + 0.5f) * (1.0f / 16777216.0f);
+  return -logf(-logf(u));
+}
+
+struct ArgBest {
+  float val;
+  int idx;
+};
+
+__device__ __forceinline__ ArgBest better(ArgBest a, ArgBest b) {
+  // larger value wins; equal values: smaller index wins
+  if (b.val > a.val || (b.val == a.val && b.idx < a.idx)) return b;
+  return a;
+}
+
+__device__ ArgBest block_argbest(ArgBest mine, ArgBest* scratch) {
+#pragma unroll
+  for (int off = MI_WAVE / 2; off > 0; off >>= 1) {
+    ArgBest other;
+    other.val = __shfl_xor(mine.val, off, MI_WAVE);
+    other.idx = __shfl_xor(mine.idx, off, MI_WAVE);
+    mine = better(mine, other);
+  }
+  const int wave = threadIdx.x / MI_WAVE, lane = threadIdx.x % MI_WAVE;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = mine;
+  __syncthreads();
+  ArgBest best = scratch[0];
+  for (int w = 1; w < SAMPLE_WAVES; ++w) best = better(best, scratch[w]);
+  return best;
+}
+
+template <typename T>
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
+    const T* __restrict__ logits, int64_t row_stride, int vocab,
+    const float* __restrict__ temperature, const int* __restrict__ top_k,
+    const float* __restrict__ top_p, const uint32_t* __restrict__ seed_lo,
+    const uint32_t* __restrict__ seed_hi, const uint32_t* __restrict__ draw_index,
+    int* __restrict__ out) {
+  __shared__ ArgBest best_scratch[SAMPLE_WAVES];
+  __shared__ uint32_t cnt[256];
+  __shared__ unsigned long long mass[256];
+  __shared__ uint32_t sh_prefix;
+  __shared__ unsigned long long sh_above;
+  __shared__ unsigned long long sh_limit;
+
+  const int row = blockIdx.x;
+  const int tid = threadIdx.x;
+  const T* x = logits + (int64_t)row * row_stride;
+  const float temp = temperature[row];
+
+  if (temp == 0.f) {
+    ArgBest mine = {-INFINITY, 0x7fffffff};
+    for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+      const float v = to_f32(x[i]);
+      if (v > mine.val || mine.idx == 0x7fffffff) { mine.val = v; mine.idx = i; }
+    }
+    const ArgBest best = block_argbest(mine, best_scratch);
+    if (tid == 0) out[row] = best.idx;
+    return;
+  }
+
+  // maximum of the scaled logits
+  ArgBest top = {-INFINITY, 0x7fffffff};
+  for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+    const float v = to_f32(x[i]) / temp;
+    if (v > top.val) { top.val = v; top.idx = i; }
+  }
+  const float v_max = block_argbest(top, best_scratch).val;
+
+  uint32_t key_floor = 0;  // tokens whose key is below this are dropped
+
+  // ---- top-k: the key of the k-th largest value ---------------------------
+  const int k = top_k[row];
+  if (k > 0 && k < vocab) {
+    uint32_t prefix = 0, mask = 0;
+    uint32_t remaining = (uint32_t)k;
+    for (int pass = 0; pass < 4; ++pass) {
+      const int shift = 24 - 8 * pass;
+      if (tid < 256) cnt[tid] = 0;
+      __syncthreads();
+      int run_bin = -1;
+      uint32_t run_cnt = 0;
+      for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+        const uint32_t key = order_key(to_f32(x[i]) / temp);
+        if ((key & mask) != prefix) continue;
+        const int bin = (key >> shift) & 255;
+        if (bin != run_bin) {
+          if (run_cnt) atomicAdd(&cnt[run_bin], run_cnt);
+          run_bin = bin;
+          run_cnt = 0;
+        }
+        ++run_cnt;
+      }
+      if (run_cnt) atomicAdd(&cnt[run_bin], run_cnt);
+      __syncthreads();
+      if (tid == 0) {
+        int bin = 255;
+        for (; bin > 0; --bin) {
+          if (remaining <= cnt[bin]) break;
+          remaining -= cnt[bin];
+        }
+        sh_prefix = prefix | ((uint32_t)bin << shift);
+        sh_above = remaining;
+      }
+      __syncthreads();
+      prefix = sh_prefix;
+      remaining = (uint32_t)sh_above;
+      mask |= 255u << shift;
+      __syncthreads();
+    }
+    key_floor = prefix;
+  }
+
+  // ---- top-p: the smallest key whose mass-above is within top_p ------------
+  const float p = top_p[row];
+  if (p < 1.f) {
+    uint32_t prefix = 0, mask = 0;
+    unsigned long long above = 0;
+    for (int pass = 0; pass < 4; ++pass) {
+      const int shift = 24 - 8 * pass;
+      if (tid < 256) { cnt[tid] = 0; mass[tid] = 0; }
+      __syncthreads();
+      int run_bin = -1;
+      uint32_t run_cnt = 0;
+      unsigned long long run_mass = 0;
+      for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+        const float v = to_f32(x[i]) / temp;
+        const uint32_t key = order_key(v);
+        if (key < key_floor || (key & mask) != prefix) continue;
+        const int bin = (key >> shift) & 255;
+        if (bin != run_bin) {
+          if (run_cnt) { atomicAdd(&cnt[run_bin], run_cnt); atomicAdd(&mass[run_bin], run_mass); }
+          run_bin = bin;
+          run_cnt = 0;
+          run_mass = 0;
+        }
+        ++run_cnt;
+        run_mass += (unsigned long long)(expf(v - v_max) * MASS_ONE);
+      }
+      if (run_cnt) { atomicAdd(&cnt[run_bin], run_cnt); atomicAdd(&mass[run_bin], run_mass); }
+      __syncthreads();
+      if (tid == 0) {
+        if (pass == 0) {
+          unsigned long long total = 0;
+          for (int b = 0; b < 256; ++b) total += mass[b];
+          sh_limit = (unsigned long long)((double)p * (double)total);
+        }
+        const unsigned long long limit = sh_limit;
+        unsigned long long run = above, chosen_above = above;
+        int chosen = -1;
+        for (int b = 255; b >= 0; --b) {
+          if (cnt[b] > 0) {
+            if (run <= limit || chosen < 0) { chosen = b; chosen_above = run; }
+            else break;
+          }
+          run += mass[b];
+        }
+        sh_prefix = prefix | ((uint32_t)chosen << shift);
+        sh_above = chosen_above;
+      }
+      __syncthreads();
+      prefix = sh_prefix;
+      above = sh_above;
+      mask |= 255u << shift;
+      __syncthreads();
+    }
+    if (prefix > key_floor) key_floor = prefix;
+  }
+
+  // ---- draw -----------------------------------------------------------------
+  const uint32_t k0 = seed_lo[row], k1 = seed_hi[row], draw = draw_index[row];
+  ArgBest mine = {-INFINITY, 0x7fffffff};
+  const int n_quads = (vocab + 3) / 4;
+  for (int quad = tid; quad < n_quads; quad += SAMPLE_THREADS) {
+    uint32_t c[4] = {(uint32_t)quad, draw, 0u, 0u};
+    philox4x32_10(c, k0, k1);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int i = quad * 4 + e;
+      if (i >= vocab) break;
+      const float v = to_f32(x[i]) / temp;
+      if (order_key(v) < key_floor) continue;
+      const float score = v + gumbel_from_bits(c[e]);
+      if (score > mine.val || mine.idx == 0x7fffffff) { mine.val = score; mine.idx = i; }
+    }
+  }
+  const ArgBest best = block_argbest(mine, best_scratch);
+  if (tid == 0) out[row] = best.idx;
+}
+
+extern "C" int mi_sample(int dtype, const void* logits, int64_t row_stride, int num_rows, int vocab,
+                         const float* temperature, const int* top_k, const float* top_p,
+                         const uint32_t* seed_lo, const uint32_t* seed_hi,
+                         const uint32_t* draw_index, int* out, hipStream_t stream) {
+  MI_REQUIRE(num_rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", num_rows, vocab);
+  MI_REQUIRE(row_stride >= vocab, "sample: row stride %lld is shorter than the vocabulary %d",
+             (long long)row_stride, vocab);
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "sample: unknown dtype %d", dtype);
+  if (num_rows == 0) return MI_OK;
+  if (dtype == MI_F32) {
+    sample_kernel<float><<<num_rows, SAMPLE_THREADS, 0, stream>>>(
+        (const float*)logits, row_stride, vocab, temperature, top_k, top_p, seed_lo, seed_hi,
+        draw_index, out);
+  } else {
+    sample_kernel<bf16_t><<<num_rows, SAMPLE_THREADS, 0, stream>>>(
+        (const bf16_t*)logits, row_stride, vocab, temperature, top_k, top_p, seed_lo, seed_hi,
+        draw_index, out);
+  }
+  MI_CHECK_LAUNCH("sample");
+  return MI_OK;
+}

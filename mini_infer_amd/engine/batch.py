@@ -1,0 +1,19 @@
+"""What one step is asked to run."""
+
+from __future__ import annotations
+
+import dataclasses
+from typing import Hashable, Sequence
+
+
+@dataclasses.dataclass
+class StepEntry:
+    """A request's next tokens, and the places among them whose logits are wanted.
+
+    A portion of a prompt (any length, cut anywhere) or a single decoded token.
+    `want` indexes into `tokens`; it is empty for a portion in the middle of a prompt.
+    """
+
+    request_id: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()

@@ -1,0 +1,232 @@
+"""The runner: a loaded model, its cache, and the one step function.
+
+`ModelRunner.from_pretrained` mirrors the reference's constructor of the same
+name (engine/model_runner.py:84-175: model folder, `dtype`, `num_blocks`,
+`block_size`).  `step` is the single primitive (the reference's
+`forward_step_packed`, engine/model_runner.py:270-395): a flattened batch of
+prompt portions beside single decoded tokens, run from the cache, returning
+logits only at the wanted places.
+"""
+
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Any, Hashable, Sequence
+
+import numpy as np
+import torch
+
+from mini_infer_amd.cache.manager import CacheManager
+from mini_infer_amd.config import DEFAULT_BLOCK_SIZE, DEFAULT_NUM_BLOCKS, read_config_json
+from mini_infer_amd.engine.batch import StepEntry
+from mini_infer_amd.models import DecoderModel, architecture_for
+from mini_infer_amd.parts.base import StepContext
+from mini_infer_amd.weights import load_checkpoint
+from mini_infer_amd.weights.random_init import fill_random_on_device
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+def resolve_dtype(dtype: str | torch.dtype | None) -> torch.dtype:
+    if dtype is None:
+        return torch.bfloat16
+    if isinstance(dtype, torch.dtype):
+        if dtype not in _DTYPES.values():
+            raise ValueError(f"dtype must be bfloat16 or float32, got {dtype}")
+        return dtype
+    if dtype not in _DTYPES:
+        raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, got {dtype!r}")
+    return _DTYPES[dtype]
+
+
+def require_gpu(device: str | torch.device) -> torch.device:
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError(
+            "mini_infer_amd runs on an AMD GPU through its HIP kernels; there is no CPU path "
+            f"(asked for {device}, torch.cuda.is_available()={torch.cuda.is_available()})"
+        )
+    return device
+
+
+class ModelRunner:
+    def __init__(
+        self,
+        model: DecoderModel,
+        config: Any,
+        *,
+        num_blocks: int = DEFAULT_NUM_BLOCKS,
+        block_size: int = DEFAULT_BLOCK_SIZE,
+        max_concurrent: int = 16,
+    ) -> None:
+        self.model = model
+        self.config = config
+        self.dtype = model.dtype
+        self.device = model.device
+        self.vocab_size = model.spec.vocab_size
+        self.block_size = block_size
+        self.num_blocks = num_blocks
+        self.cache = CacheManager(
+            model.cache_needs(),
+            page_size=block_size,
+            num_pages=num_blocks,
+            max_requests=max_concurrent,
+            dtype=model.dtype,
+            device=model.device,
+        )
+        self._layer_caches = self.cache.layer_caches()
+
+    # -- construction -----------------------------------------------------------
+
+    @classmethod
+    def from_pretrained(
+        cls,
+        model_name: str | Path,
+        *,
+        device: str = "cuda:0",
+        dtype: str | torch.dtype | None = None,
+        num_blocks: int = DEFAULT_NUM_BLOCKS,
+        block_size: int = DEFAULT_BLOCK_SIZE,
+        max_concurrent: int = 16,
+    ) -> "ModelRunner":
+        """Load the model folder `model_name` (config.json + safetensors) and build its cache."""
+        dev = require_gpu(device)
+        raw = read_config_json(model_name)
+        arch = architecture_for(raw)
+        config = arch.parse_config(raw)
+        model = DecoderModel(arch.build_spec(config), resolve_dtype(dtype), dev)
+        load_checkpoint(model, model_name)
+        return cls(model, config, num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent)
+
+    @classmethod
+    def from_random(
+        cls,
+        raw_config: dict[str, Any],
+        seed: int,
+        *,
+        device: str = "cuda:0",
+        dtype: str | torch.dtype | None = None,
+        num_blocks: int = DEFAULT_NUM_BLOCKS,
+        block_size: int = DEFAULT_BLOCK_SIZE,
+        max_concurrent: int = 16,
+        std: float = 0.02,
+        norm_jitter: float = 0.0,
+    ) -> "ModelRunner":
+        """Random weights made on the device (no file): for sizes too large to write out."""
+        dev = require_gpu(device)
+        arch = architecture_for(raw_config)
+        config = arch.parse_config(raw_config)
+        model = DecoderModel(arch.build_spec(config), resolve_dtype(dtype), dev)
+        fill_random_on_device(model, seed, std=std, norm_jitter=norm_jitter)
+        return cls(model, config, num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent)
+
+    # -- requests ---------------------------------------------------------------
+
+    def add_request(self, request_id: Hashable) -> None:
+        self.cache.add_request(request_id)
+
+    def has_request(self, request_id: Hashable) -> bool:
+        return self.cache.has_request(request_id)
+
+    def free_request(self, request_id: Hashable) -> None:
+        self.cache.free_request(request_id)
+
+    def num_free_blocks(self) -> int:
+        return min(self.cache.num_free_pages(g.index) for g in self.cache.groups) if self.cache.groups else 0
+
+    # -- the step ---------------------------------------------------------------
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run the given tokens as one batch from the cache; logits [wanted, vocab] float32.
+
+        Rows come in the order of `entries` and, within an entry, of its `want`.
+        Requests seen for the first time are admitted.  Raises `OutOfMemoryError`
+        before anything changes if the pages for this step are not there.
+        """
+        entries = [e for e in entries if len(e.tokens) > 0]
+        if not entries:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        seen: set[Hashable] = set()
+        for entry in entries:
+            if entry.request_id in seen:
+                raise ValueError(f"request {entry.request_id!r} appears twice in one step")
+            seen.add(entry.request_id)
+            for w in entry.want:
+                if not 0 <= w < len(entry.tokens):
+                    raise ValueError(
+                        f"request {entry.request_id!r}: wanted place {w} is outside its {len(entry.tokens)} tokens"
+                    )
+        token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+        if token_ids.min() < 0 or token_ids.max() >= self.vocab_size:
+            raise ValueError(f"token ids must lie in 0..{self.vocab_size - 1}")
+
+        admitted: list[Hashable] = []
+        try:
+            for entry in entries:
+                if not self.cache.has_request(entry.request_id):
+                    self.cache.add_request(entry.request_id)
+                    admitted.append(entry.request_id)
+            extents = {e.request_id: len(e.tokens) for e in entries}
+            self.cache.reserve(extents)
+        except Exception:
+            for request_id in admitted:
+                self.cache.free_request(request_id)
+            raise
+
+        index = self.cache.build_step_index([(e.request_id, len(e.tokens)) for e in entries])
+        rows = np.fromiter(
+            (int(index.cu_seqlens_q[b]) + w for b, e in enumerate(entries) for w in e.want),
+            dtype=np.int32,
+        )
+        ctx = self._to_device(token_ids.astype(np.int32), rows, index)
+        logits = self.model.forward(ctx, self._layer_caches)
+        self.cache.commit(extents)
+        return logits
+
+    def _to_device(self, token_ids: np.ndarray, rows: np.ndarray, index) -> StepContext:
+        """All of a step's integers in one pinned buffer and one copy to the device."""
+        pieces = [
+            token_ids,
+            index.positions,
+            index.token_request,
+            index.cu_seqlens_q,
+            index.seq_lens,
+            index.state_slots,
+            rows,
+        ]
+        for mapping, table in zip(index.slot_mapping, index.block_tables):
+            pieces.append(mapping)
+            pieces.append(table.reshape(-1))
+        sizes = [int(p.size) for p in pieces]
+        staging = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=True)
+        host = staging.numpy()
+        offset = 0
+        for piece, size in zip(pieces, sizes):
+            host[offset : offset + size] = piece
+            offset += size
+        on_device = staging.to(self.device, non_blocking=True)
+        views = list(torch.split(on_device, sizes))
+        token_ids_d, positions, token_request, cu, seq_lens, state_slots, rows_d = views[:7]
+        slot_mapping, block_tables = [], []
+        for g, table in enumerate(index.block_tables):
+            slot_mapping.append(views[7 + 2 * g])
+            block_tables.append(views[8 + 2 * g].view(table.shape))
+        return StepContext(
+            num_tokens=int(token_ids.size),
+            num_requests=len(index.request_ids),
+            page_size=self.block_size,
+            token_ids=token_ids_d,
+            positions=positions,
+            token_request=token_request,
+            cu_seqlens_q=cu,
+            seq_lens=seq_lens,
+            state_slots=state_slots,
+            logit_rows=rows_d,
+            slot_mapping=slot_mapping,
+            block_tables=block_tables,
+            max_q_len=index.max_q_len,
+            max_seq_len=index.max_seq_len,
+            host_cu_seqlens_q=index.cu_seqlens_q.tolist(),
+            host_seq_lens=index.seq_lens.tolist(),
+            host_state_slots=index.state_slots.tolist(),
+        )

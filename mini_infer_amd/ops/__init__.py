@@ -1,0 +1,27 @@
+"""The hand-written HIP kernels of the engine, as functions on torch tensors."""
+
+from mini_infer_amd.ops.kernels import (
+    add_rmsnorm,
+    attention_splits,
+    embed_gather,
+    gemm_f32,
+    linear,
+    paged_attention,
+    rope_kv_write,
+    rope_table,
+    sample,
+    silu_mul,
+)
+
+__all__ = [
+    "add_rmsnorm",
+    "attention_splits",
+    "embed_gather",
+    "gemm_f32",
+    "linear",
+    "paged_attention",
+    "rope_kv_write",
+    "rope_table",
+    "sample",
+    "silu_mul",
+]

@@ -1,0 +1,352 @@
+"""Thin wrappers that hand torch tensors to the HIP entry points.
+
+Each wrapper checks device, dtype and layout on the host, passes raw pointers and
+the current HIP stream, and raises with the library's message when a kernel
+refuses a size.  There is no CPU path: a CPU tensor is an error.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from mini_infer_amd.exceptions import KernelShapeError
+from mini_infer_amd.ops import library
+
+F32, BF16 = 0, 1
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise KernelShapeError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}")
+
+
+def _need_cuda(*tensors: torch.Tensor | None) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "mini_infer_amd kernels run on the GPU only (there is no CPU fallback); "
+                f"got a tensor on {t.device}"
+            )
+
+
+def _need_contiguous(name: str, t: torch.Tensor | None) -> None:
+    if t is not None and not t.is_contiguous():
+        raise KernelShapeError(f"{name} must be contiguous, got strides {t.stride()}")
+
+
+def _need_int32(name: str, t: torch.Tensor | None) -> None:
+    if t is not None and t.dtype != torch.int32:
+        raise KernelShapeError(f"{name} must be int32, got {t.dtype}")
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+# ----------------------------------------------------------------------------
+
+
+def embed_gather(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """`float32(table[ids])`: the start of the residual stream, [T, H] float32."""
+    _need_cuda(table, ids)
+    _need_contiguous("table", table)
+    _need_contiguous("ids", ids)
+    _need_int32("ids", ids)
+    vocab, hidden = table.shape
+    out = torch.empty((ids.numel(), hidden), dtype=torch.float32, device=table.device)
+    lib = library.load()
+    library.check(
+        lib.mi_embed_gather(
+            _dtype_code(table), _ptr(table), _ptr(ids), _ptr(out), ids.numel(), hidden, vocab,
+            _stream(),
+        )
+    )
+    return out
+
+
+def add_rmsnorm(
+    delta: torch.Tensor | None,
+    residual: torch.Tensor,
+    weight: torch.Tensor,
+    eps: float,
+    rows: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """`residual += delta` in float32 (kept unless `rows`), then RMSNorm times `weight`.
+
+    Returns [T, H] (or [len(rows), H]) in the dtype of `weight`.
+    """
+    _need_cuda(delta, residual, weight, rows)
+    _need_contiguous("residual", residual)
+    _need_contiguous("delta", delta)
+    _need_contiguous("weight", weight)
+    _need_contiguous("rows", rows)
+    _need_int32("rows", rows)
+    if residual.dtype != torch.float32:
+        raise KernelShapeError(f"the residual stream is float32, got {residual.dtype}")
+    tokens, hidden = residual.shape
+    if weight.shape != (hidden,):
+        raise KernelShapeError(f"norm weight has shape {tuple(weight.shape)}, expected ({hidden},)")
+    if delta is not None and (delta.shape != residual.shape or delta.dtype != weight.dtype):
+        raise KernelShapeError(
+            f"delta {tuple(delta.shape)} {delta.dtype} does not fit residual "
+            f"{tuple(residual.shape)} and weight dtype {weight.dtype}"
+        )
+    n_out = tokens if rows is None else rows.numel()
+    out = torch.empty((n_out, hidden), dtype=weight.dtype, device=residual.device)
+    lib = library.load()
+    library.check(
+        lib.mi_add_rmsnorm(
+            _dtype_code(weight), _ptr(delta), _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows),
+            n_out, hidden, float(eps), _stream(),
+        )
+    )
+    return out
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """`cos, sin` of `position * inv_freq`, both [T, len(inv_freq)] float32."""
+    _need_cuda(positions, inv_freq)
+    _need_contiguous("positions", positions)
+    _need_contiguous("inv_freq", inv_freq)
+    _need_int32("positions", positions)
+    if inv_freq.dtype != torch.float32:
+        raise KernelShapeError(f"inv_freq stays float32, got {inv_freq.dtype}")
+    tokens, half = positions.numel(), inv_freq.numel()
+    cos = torch.empty((tokens, half), dtype=torch.float32, device=positions.device)
+    sin = torch.empty_like(cos)
+    lib = library.load()
+    library.check(
+        lib.mi_rope_table(_ptr(positions), _ptr(inv_freq), _ptr(cos), _ptr(sin), tokens, half, _stream())
+    )
+    return cos, sin
+
+
+def rope_kv_write(
+    qkv: torch.Tensor,
+    cos: torch.Tensor,
+    sin: torch.Tensor,
+    slot_mapping: torch.Tensor | None,
+    k_pages: torch.Tensor | None,
+    v_pages: torch.Tensor | None,
+    *,
+    q_heads: int,
+    kv_heads: int,
+    head_dim: int,
+    rotary_dim: int,
+    interleaved: bool = False,
+) -> None:
+    """Rotate q in place inside `qkv`; rotate k and write k, v into their page slots.
+
+    `qkv` is [T, (q_heads + 2*kv_heads) * head_dim] (rows may be strided); pages are
+    [num_pages, kv_heads, page_size, head_dim].  `kv_heads=0` rotates q only.
+    """
+    _need_cuda(qkv, cos, sin, slot_mapping, k_pages, v_pages)
+    _need_contiguous("cos", cos)
+    _need_contiguous("sin", sin)
+    _need_contiguous("slot_mapping", slot_mapping)
+    _need_contiguous("k_pages", k_pages)
+    _need_contiguous("v_pages", v_pages)
+    _need_int32("slot_mapping", slot_mapping)
+    if qkv.dim() != 2 or qkv.stride(1) != 1:
+        raise KernelShapeError(f"qkv must be [T, width] with unit inner stride, got {qkv.stride()}")
+    tokens = qkv.shape[0]
+    if qkv.shape[1] < (q_heads + 2 * kv_heads) * head_dim:
+        raise KernelShapeError(
+            f"qkv rows hold {qkv.shape[1]} values, fewer than (q+2kv)*head_dim = "
+            f"{(q_heads + 2 * kv_heads) * head_dim}"
+        )
+    if cos.shape != (tokens, rotary_dim // 2) or sin.shape != cos.shape or cos.dtype != torch.float32:
+        raise KernelShapeError(
+            f"cos/sin must be float32 [{tokens}, {rotary_dim // 2}], got {tuple(cos.shape)} {cos.dtype}"
+        )
+    page_size = num_pages = 0
+    if kv_heads > 0 and slot_mapping is not None:
+        if k_pages is None or v_pages is None:
+            raise KernelShapeError("writing keys and values needs k_pages and v_pages")
+        if k_pages.dtype != qkv.dtype or v_pages.dtype != qkv.dtype:
+            raise KernelShapeError(f"pages are {k_pages.dtype}, activations {qkv.dtype}")
+        if k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != head_dim:
+            raise KernelShapeError(
+                f"pages must be [num_pages, {kv_heads}, page_size, {head_dim}], got {tuple(k_pages.shape)}"
+            )
+        if v_pages.shape != k_pages.shape:
+            raise KernelShapeError("k_pages and v_pages differ in shape")
+        if slot_mapping.numel() != tokens:
+            raise KernelShapeError(f"slot_mapping has {slot_mapping.numel()} entries for {tokens} tokens")
+        num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
+    lib = library.load()
+    library.check(
+        lib.mi_rope_kv_write(
+            _dtype_code(qkv), _ptr(qkv), qkv.stride(0), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
+            _ptr(k_pages), _ptr(v_pages), tokens, q_heads, kv_heads, head_dim, rotary_dim,
+            int(interleaved), page_size, num_pages, _stream(),
+        )
+    )
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """`silu(gate) * up` for rows laid out [gate | up]; returns [T, I]."""
+    _need_cuda(gate_up)
+    _need_contiguous("gate_up", gate_up)
+    tokens, width = gate_up.shape
+    if width % 2 != 0:
+        raise KernelShapeError(f"gate_up rows must hold gate and up halves, got width {width}")
+    out = torch.empty((tokens, width // 2), dtype=gate_up.dtype, device=gate_up.device)
+    lib = library.load()
+    library.check(
+        lib.mi_silu_mul(_dtype_code(gate_up), _ptr(gate_up), _ptr(out), tokens, width // 2, _stream())
+    )
+    return out
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """`a @ w.T` in true float32: a [M, K], w [N, K] -> [M, N]."""
+    _need_cuda(a, w)
+    if a.dtype != torch.float32 or w.dtype != torch.float32:
+        raise KernelShapeError(f"gemm_f32 takes float32, got {a.dtype} and {w.dtype}")
+    if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
+        raise KernelShapeError(f"gemm_f32: shapes {tuple(a.shape)} and {tuple(w.shape)} do not fit")
+    if a.stride(1) != 1 or w.stride(1) != 1:
+        raise KernelShapeError("gemm_f32: rows must have unit inner stride")
+    m, k = a.shape
+    n = w.shape[0]
+    c = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    lib = library.load()
+    library.check(
+        lib.mi_gemm_f32(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(c), c.stride(0), m, n, k, _stream())
+    )
+    return c
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """`x @ weight.T` without bias.
+
+    float32 runs the hand-written true-float32 kernel.  bfloat16 goes to the
+    vendor GEMM library through torch, as the reference's engine does
+    (distributed/linear.py:167, `F.linear` -> the vendor BLAS).
+    """
+    if x.dtype == torch.float32:
+        return gemm_f32(x, weight)
+    _need_cuda(x, weight)
+    return torch.matmul(x, weight.t())
+
+
+def attention_splits(num_tokens: int, q_heads: int, kv_heads: int, max_seq_len: int) -> int:
+    """How many key ranges each (token, head group) is cut into to fill the GPU."""
+    group = q_heads // kv_heads
+    work_items = max(1, num_tokens * kv_heads * math.ceil(group / 4))
+    target = 2048  # waves wanted in flight: 256 CUs x 8
+    by_fill = max(1, target // work_items)
+    by_len = max(1, max_seq_len // 256)
+    return int(min(by_fill, by_len, 64))
+
+
+def paged_attention(
+    q: torch.Tensor,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    block_table: torch.Tensor,
+    token_request: torch.Tensor,
+    positions: torch.Tensor,
+    *,
+    q_heads: int,
+    kv_heads: int,
+    head_dim: int,
+    scale: float,
+    window: int | None,
+    max_seq_len: int,
+) -> torch.Tensor:
+    """Causal attention of every token over its request's pages; returns [T, q_heads*head_dim].
+
+    `q` is [T, >= q_heads*head_dim] with the rotated queries in its first columns
+    (rows may be strided, so the merged projection's buffer can be passed as it is).
+    """
+    _need_cuda(q, k_pages, v_pages, block_table, token_request, positions)
+    for name, t in (("k_pages", k_pages), ("v_pages", v_pages), ("block_table", block_table),
+                    ("token_request", token_request), ("positions", positions)):
+        _need_contiguous(name, t)
+    for name, t in (("block_table", block_table), ("token_request", token_request),
+                    ("positions", positions)):
+        _need_int32(name, t)
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < q_heads * head_dim:
+        raise KernelShapeError(f"q must be [T, >= {q_heads * head_dim}] with unit inner stride")
+    if k_pages.dtype != q.dtype or v_pages.dtype != q.dtype:
+        raise KernelShapeError(f"pages are {k_pages.dtype}, queries {q.dtype}")
+    if k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != head_dim:
+        raise KernelShapeError(
+            f"pages must be [num_pages, {kv_heads}, page_size, {head_dim}], got {tuple(k_pages.shape)}"
+        )
+    if v_pages.shape != k_pages.shape:
+        raise KernelShapeError("k_pages and v_pages differ in shape")
+    tokens = q.shape[0]
+    if token_request.numel() != tokens or positions.numel() != tokens:
+        raise KernelShapeError("token_request and positions need one entry per token")
+    if block_table.dim() != 2:
+        raise KernelShapeError("block_table must be [requests, max_blocks]")
+    num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
+    out = torch.empty((tokens, q_heads * head_dim), dtype=q.dtype, device=q.device)
+    splits = attention_splits(tokens, q_heads, kv_heads, max_seq_len)
+    part_acc = part_ml = None
+    if splits > 1:
+        part_acc = torch.empty((tokens * q_heads * splits, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((tokens * q_heads * splits, 2), dtype=torch.float32, device=q.device)
+    lib = library.load()
+    library.check(
+        lib.mi_attn_generic(
+            _dtype_code(q), _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+            block_table.shape[1], _ptr(token_request), _ptr(positions), _ptr(out), out.stride(0),
+            _ptr(part_acc), _ptr(part_ml), tokens, q_heads, kv_heads, head_dim, page_size, num_pages,
+            float(scale), int(window or 0), splits, _stream(),
+        )
+    )
+    return out
+
+
+def sample(
+    logits: torch.Tensor,
+    temperature: torch.Tensor,
+    top_k: torch.Tensor,
+    top_p: torch.Tensor,
+    seed_lo: torch.Tensor,
+    seed_hi: torch.Tensor,
+    draw_index: torch.Tensor,
+) -> torch.Tensor:
+    """One token id per row of `logits` [B, V]; per-row settings are device tensors of length B.
+
+    `temperature` and `top_p` are float32, `top_k` int32, `seed_lo`, `seed_hi` and
+    `draw_index` int32 holding unsigned 32-bit patterns.
+    """
+    _need_cuda(logits, temperature, top_k, top_p, seed_lo, seed_hi, draw_index)
+    if logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelShapeError("logits must be [rows, vocab] with unit inner stride")
+    rows, vocab = logits.shape
+    for name, t, dt in (
+        ("temperature", temperature, torch.float32),
+        ("top_k", top_k, torch.int32),
+        ("top_p", top_p, torch.float32),
+        ("seed_lo", seed_lo, torch.int32),
+        ("seed_hi", seed_hi, torch.int32),
+        ("draw_index", draw_index, torch.int32),
+    ):
+        _need_contiguous(name, t)
+        if t.dtype != dt or t.numel() != rows:
+            raise KernelShapeError(f"{name} must be {dt} with {rows} entries, got {t.dtype} x {t.numel()}")
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    lib = library.load()
+    library.check(
+        lib.mi_sample(
+            _dtype_code(logits), _ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature),
+            _ptr(top_k), _ptr(top_p), _ptr(seed_lo), _ptr(seed_hi), _ptr(draw_index), _ptr(out),
+            _stream(),
+        )
+    )
+    return out

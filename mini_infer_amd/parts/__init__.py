@@ -1,0 +1,32 @@
+"""Parts a layer is put together from.  Importing this package registers the built-in kinds."""
+
+from mini_infer_amd.parts import attention, block, feed_forward, norm, position  # noqa: F401
+from mini_infer_amd.parts.base import (
+    Block,
+    CacheNeeds,
+    FeedForward,
+    LayerCache,
+    Mixer,
+    Norm,
+    PagedKVNeeds,
+    ParamSpec,
+    Part,
+    PositionEncoding,
+    StateNeeds,
+    StepContext,
+)
+
+__all__ = [
+    "Block",
+    "CacheNeeds",
+    "FeedForward",
+    "LayerCache",
+    "Mixer",
+    "Norm",
+    "PagedKVNeeds",
+    "ParamSpec",
+    "Part",
+    "PositionEncoding",
+    "StateNeeds",
+    "StepContext",
+]

@@ -1,0 +1,130 @@
+"""Grouped-query attention over the paged cache.
+
+Order of operations as in the reference's `GroupedQueryAttention.forward`
+(models/blocks/gqa.py:107-154): one merged q|k|v projection, rotary encoding of
+q and k fused with the write of k and v into cache pages
+(rope_write_kernel.py:75-152), causal attention over the pages with scale
+1/sqrt(head_dim) (cache/packed_attention.py:126-127, :296-338), output
+projection.  A window, if given, limits each query to the last `window` keys.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from mini_infer_amd import ops
+from mini_infer_amd.parts.base import (
+    CacheNeeds,
+    LayerCache,
+    Mixer,
+    PagedKVNeeds,
+    ParamSpec,
+    StepContext,
+    TensorGetter,
+)
+from mini_infer_amd.parts.linear import Linear
+from mini_infer_amd.parts.position import RotaryPosition
+from mini_infer_amd.registry import POSITION_ENCODINGS, register_mixer
+
+
+class GQAttention(Mixer):
+    def __init__(
+        self,
+        hidden_size: int,
+        num_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        position: RotaryPosition | None,
+        dtype: torch.dtype,
+        device,
+        *,
+        window: int | None = None,
+        scale: float | None = None,
+    ) -> None:
+        super().__init__(dtype, device)
+        if num_heads % num_kv_heads != 0:
+            raise ValueError(f"num_heads={num_heads} is not a multiple of num_kv_heads={num_kv_heads}")
+        if window is not None and window <= 0:
+            raise ValueError(f"window must be positive, got {window}")
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.position = position
+        self.window = window
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        q_width, kv_width = num_heads * head_dim, num_kv_heads * head_dim
+        self.qkv = Linear(hidden_size, [q_width, kv_width, kv_width], ["q_proj", "k_proj", "v_proj"], dtype, device)
+        self.out = Linear(q_width, hidden_size, "o_proj", dtype, device)
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        return {**self.qkv.param_specs(prefix), **self.out.param_specs(prefix)}
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        self.qkv.load_params(prefix, get)
+        self.out.load_params(prefix, get)
+
+    def cache_needs(self) -> CacheNeeds:
+        return CacheNeeds(pages=PagedKVNeeds(self.num_kv_heads, self.head_dim, self.window))
+
+    def forward(
+        self, x: torch.Tensor, ctx: StepContext, cache: LayerCache, writes_cache: bool = True
+    ) -> torch.Tensor:
+        assert cache.group is not None and cache.k_pages is not None and cache.v_pages is not None
+        q_width = self.num_heads * self.head_dim
+        if writes_cache:
+            qkv = self.qkv.forward(x)
+            kv_heads, slots = self.num_kv_heads, ctx.slot_mapping[cache.group]
+        else:
+            # reads another call's keys and values: only q is projected
+            assert self.qkv.weight is not None
+            qkv = ops.linear(x, self.qkv.weight[:q_width])
+            kv_heads, slots = 0, None
+        if self.position is not None:
+            cos, sin = self.position.tables(ctx)
+            ops.rope_kv_write(
+                qkv, cos, sin, slots, cache.k_pages, cache.v_pages,
+                q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
+                rotary_dim=self.position.rotary_dim, interleaved=self.position.interleaved,
+            )
+        else:
+            empty = torch.empty((ctx.num_tokens, 0), dtype=torch.float32, device=x.device)
+            ops.rope_kv_write(
+                qkv, empty, empty, slots, cache.k_pages, cache.v_pages,
+                q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
+                rotary_dim=0, interleaved=False,
+            )
+        attended = ops.paged_attention(
+            qkv, cache.k_pages, cache.v_pages, ctx.block_tables[cache.group], ctx.token_request,
+            ctx.positions, q_heads=self.num_heads, kv_heads=self.num_kv_heads,
+            head_dim=self.head_dim, scale=self.scale, window=self.window,
+            max_seq_len=ctx.max_seq_len,
+        )
+        return self.out.forward(attended)
+
+
+@register_mixer("gqa_attention")
+def build_gqa_attention(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> GQAttention:
+    position = None
+    pos_desc = desc.get("position")
+    if pos_desc is not None:
+        key = ("position", repr(sorted(pos_desc.items(), key=lambda kv: kv[0])))
+        if shared is not None and key in shared:
+            position = shared[key]
+        else:
+            position = POSITION_ENCODINGS.lookup(pos_desc["kind"])(pos_desc, dtype, device, shared)
+            if shared is not None:
+                shared[key] = position
+    return GQAttention(
+        int(desc["hidden_size"]),
+        int(desc["num_heads"]),
+        int(desc["num_kv_heads"]),
+        int(desc["head_dim"]),
+        position,
+        dtype,
+        device,
+        window=desc.get("window"),
+        scale=desc.get("scale"),
+    )

@@ -1,0 +1,346 @@
+"""A plain, slow NumPy implementation of the Llama decoder: whole sequences, no cache.
+
+One function per part, written from the formulas of the reference
+(JonathanBerhe/mini-infer; paths below are relative to its `src/mini_infer/`).
+It shares no code with the engine.  Matrix products, norm statistics and the
+softmax accumulate in float64 (`ACC`); the rotation angles follow the
+reference's float32 arithmetic so both sides see the same table.
+
+Weights are a dict of NumPy arrays under the checkpoint's tensor names.
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+ACC = np.float64
+
+
+# ----------------------------------------------------------------------------
+# position encoding
+# ----------------------------------------------------------------------------
+
+
+def inv_freq_default(head_dim: int, theta: float) -> np.ndarray:
+    """`1 / theta^(2j/D)`, j = 0..D/2-1, in float32.
+
+    models/blocks/rope.py:343-346 (`1.0 / base ** (arange(0, D, 2) / D)`).
+    """
+    exponent = np.arange(0, head_dim, 2, dtype=np.float32) / np.float32(head_dim)
+    return (np.float32(1.0) / np.power(np.float32(theta), exponent)).astype(np.float32)
+
+
+def inv_freq_llama3(
+    inv_freq: np.ndarray,
+    factor: float,
+    low_freq_factor: float,
+    high_freq_factor: float,
+    original_max_position_embeddings: int,
+) -> np.ndarray:
+    """The llama3 rescale of an inverse-frequency table, float32 in and out.
+
+    models/blocks/rope.py:200-225: wavelengths above L/low are divided by
+    `factor`, those below L/high are kept, the band between is blended with
+    `smooth = (L/wavelen - low) / (high - low)`.
+    """
+    inv_freq = inv_freq.astype(np.float32)
+    old_len = original_max_position_embeddings
+    low_wavelen = old_len / low_freq_factor
+    high_wavelen = old_len / high_freq_factor
+    wavelen = (np.float32(2 * math.pi) / inv_freq).astype(np.float32)
+    scaled = np.where(wavelen > low_wavelen, inv_freq / np.float32(factor), inv_freq).astype(
+        np.float32
+    )
+    smooth = (np.float32(old_len) / wavelen - np.float32(low_freq_factor)) / np.float32(
+        high_freq_factor - low_freq_factor
+    )
+    smoothed = ((1 - smooth) * scaled / np.float32(factor) + smooth * scaled).astype(np.float32)
+    medium = ~(wavelen < high_wavelen) & ~(wavelen > low_wavelen)
+    return np.where(medium, smoothed, scaled).astype(np.float32)
+
+
+def rope_tables(positions: np.ndarray, inv_freq: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+    """`cos, sin` of shape [T, D]: angle = pos * inv_freq in float32, halves repeated.
+
+    models/blocks/rope.py:392-408 (`freqs = inv_freq @ pos`, `emb = cat(freqs, freqs)`).
+    """
+    pos = positions.astype(np.float32)
+    freqs = (pos[:, None] * inv_freq.astype(np.float32)[None, :]).astype(np.float32)
+    emb = np.concatenate([freqs, freqs], axis=-1)
+    return np.cos(emb.astype(ACC)), np.sin(emb.astype(ACC))
+
+
+def rotate_half(x: np.ndarray) -> np.ndarray:
+    """`(-x_high, x_low)` on the last axis.  models/blocks/rope.py:411-416."""
+    half = x.shape[-1] // 2
+    return np.concatenate([-x[..., half:], x[..., :half]], axis=-1)
+
+
+def apply_rope(x: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:
+    """`x*cos + rotate_half(x)*sin` for x of shape [T, heads, D], tables [T, D].
+
+    models/blocks/rope.py:419-431.
+    """
+    return x * cos[:, None, :] + rotate_half(x) * sin[:, None, :]
+
+
+# ----------------------------------------------------------------------------
+# norm, feed-forward, embedding
+# ----------------------------------------------------------------------------
+
+
+def rms_norm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
+    """`w * x * rsqrt(mean(x^2) + eps)` over the last axis.
+
+    models/blocks/rmsnorm.py:81-93.
+    """
+    x = x.astype(ACC)
+    variance = np.mean(x * x, axis=-1, keepdims=True)
+    return weight.astype(ACC) * (x / np.sqrt(variance + eps))
+
+
+def silu(x: np.ndarray) -> np.ndarray:
+    """`x / (1 + exp(-x))`.  models/blocks/silu_mul_kernel.py:86-90."""
+    return x / (1.0 + np.exp(-x))
+
+
+def swiglu(x: np.ndarray, w_gate: np.ndarray, w_up: np.ndarray, w_down: np.ndarray) -> np.ndarray:
+    """`down(silu(gate(x)) * up(x))`, weights in [out, in] layout, no biases.
+
+    models/blocks/swiglu.py:44-46, models/blocks/activations.py:36-45.
+    """
+    x = x.astype(ACC)
+    gate = x @ w_gate.astype(ACC).T
+    up = x @ w_up.astype(ACC).T
+    return (silu(gate) * up) @ w_down.astype(ACC).T
+
+
+def embedding(table: np.ndarray, ids: np.ndarray) -> np.ndarray:
+    """Row lookup.  models/llama/llama.py:159."""
+    return table[ids].astype(ACC)
+
+
+# ----------------------------------------------------------------------------
+# attention
+# ----------------------------------------------------------------------------
+
+
+def causal_attention(
+    q: np.ndarray,
+    k: np.ndarray,
+    v: np.ndarray,
+    scale: float,
+    window: int | None = None,
+) -> np.ndarray:
+    """Causal grouped-query attention of one whole sequence.
+
+    q: [Tq, Hq, D]; k, v: [Tk, Hkv, D] with Tq <= Tk; the queries are the last
+    Tq positions.  Query head h reads key/value head h // (Hq/Hkv); query at
+    absolute position p sees keys 0..p, or p-window+1..p with a window.
+    cache/packed_attention.py:296-338.
+    """
+    tq, hq, _ = q.shape
+    tk, hkv, _ = k.shape
+    if hq % hkv != 0:
+        raise ValueError(f"num_q_heads={hq} not a multiple of num_kv_heads={hkv}")
+    if tq > tk:
+        raise ValueError(f"q_len={tq} > k_len={tk}")
+    group = hq // hkv
+    k = np.repeat(k.astype(ACC), group, axis=1)
+    v = np.repeat(v.astype(ACC), group, axis=1)
+    scores = np.einsum("qhd,khd->qhk", q.astype(ACC), k) * scale
+    q_pos = np.arange(tq) + (tk - tq)
+    k_pos = np.arange(tk)
+    invalid = k_pos[None, :] > q_pos[:, None]
+    if window is not None:
+        invalid |= k_pos[None, :] < (q_pos[:, None] - window + 1)
+    scores = np.where(invalid[:, None, :], -np.inf, scores)
+    scores = scores - scores.max(axis=-1, keepdims=True)
+    weights = np.exp(scores)
+    weights = weights / weights.sum(axis=-1, keepdims=True)
+    return np.einsum("qhk,khd->qhd", weights, v)
+
+
+def attention_layer(
+    x: np.ndarray,
+    w_q: np.ndarray,
+    w_k: np.ndarray,
+    w_v: np.ndarray,
+    w_o: np.ndarray,
+    cos: np.ndarray,
+    sin: np.ndarray,
+    num_heads: int,
+    num_kv_heads: int,
+    head_dim: int,
+    window: int | None = None,
+    kv_override: tuple[np.ndarray, np.ndarray] | None = None,
+) -> tuple[np.ndarray, tuple[np.ndarray, np.ndarray]]:
+    """Project, rotate q and k, attend with scale 1/sqrt(D), project out.
+
+    models/blocks/gqa.py:107-154 (scale: cache/packed_attention.py:126-127).
+    Returns the output and the (rotated k, v) it used; `kv_override` makes the
+    layer attend over another layer's keys and values instead of its own.
+    """
+    t = x.shape[0]
+    x = x.astype(ACC)
+    q = (x @ w_q.astype(ACC).T).reshape(t, num_heads, head_dim)
+    q = apply_rope(q, cos, sin)
+    if kv_override is None:
+        k = (x @ w_k.astype(ACC).T).reshape(t, num_kv_heads, head_dim)
+        v = (x @ w_v.astype(ACC).T).reshape(t, num_kv_heads, head_dim)
+        k = apply_rope(k, cos, sin)
+    else:
+        k, v = kv_override
+    out = causal_attention(q, k, v, 1.0 / math.sqrt(head_dim), window)
+    return out.reshape(t, num_heads * head_dim) @ w_o.astype(ACC).T, (k, v)
+
+
+# ----------------------------------------------------------------------------
+# whole model
+# ----------------------------------------------------------------------------
+
+
+def config_inv_freq(cfg: dict) -> np.ndarray:
+    """The inverse-frequency table a config.json asks for.
+
+    models/blocks/rope.py:228-269: `rope_parameters` or `rope_scaling`, type
+    under `rope_type` or `type`, theta inside the dict or at top level.
+    """
+    head_dim = cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_attention_heads"]
+    params = dict(cfg.get("rope_parameters") or cfg.get("rope_scaling") or {})
+    theta = float(params.get("rope_theta") or cfg.get("rope_theta") or 10000.0)
+    table = inv_freq_default(head_dim, theta)
+    kind = params.get("rope_type") or params.get("type") or "default"
+    if kind == "llama3":
+        table = inv_freq_llama3(
+            table,
+            float(params["factor"]),
+            float(params["low_freq_factor"]),
+            float(params["high_freq_factor"]),
+            int(params["original_max_position_embeddings"]),
+        )
+    elif kind != "default":
+        raise NotImplementedError(kind)
+    return table
+
+
+def llama_logits(
+    cfg: dict,
+    weights: dict[str, np.ndarray],
+    token_ids: np.ndarray,
+    *,
+    first_position: int = 0,
+    order: list[tuple[int, int | None]] | None = None,
+    window: int | None = None,
+) -> np.ndarray:
+    """Logits [T, V] of one whole sequence, float64.
+
+    models/llama/llama.py:149-172 and models/blocks/transformer_block.py:95-153:
+    embed; per layer `r += attn(norm(r))`, `r += mlp(norm(r))`; final norm; head
+    (the embedding table when `tie_word_embeddings`).
+
+    `order` lists (layer, call whose keys and values it reads or None) in
+    running order; the default runs every layer once with its own keys.
+    `first_position` shifts all positions (only distances matter to the result).
+    """
+    heads = cfg["num_attention_heads"]
+    kv_heads = cfg["num_key_value_heads"]
+    head_dim = cfg.get("head_dim") or cfg["hidden_size"] // heads
+    eps = cfg["rms_norm_eps"]
+    ids = np.asarray(token_ids, dtype=np.int64)
+    positions = np.arange(len(ids)) + first_position
+    cos, sin = rope_tables(positions, config_inv_freq(cfg))
+
+    if order is None:
+        order = [(i, None) for i in range(cfg["num_hidden_layers"])]
+    r = embedding(weights["model.embed_tokens.weight"], ids)
+    kept: list[tuple[np.ndarray, np.ndarray]] = []
+    for layer, reads in order:
+        p = f"model.layers.{layer}."
+        h = rms_norm(r, weights[p + "input_layernorm.weight"], eps)
+        a, kv = attention_layer(
+            h,
+            weights[p + "self_attn.q_proj.weight"],
+            weights[p + "self_attn.k_proj.weight"],
+            weights[p + "self_attn.v_proj.weight"],
+            weights[p + "self_attn.o_proj.weight"],
+            cos,
+            sin,
+            heads,
+            kv_heads,
+            head_dim,
+            window,
+            kv_override=None if reads is None else kept[reads],
+        )
+        kept.append(kv)
+        r = r + a
+        h = rms_norm(r, weights[p + "post_attention_layernorm.weight"], eps)
+        r = r + swiglu(
+            h,
+            weights[p + "mlp.gate_proj.weight"],
+            weights[p + "mlp.up_proj.weight"],
+            weights[p + "mlp.down_proj.weight"],
+        )
+    h = rms_norm(r, weights["model.norm.weight"], eps)
+    head = (
+        weights["model.embed_tokens.weight"]
+        if cfg.get("tie_word_embeddings", False)
+        else weights["lm_head.weight"]
+    )
+    return h @ head.astype(ACC).T
+
+
+# ----------------------------------------------------------------------------
+# sampling
+# ----------------------------------------------------------------------------
+
+
+def greedy(logits: np.ndarray) -> int:
+    """First index of the maximum.  engine/sampler.py:26-27."""
+    return int(np.argmax(logits))
+
+
+def top_k_filter(logits: np.ndarray, k: int) -> np.ndarray:
+    """Logits below the k-th largest become -inf; k = 0 or k >= V keeps all.
+
+    engine/sampler.py:93-98.
+    """
+    if k <= 0 or k >= logits.shape[-1]:
+        return logits
+    threshold = np.sort(logits)[-k]
+    return np.where(logits < threshold, -np.inf, logits)
+
+
+def top_p_filter(logits: np.ndarray, p: float) -> np.ndarray:
+    """Drop a token when the probability mass sorted before it exceeds p.
+
+    engine/sampler.py:101-110 (the boundary token is kept).
+    """
+    if p >= 1.0:
+        return logits
+    order = np.argsort(-logits, kind="stable")
+    sorted_logits = logits[order]
+    probs = softmax(sorted_logits)
+    cum = np.cumsum(probs)
+    exclude = np.concatenate([[False], (cum > p)[:-1]])
+    out = logits.copy()
+    out[order[exclude]] = -np.inf
+    return out
+
+
+def softmax(x: np.ndarray) -> np.ndarray:
+    x = x.astype(ACC)
+    e = np.exp(x - np.max(x))
+    return e / e.sum()
+
+
+def sampling_distribution(
+    logits: np.ndarray, temperature: float, top_k: int = 0, top_p: float = 1.0
+) -> np.ndarray:
+    """The distribution a sampling row draws from.  engine/sampler.py:29-35."""
+    scaled = logits.astype(ACC) / temperature
+    scaled = top_k_filter(scaled, top_k)
+    scaled = top_p_filter(scaled, top_p)
+    return softmax(scaled)
