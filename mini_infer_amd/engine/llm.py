@@ -1,0 +1,74 @@
+"""`LLM(...).generate(...)`: the short way from a model folder to generated tokens.
+
+It is the reference's quick-start (README.md:106-131: `ModelRunner.from_pretrained`
++ `ContinuousScheduler` + `Request`) in one object, driven synchronously.
+"""
+
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Sequence
+
+from mini_infer_amd.config import DEFAULT_BLOCK_SIZE, DEFAULT_NUM_BLOCKS, read_config_json
+from mini_infer_amd.engine.model_runner import ModelRunner
+from mini_infer_amd.engine.request import GenerationResult, Request
+from mini_infer_amd.engine.scheduler import (
+    DEFAULT_CHUNK_SIZE,
+    DEFAULT_DECODE_HEADROOM_BLOCKS,
+    ContinuousScheduler,
+)
+from mini_infer_amd.engine.tokenizer import Tokenizer
+from mini_infer_amd.sampling.params import SamplingParams
+
+
+class LLM:
+    def __init__(
+        self,
+        model: str | Path,
+        *,
+        dtype: str = "bfloat16",
+        device: str = "cuda:0",
+        num_blocks: int = DEFAULT_NUM_BLOCKS,
+        block_size: int = DEFAULT_BLOCK_SIZE,
+        max_concurrent: int = 16,
+        max_num_batched_tokens: int = 2048,
+        chunk_size: int = DEFAULT_CHUNK_SIZE,
+        decode_headroom_blocks: int = DEFAULT_DECODE_HEADROOM_BLOCKS,
+        seed: int = 0,
+    ) -> None:
+        self.runner = ModelRunner.from_pretrained(
+            model,
+            device=device,
+            dtype=dtype,
+            num_blocks=num_blocks,
+            block_size=block_size,
+            max_concurrent=max_concurrent,
+        )
+        raw = read_config_json(model)
+        self.tokenizer = Tokenizer.from_pretrained(model)
+        self.scheduler = ContinuousScheduler(
+            self.runner,
+            max_concurrent=max_concurrent,
+            decode_headroom_blocks=decode_headroom_blocks,
+            chunk_size=chunk_size,
+            max_num_batched_tokens=max_num_batched_tokens,
+            eos_token_id=raw.get("eos_token_id"),
+            tokenizer=self.tokenizer,
+            base_seed=seed,
+        )
+
+    def generate(
+        self,
+        prompts: Sequence[str | Sequence[int]],
+        sampling_params: SamplingParams | Sequence[SamplingParams] | None = None,
+        max_tokens: int = 16,
+    ) -> list[GenerationResult]:
+        """One result per prompt (text or token ids), in order."""
+        if sampling_params is None:
+            sampling_params = SamplingParams()
+        if isinstance(sampling_params, SamplingParams):
+            sampling_params = [sampling_params] * len(prompts)
+        if len(sampling_params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt (or one for all)")
+        requests = [Request(p, sp, max_tokens) for p, sp in zip(prompts, sampling_params)]
+        return self.scheduler.run_all(requests)

@@ -1,0 +1,401 @@
+"""Continuous batching above the step function.
+
+Each step: finished requests have already given their pages back; waiting
+requests are admitted first-come-first-served while a seat and enough pages are
+free; then ONE batch is built under a token budget: every decoding request feeds
+its last token, and what is left of the budget is handed to prefilling requests
+in admission order as portions of their prompts, cut wherever the budget ends.
+The step runs, and every request whose last fed token completed what it had to
+feed gets its next token sampled on the device.
+
+Names and policies follow the reference's `ContinuousScheduler`
+(scheduler/continuous_scheduler.py): `max_concurrent`, `decode_headroom_blocks`,
+`chunk_size` (:144-177); FIFO admission by block budget, with a prompt that can
+never fit finished as "cancelled" (:670-773); EOS ends with "stop" and is not
+emitted, `max_tokens` ends with "length", the last emitted token is never fed
+(:847-860).  Two things differ by design:
+  * a global token budget per step (`max_num_batched_tokens`); the reference only
+    bounds each request's chunk;
+  * when pages run out mid-flight, the youngest running request is preempted and
+    recomputed later (its pages are freed, it goes back to the FRONT of the
+    queue and feeds prompt + generated tokens again), so no request is lost and
+    greedy and seeded outputs are unchanged.  The reference cancels the youngest
+    request instead (:388-416).  A request that cannot fit even alone is
+    finished as "cancelled".
+"""
+
+from __future__ import annotations
+
+import collections
+import threading
+import time
+from typing import Any, Callable, Iterable, Sequence
+
+from mini_infer_amd.engine.batch import StepEntry
+from mini_infer_amd.engine.request import (
+    GenerationResult,
+    GenerationStep,
+    Request,
+    RequestState,
+    RunningRequest,
+)
+from mini_infer_amd.exceptions import EngineNotRunningError, OutOfMemoryError
+
+DEFAULT_DECODE_HEADROOM_BLOCKS = 8
+DEFAULT_CHUNK_SIZE = 256
+IDLE_SLEEP_SECONDS = 0.005
+
+
+def _device_sampler(logits, params, seeds, draws) -> list[int]:
+    from mini_infer_amd.sampling.sampler import sample_batch
+
+    return sample_batch(logits, params, seeds, draws)
+
+
+class RequestHandle:
+    """What `submit` returns: wait for the result or walk the steps so far."""
+
+    def __init__(self, scheduler: "ContinuousScheduler", running: RunningRequest) -> None:
+        self._scheduler = scheduler
+        self._running = running
+
+    @property
+    def request_id(self) -> int:
+        return self._running.request_id
+
+    def done(self) -> bool:
+        return self._running.done_event.is_set()
+
+    def cancel(self) -> None:
+        self._running.cancel_requested = True
+
+    def wait(self, timeout: float | None = None) -> GenerationResult:
+        deadline = None if timeout is None else time.time() + timeout
+        while not self._running.done_event.wait(0.05):
+            if self._scheduler._thread is not None and not self._scheduler.engine_alive:
+                raise EngineNotRunningError("the engine stopped before the request finished")
+            if self._scheduler._thread is None:
+                # no engine thread: drive the engine from the caller
+                self._scheduler.step()
+            if deadline is not None and time.time() > deadline:
+                raise TimeoutError("request did not finish in time")
+        return self._scheduler._result_of(self._running)
+
+    def steps(self) -> list[GenerationStep]:
+        return list(self._running.steps)
+
+
+class ContinuousScheduler:
+    def __init__(
+        self,
+        runner: Any,
+        max_concurrent: int = 16,
+        decode_headroom_blocks: int = DEFAULT_DECODE_HEADROOM_BLOCKS,
+        chunk_size: int = DEFAULT_CHUNK_SIZE,
+        max_num_batched_tokens: int = 2048,
+        *,
+        eos_token_id: int | Sequence[int] | None = None,
+        tokenizer: Any = None,
+        base_seed: int = 0,
+        sampler: Callable[..., list[int]] | None = None,
+    ) -> None:
+        if max_concurrent <= 0 or chunk_size <= 0 or max_num_batched_tokens <= 0:
+            raise ValueError("max_concurrent, chunk_size and max_num_batched_tokens must be positive")
+        if decode_headroom_blocks < 0:
+            raise ValueError("decode_headroom_blocks must be >= 0")
+        self.runner = runner
+        self.cache = runner.cache
+        self.max_concurrent = max_concurrent
+        self.decode_headroom_blocks = decode_headroom_blocks
+        self.chunk_size = chunk_size
+        self.max_num_batched_tokens = max_num_batched_tokens
+        if eos_token_id is None:
+            self.eos_token_ids: frozenset[int] = frozenset()
+        elif isinstance(eos_token_id, int):
+            self.eos_token_ids = frozenset([eos_token_id])
+        else:
+            self.eos_token_ids = frozenset(int(t) for t in eos_token_id)
+        self.tokenizer = tokenizer
+        self.base_seed = base_seed
+        self._sample = sampler or _device_sampler
+        self._waiting: collections.deque[RunningRequest] = collections.deque()
+        self._running: list[RunningRequest] = []
+        self._next_id = 0
+        self._admitted = 0
+        self._lock = threading.Lock()
+        self._thread: threading.Thread | None = None
+        self._stop = threading.Event()
+        self._crashed: BaseException | None = None
+        self.stats = {"steps": 0, "preemptions": 0, "tokens_run": 0, "rejected": 0}
+
+    # -- submitting -----------------------------------------------------------
+
+    def _tokenize(self, prompt: str | Sequence[int]) -> list[int]:
+        if isinstance(prompt, str):
+            if self.tokenizer is None:
+                raise ValueError("a text prompt needs a tokenizer; pass token ids instead")
+            return list(self.tokenizer.encode(prompt))
+        return [int(t) for t in prompt]
+
+    def submit(self, request: Request) -> RequestHandle:
+        if self._crashed is not None:
+            raise EngineNotRunningError(f"the engine has failed: {self._crashed!r}")
+        with self._lock:
+            request_id = self._next_id
+            self._next_id += 1
+        seed = request.sampling_params.seed
+        if seed is None:
+            seed = (self.base_seed * 0x9E3779B97F4A7C15 + request_id) & 0xFFFFFFFFFFFFFFFF
+        running = RunningRequest(
+            request_id=request_id,
+            request=request,
+            prompt_token_ids=self._tokenize(request.prompt),
+            seed=seed,
+        )
+        with self._lock:
+            self._waiting.append(running)
+        return RequestHandle(self, running)
+
+    def run(self, request: Request) -> GenerationResult:
+        return self.submit(request).wait()
+
+    def run_all(self, requests: Iterable[Request]) -> list[GenerationResult]:
+        """Submit all, drive the engine until all are done; results in submission order."""
+        handles = [self.submit(r) for r in requests]
+        if self._thread is None:
+            while not all(h.done() for h in handles):
+                if not self.step() and not self.has_work():
+                    break
+        return [h.wait() for h in handles]
+
+    # -- engine thread (optional) -------------------------------------------------
+
+    @property
+    def engine_alive(self) -> bool:
+        return self._thread is not None and self._thread.is_alive() and self._crashed is None
+
+    def start(self) -> None:
+        if self._thread is not None:
+            return
+        self._stop.clear()
+        self._thread = threading.Thread(target=self._engine_loop, name="mini-infer-engine", daemon=True)
+        self._thread.start()
+
+    def stop(self) -> None:
+        thread = self._thread
+        if thread is None:
+            return
+        self._stop.set()
+        thread.join()
+        self._thread = None
+        for running in list(self._running) + list(self._waiting):
+            self._finish(running, "cancelled")
+        self._running.clear()
+        self._waiting.clear()
+
+    def _engine_loop(self) -> None:
+        try:
+            while not self._stop.is_set():
+                if not self.step():
+                    time.sleep(IDLE_SLEEP_SECONDS)
+        except BaseException as err:  # noqa: BLE001
+            self._crashed = err
+            for running in list(self._running) + list(self._waiting):
+                self._finish(running, "cancelled")
+            raise
+
+    # -- one step -------------------------------------------------------------------
+
+    def has_work(self) -> bool:
+        return bool(self._waiting or self._running)
+
+    def step(self) -> bool:
+        """Admit, build one batch, run it, sample, finish.  False when there was nothing to do."""
+        self._cancel_pending()
+        self._admit_waiting()
+        if not self._running:
+            return False
+        while True:
+            entries, owners = self._build_batch()
+            if not entries:
+                return False
+            try:
+                logits = self.runner.step(entries)
+                break
+            except OutOfMemoryError:
+                if not self._preempt_youngest():
+                    raise
+        self.stats["steps"] += 1
+        self.stats["tokens_run"] += sum(len(e.tokens) for e in entries)
+        sampled_for: list[RunningRequest] = []
+        for entry, running in zip(entries, owners):
+            running.tokens_fed += len(entry.tokens)
+            running.state = (
+                RequestState.DECODING if running.prefill_remaining == 0 else RequestState.CHUNKED_PREFILLING
+            )
+            if entry.want:
+                sampled_for.append(running)
+        if sampled_for:
+            token_ids = self._sample(
+                logits,
+                [r.request.sampling_params for r in sampled_for],
+                [r.seed for r in sampled_for],
+                [len(r.tokens_generated) for r in sampled_for],
+            )
+            for running, token in zip(sampled_for, token_ids):
+                self._accept_token(running, int(token))
+        self._reap_done()
+        return True
+
+    # -- pieces of a step ---------------------------------------------------------------
+
+    def _cancel_pending(self) -> None:
+        for running in list(self._running):
+            if running.cancel_requested:
+                self._finish(running, "cancelled")
+        with self._lock:
+            waiting = list(self._waiting)
+        for running in waiting:
+            if running.cancel_requested:
+                with self._lock:
+                    self._waiting.remove(running)
+                self._finish(running, "cancelled")
+        self._reap_done()
+
+    def _pages_for(self, tokens: int) -> int:
+        return self.cache.pages_for_tokens(tokens)
+
+    def _free_pages(self) -> int:
+        return self.runner.num_free_blocks()
+
+    def _admit_waiting(self) -> None:
+        while len(self._running) < self.max_concurrent:
+            with self._lock:
+                if not self._waiting:
+                    return
+                running = self._waiting[0]
+            if running.cancel_requested:
+                with self._lock:
+                    self._waiting.popleft()
+                self._finish(running, "cancelled")
+                continue
+            if not running.prompt_token_ids:
+                with self._lock:
+                    self._waiting.popleft()
+                self._finish(running, "stop")
+                continue
+            if running.request.max_tokens <= 0:
+                with self._lock:
+                    self._waiting.popleft()
+                self._finish(running, "length")
+                continue
+            to_feed = len(running.feed)
+            remaining_new = running.request.max_tokens - len(running.tokens_generated)
+            need_now = self._pages_for(to_feed)
+            if need_now > self.runner.num_blocks:
+                # can never fit, not even alone
+                with self._lock:
+                    self._waiting.popleft()
+                self.stats["rejected"] += 1
+                self._finish(running, "cancelled")
+                continue
+            # the prompt plus some runway for decoding, but never more than it can ever use
+            required = max(
+                need_now,
+                min(need_now + self.decode_headroom_blocks, self._pages_for(to_feed + remaining_new - 1)),
+            )
+            free = self._free_pages()
+            if free < required and (self._running or free < need_now):
+                return
+            with self._lock:
+                self._waiting.popleft()
+            self.cache.add_request(running.request_id)
+            running.state = RequestState.PREFILLING
+            running.tokens_fed = 0
+            running.admitted_order = self._admitted
+            self._admitted += 1
+            self._running.append(running)
+
+    def _build_batch(self) -> tuple[list[StepEntry], list[RunningRequest]]:
+        budget = self.max_num_batched_tokens
+        entries: list[StepEntry] = []
+        owners: list[RunningRequest] = []
+        decoders = [r for r in self._running if r.prefill_remaining == 1 and r.tokens_fed > 0]
+        prefillers = [r for r in self._running if r not in decoders]
+        for running in decoders:
+            if budget <= 0:
+                break
+            entries.append(StepEntry(running.request_id, [running.feed[-1]], [0]))
+            owners.append(running)
+            budget -= 1
+        for running in sorted(prefillers, key=lambda r: r.admitted_order):
+            if budget <= 0:
+                break
+            count = min(self.chunk_size, running.prefill_remaining, budget)
+            if count <= 0:
+                continue
+            feed = running.feed
+            portion = feed[running.tokens_fed : running.tokens_fed + count]
+            completes = running.tokens_fed + count == len(feed)
+            entries.append(StepEntry(running.request_id, portion, [count - 1] if completes else []))
+            owners.append(running)
+            budget -= count
+        return entries, owners
+
+    def _preempt_youngest(self) -> bool:
+        """Free the youngest running request and queue it first for recompute.
+
+        Returns False when nothing can be preempted (then the error is real).  A
+        request that is alone and still does not fit is finished as "cancelled".
+        """
+        if not self._running:
+            return False
+        victim = max(self._running, key=lambda r: r.admitted_order)
+        self._running.remove(victim)
+        self.cache.free_request(victim.request_id)
+        if not self._running:
+            self.stats["rejected"] += 1
+            self._finish(victim, "cancelled", already_freed=True)
+            return True
+        victim.state = RequestState.WAITING
+        victim.tokens_fed = 0
+        victim.preemptions += 1
+        self.stats["preemptions"] += 1
+        with self._lock:
+            self._waiting.appendleft(victim)
+        return True
+
+    def _accept_token(self, running: RunningRequest, token: int) -> None:
+        params = running.request.sampling_params
+        if token in self.eos_token_ids and not params.ignore_eos:
+            self._finish(running, "stop")
+            return
+        running.tokens_generated.append(token)
+        text = self.tokenizer.decode([token]) if self.tokenizer is not None else ""
+        running.steps.append(GenerationStep(text=text, num_tokens=1, tokens=(token,)))
+        if len(running.tokens_generated) >= running.request.max_tokens:
+            self._finish(running, "length")
+
+    def _finish(self, running: RunningRequest, reason: str, already_freed: bool = False) -> None:
+        if running.state == RequestState.DONE:
+            return
+        running.finish_reason = reason  # type: ignore[assignment]
+        in_cache = running in self._running and not already_freed
+        running.state = RequestState.DONE
+        if in_cache and self.cache.has_request(running.request_id):
+            self.cache.free_request(running.request_id)
+        running.steps.append(GenerationStep(text="", finish_reason=reason))  # type: ignore[arg-type]
+        running.done_event.set()
+
+    def _reap_done(self) -> None:
+        self._running = [r for r in self._running if r.state != RequestState.DONE]
+
+    def _result_of(self, running: RunningRequest) -> GenerationResult:
+        tokens = list(running.tokens_generated)
+        text = self.tokenizer.decode(tokens) if self.tokenizer is not None else ""
+        return GenerationResult(
+            text=text,
+            tokens=tokens,
+            finish_reason=running.finish_reason or "cancelled",
+            prompt_tokens=len(running.prompt_token_ids),
+        )

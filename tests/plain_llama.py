@@ -233,7 +233,7 @@ def llama_logits(
     *,
     first_position: int = 0,
     order: list[tuple[int, int | None]] | None = None,
-    window: int | None = None,
+    window: int | None | list[int | None] = None,
 ) -> np.ndarray:
     """Logits [T, V] of one whole sequence, float64.
 
@@ -244,6 +244,7 @@ def llama_logits(
     `order` lists (layer, call whose keys and values it reads or None) in
     running order; the default runs every layer once with its own keys.
     `first_position` shifts all positions (only distances matter to the result).
+    `window` is one window for every call, or a list with one entry per call.
     """
     heads = cfg["num_attention_heads"]
     kv_heads = cfg["num_key_value_heads"]
@@ -257,7 +258,8 @@ def llama_logits(
         order = [(i, None) for i in range(cfg["num_hidden_layers"])]
     r = embedding(weights["model.embed_tokens.weight"], ids)
     kept: list[tuple[np.ndarray, np.ndarray]] = []
-    for layer, reads in order:
+    windows = window if isinstance(window, list) else [window] * len(order)
+    for call, (layer, reads) in enumerate(order):
         p = f"model.layers.{layer}."
         h = rms_norm(r, weights[p + "input_layernorm.weight"], eps)
         a, kv = attention_layer(
@@ -271,7 +273,7 @@ def llama_logits(
             heads,
             kv_heads,
             head_dim,
-            window,
+            windows[call],
             kv_override=None if reads is None else kept[reads],
         )
         kept.append(kv)
