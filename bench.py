@@ -1,0 +1,224 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+
+Default workload: the layer sizes of Llama 3.1 8B with random bfloat16 weights
+made on the device, a batch of 8 requests with 2,048-token uniform-random prompts,
+decoded greedily from position 2,048 on; one "step" is one decode step of the whole
+batch (step function + greedy choice on the device + ids back to the host).  The
+line it prints also holds the prefill rate of one 2,048-token prompt, the decode
+rates at batch 1 and 64, and the decode step's share of the HBM roofline.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, GB/s
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+LLAMA_31_8B = {
+    "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 32,
+    "hidden_size": 4096,
+    "num_attention_heads": 32,
+    "num_key_value_heads": 8,
+    "head_dim": 128,
+    "intermediate_size": 14336,
+    "vocab_size": 128256,
+    "rope_theta": 500000.0,
+    "rope_scaling": {
+        "rope_type": "llama3",
+        "factor": 8.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 4.0,
+        "original_max_position_embeddings": 8192,
+    },
+    "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": False,
+    "max_position_embeddings": 131072,
+}
+FULL_LAYERS = LLAMA_31_8B["num_hidden_layers"]
+PROMPT_LEN = 2048
+BLOCK_SIZE = 16
+
+
+def weight_bytes(cfg: dict, elem: int) -> int:
+    """Bytes of every weight a decode step reads once (the embedding table is only gathered)."""
+    h, i, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    d = cfg["head_dim"]
+    q, kv = cfg["num_attention_heads"] * d, cfg["num_key_value_heads"] * d
+    per_layer = (q + 2 * kv) * h + h * q + 2 * i * h + h * i + 2 * h
+    return (cfg["num_hidden_layers"] * per_layer + v * h + h) * elem
+
+
+def kv_bytes_per_token(cfg: dict, elem: int) -> int:
+    return 2 * cfg["num_hidden_layers"] * cfg["num_key_value_heads"] * cfg["head_dim"] * elem
+
+
+def prefill_flops(cfg: dict, tokens: int) -> float:
+    h, i, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    d = cfg["head_dim"]
+    q, kv = cfg["num_attention_heads"] * d, cfg["num_key_value_heads"] * d
+    per_layer_params = (q + 2 * kv) * h + h * q + 2 * i * h + h * i
+    linear = 2.0 * tokens * cfg["num_hidden_layers"] * per_layer_params
+    # causal attention: QK^T and PV over tokens*(tokens+1)/2 query-key pairs per head
+    attention = 4.0 * (tokens * (tokens + 1) / 2) * d * cfg["num_attention_heads"] * cfg["num_hidden_layers"]
+    head = 2.0 * v * h
+    return linear + attention + head
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=256)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--layers", type=int, default=FULL_LAYERS)
+    parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
+    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    parser.add_argument("--no-prefill", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+    if not 0 < args.steps <= PROMPT_LEN:
+        print(f"bench.py: --steps must be in 1..{PROMPT_LEN} (decoding runs from 2,048 to at most 4,096)")
+        return 2
+
+    import numpy as np
+    import torch
+
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.sampling import SamplingParams, sample_tokens
+
+    cfg = dict(LLAMA_31_8B)
+    cfg["num_hidden_layers"] = args.layers
+    elem = 2 if args.dtype == "bfloat16" else 4
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    context_end = PROMPT_LEN + args.warmup + args.steps
+    pages_per_request = -(-(context_end + 1) // BLOCK_SIZE)
+    num_blocks = max(batches) * pages_per_request + 8
+    runner = ModelRunner.from_random(
+        cfg,
+        seed=0,
+        dtype=args.dtype,
+        num_blocks=num_blocks,
+        block_size=BLOCK_SIZE,
+        max_concurrent=max(batches),
+    )
+    rng = np.random.default_rng(0)
+    greedy = SamplingParams()
+
+    def sync() -> None:
+        torch.cuda.synchronize()
+
+    def prefill(request_id, tokens) -> torch.Tensor:
+        return runner.step([StepEntry(request_id, tokens, [len(tokens) - 1])])
+
+    def measure_decode(batch: int) -> tuple[float, float]:
+        """(seconds per step, mean context length) over `--steps` decode steps."""
+        ids = [f"b{batch}_{i}" for i in range(batch)]
+        last = []
+        for rid in ids:
+            prompt = rng.integers(0, cfg["vocab_size"], size=PROMPT_LEN).tolist()
+            logits = prefill(rid, prompt)
+            last.append(int(sample_tokens(logits, [greedy], [0], [0]).tolist()[0]))
+        params, seeds = [greedy] * batch, [0] * batch
+
+        def one_step(tokens: list[int], draw: int) -> list[int]:
+            logits = runner.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
+            return sample_tokens(logits, params, seeds, [draw] * batch).tolist()
+
+        for w in range(args.warmup):
+            last = one_step(last, w)
+        sync()
+        started = time.perf_counter()
+        for k in range(args.steps):
+            last = one_step(last, args.warmup + k)
+        sync()
+        seconds = (time.perf_counter() - started) / args.steps
+        for rid in ids:
+            runner.free_request(rid)
+        mean_context = PROMPT_LEN + args.warmup + (args.steps + 1) / 2
+        return seconds, mean_context
+
+    result_prefill = None
+    if not args.no_prefill:
+        times = []
+        for rep in range(4):
+            prompt = rng.integers(0, cfg["vocab_size"], size=PROMPT_LEN).tolist()
+            sync()
+            started = time.perf_counter()
+            prefill(f"p{rep}", prompt)
+            sync()
+            times.append(time.perf_counter() - started)
+            runner.free_request(f"p{rep}")
+        seconds = min(times[1:])
+        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+        result_prefill = {
+            "value": round(PROMPT_LEN / seconds, 1),
+            "tokens": PROMPT_LEN,
+            "ms": round(seconds * 1e3, 3),
+            "frac": round(prefill_flops(cfg, PROMPT_LEN) / seconds / peak, 4),
+        }
+
+    per_batch: dict[int, tuple[float, float]] = {}
+    for batch in batches:
+        per_batch[batch] = measure_decode(batch)
+
+    seconds, mean_context = per_batch[args.batch]
+    step_bytes = weight_bytes(cfg, elem) + args.batch * mean_context * kv_bytes_per_token(cfg, elem)
+    achieved = step_bytes / seconds / 1e9
+    line = {
+        "metric": "decode tok/s at batch 8, Llama-3.1-8B layer sizes, 2048-token prompts",
+        "value": round(args.batch / seconds, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(seconds * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: uniform-random token ids, random-init weights N(0, 0.02)",
+        "config": {
+            "model": "Llama-3.1-8B layer sizes",
+            "layers": args.layers,
+            "layers_full_model": FULL_LAYERS,
+            "hidden_size": cfg["hidden_size"],
+            "num_attention_heads": cfg["num_attention_heads"],
+            "num_key_value_heads": cfg["num_key_value_heads"],
+            "head_dim": cfg["head_dim"],
+            "intermediate_size": cfg["intermediate_size"],
+            "vocab_size": cfg["vocab_size"],
+            "global_batch": args.batch,
+            "seq_len": PROMPT_LEN,
+            "context_start": PROMPT_LEN + args.warmup,
+            "context_end": context_end,
+            "kv_block_size": BLOCK_SIZE,
+            "parallelism": "single GPU",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": PEAK_HBM_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / PEAK_HBM_GBS, 4),
+        },
+    }
+    if result_prefill is not None:
+        line["prefill"] = result_prefill
+    points = {f"decode_b{b}": round(b / per_batch[b][0], 2) for b in batches if b != args.batch}
+    if points:
+        line["points"] = points
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
