@@ -1,0 +1,248 @@
+"""The scheduler's decisions, with a model-free runner over the real cache manager (no GPU).
+
+The fake runner's "logits" are a pure function of the tokens a request has fed so
+far, so the tokens a request generates must not depend on batching, portions or
+preemption; it also records every step so the tests can read the decisions.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from mini_infer_amd.cache import CacheManager
+from mini_infer_amd.engine.request import Request
+from mini_infer_amd.engine.scheduler import ContinuousScheduler
+from mini_infer_amd.exceptions import OutOfMemoryError
+from mini_infer_amd.parts.base import CacheNeeds, PagedKVNeeds
+from mini_infer_amd.sampling import SamplingParams
+
+VOCAB = 50
+
+
+def next_token(history: list[int]) -> int:
+    return (sum(history) * 31 + 7 * len(history)) % VOCAB
+
+
+class FakeRunner:
+    def __init__(self, num_blocks=64, block_size=4, max_concurrent=8):
+        self.num_blocks, self.block_size = num_blocks, block_size
+        self.cache = CacheManager([CacheNeeds(pages=PagedKVNeeds(1, 16))], page_size=block_size,
+                                  num_pages=num_blocks, max_requests=max_concurrent, allocate_storage=False)
+        self.history: dict[int, list[int]] = {}
+        self.steps: list[list[tuple[int, int, tuple]]] = []
+
+    def num_free_blocks(self):
+        return self.cache.num_free_pages()
+
+    def step(self, entries):
+        extents = {e.request_id: len(e.tokens) for e in entries}
+        self.cache.reserve(extents)  # raises OutOfMemoryError with nothing changed
+        rows = []
+        for e in entries:
+            if self.cache.length(e.request_id) == 0:
+                self.history[e.request_id] = []
+            assert len(self.history[e.request_id]) == self.cache.length(e.request_id)
+            for i, token in enumerate(e.tokens):
+                self.history[e.request_id].append(token)
+                if i in e.want:
+                    row = torch.zeros(VOCAB)
+                    row[next_token(self.history[e.request_id])] = 1.0
+                    rows.append(row)
+        self.cache.commit(extents)
+        self.cache.check()
+        self.steps.append([(e.request_id, len(e.tokens), tuple(e.want)) for e in entries])
+        return torch.stack(rows) if rows else torch.zeros((0, VOCAB))
+
+
+def argmax_sampler(logits, params, seeds, draws):
+    assert logits.shape[0] == len(params) == len(seeds) == len(draws)
+    return logits.argmax(dim=-1).tolist()
+
+
+def expected_tokens(prompt, count, eos=None):
+    history, out = list(prompt), []
+    for _ in range(count):
+        token = next_token(history)
+        if token == eos:
+            break
+        out.append(token)
+        history.append(token)
+    return out
+
+
+def make(runner, **kwargs):
+    kwargs.setdefault("sampler", argmax_sampler)
+    return ContinuousScheduler(runner, **kwargs)
+
+
+def prompt(n, seed):
+    return np.random.default_rng(seed).integers(0, VOCAB, size=n).tolist()
+
+
+def test_one_request_runs_to_length_and_frees_its_pages():
+    runner = FakeRunner()
+    sched = make(runner)
+    result = sched.run(Request(prompt(10, 0), SamplingParams(), max_tokens=6))
+    assert result.tokens == expected_tokens(prompt(10, 0), 6)
+    assert result.finish_reason == "length" and result.prompt_tokens == 10
+    assert runner.num_free_blocks() == runner.num_blocks
+    # the prompt in one step, then one token a step; the last emitted token is never fed
+    assert [s[0][1] for s in runner.steps] == [10, 1, 1, 1, 1, 1]
+    assert len(runner.history[0]) == 10 + 5
+
+
+def test_prompt_is_cut_by_chunk_size_and_logits_wanted_only_at_its_end():
+    runner = FakeRunner()
+    sched = make(runner, chunk_size=4)
+    result = sched.run(Request(prompt(10, 1), SamplingParams(), max_tokens=2))
+    assert [(n, want) for _, n, want in (s[0] for s in runner.steps)] == [(4, ()), (4, ()), (2, (1,)), (1, (0,))]
+    assert result.tokens == expected_tokens(prompt(10, 1), 2)
+
+
+def test_token_budget_decodes_first_then_portions_in_admission_order():
+    runner = FakeRunner()
+    sched = make(runner, chunk_size=100, max_num_batched_tokens=8)
+    handles = [sched.submit(Request(prompt(n, n), SamplingParams(), max_tokens=4)) for n in (3, 9, 12)]
+    while sched.step():
+        pass
+    for step in runner.steps:
+        assert sum(n for _, n, _ in step) <= 8
+    # step 0: request 0 whole (3), request 1 gets the remaining 5 of the budget
+    assert runner.steps[0] == [(0, 3, (2,)), (1, 5, ())]
+    # step 1: request 0 decodes first (1 token), then request 1's last 4, then 3 of request 2
+    assert runner.steps[1] == [(0, 1, (0,)), (1, 4, (3,)), (2, 3, ())]
+    assert any(n == 2 or n == 1 for s in runner.steps for _, n, _ in s)
+    for handle, n in zip(handles, (3, 9, 12)):
+        assert handle.wait().tokens == expected_tokens(prompt(n, n), 4)
+    assert runner.num_free_blocks() == runner.num_blocks
+
+
+def test_batched_equals_serial():
+    prompts = [prompt(n, 10 + n) for n in (1, 5, 17, 30, 8)]
+    serial = []
+    for p in prompts:
+        serial.append(make(FakeRunner()).run(Request(p, SamplingParams(), max_tokens=7)).tokens)
+    runner = FakeRunner()
+    sched = make(runner, chunk_size=6, max_num_batched_tokens=16, max_concurrent=3)
+    results = sched.run_all([Request(p, SamplingParams(), max_tokens=7) for p in prompts])
+    assert [r.tokens for r in results] == serial
+    assert max(len(s) for s in runner.steps) == 3  # never more than max_concurrent live
+    assert runner.num_free_blocks() == runner.num_blocks
+
+
+def test_eos_stops_and_is_not_emitted():
+    p = prompt(6, 3)
+    free_run = expected_tokens(p, 10)
+    eos = free_run[3]
+    stop_at = free_run.index(eos)
+    runner = FakeRunner()
+    result = make(runner, eos_token_id=eos).run(Request(p, SamplingParams(), max_tokens=10))
+    assert result.finish_reason == "stop" and result.tokens == free_run[:stop_at]
+    ignoring = make(FakeRunner(), eos_token_id=eos).run(
+        Request(p, SamplingParams(ignore_eos=True), max_tokens=10))
+    assert ignoring.finish_reason == "length" and ignoring.tokens == free_run
+
+
+def test_empty_prompt_zero_max_tokens_and_cancel():
+    sched = make(FakeRunner())
+    assert sched.run(Request([], SamplingParams(), max_tokens=5)).finish_reason == "stop"
+    assert sched.run(Request([1, 2], SamplingParams(), max_tokens=0)).finish_reason == "length"
+    handle = sched.submit(Request(prompt(5, 0), SamplingParams(), max_tokens=100))
+    sched.step()
+    handle.cancel()
+    result = handle.wait()
+    assert result.finish_reason == "cancelled" and 1 <= len(result.tokens) < 100
+    assert sched.runner.num_free_blocks() == sched.runner.num_blocks
+
+
+def test_prompt_that_can_never_fit_is_cancelled_others_go_on():
+    runner = FakeRunner(num_blocks=4, block_size=4)
+    sched = make(runner, decode_headroom_blocks=1)
+    big = sched.submit(Request(prompt(17, 0), SamplingParams(), max_tokens=2))
+    small = sched.submit(Request(prompt(5, 1), SamplingParams(), max_tokens=2))
+    while sched.step():
+        pass
+    assert big.wait().finish_reason == "cancelled" and big.wait().tokens == []
+    assert small.wait().tokens == expected_tokens(prompt(5, 1), 2)
+    assert sched.stats["rejected"] == 1
+
+
+def test_admission_waits_for_pages_and_fills_a_freed_seat():
+    runner = FakeRunner(num_blocks=6, block_size=4)
+    sched = make(runner, decode_headroom_blocks=1, max_concurrent=4)
+    first = sched.submit(Request(prompt(14, 0), SamplingParams(), max_tokens=3))   # 4 pages + 1 headroom
+    second = sched.submit(Request(prompt(10, 1), SamplingParams(), max_tokens=3))  # needs 3 + 1: must wait
+    sched.step()
+    assert [rid for rid, _, _ in runner.steps[0]] == [0]
+    while sched.step():
+        pass
+    assert first.wait().tokens == expected_tokens(prompt(14, 0), 3)
+    assert second.wait().tokens == expected_tokens(prompt(10, 1), 3)
+    # the second request was admitted in the step right after the first finished
+    first_step_of_second = next(i for i, s in enumerate(runner.steps) if any(r == 1 for r, _, _ in s))
+    last_step_of_first = max(i for i, s in enumerate(runner.steps) if any(r == 0 for r, _, _ in s))
+    assert first_step_of_second == last_step_of_first + 1
+
+
+def test_out_of_pages_preempts_the_youngest_and_recomputes_it():
+    """Decoding outgrows the pool: the youngest request is freed, queued first and
+    fed again (prompt + what it generated); every request still gets the tokens it
+    would get alone, and nothing is emitted twice."""
+    prompts = [prompt(8, 20), prompt(8, 21), prompt(8, 22)]
+    runner = FakeRunner(num_blocks=9, block_size=4)
+    sched = make(runner, decode_headroom_blocks=0, max_concurrent=3)
+    results = sched.run_all([Request(p, SamplingParams(), max_tokens=12) for p in prompts])
+    assert sched.stats["preemptions"] >= 1
+    for p, result in zip(prompts, results):
+        assert result.tokens == expected_tokens(p, 12) and result.finish_reason == "length"
+    assert runner.num_free_blocks() == runner.num_blocks
+    # a preempted request comes back as a portion longer than its prompt
+    assert any(n > 8 for s in runner.steps for _, n, _ in s)
+
+
+def test_request_that_outgrows_the_whole_pool_alone_is_cancelled_with_what_it_has():
+    runner = FakeRunner(num_blocks=3, block_size=4)
+    sched = make(runner, decode_headroom_blocks=0)
+    result = sched.run(Request(prompt(8, 5), SamplingParams(), max_tokens=50))
+    assert result.finish_reason == "cancelled"
+    assert result.tokens == expected_tokens(prompt(8, 5), len(result.tokens)) and len(result.tokens) >= 4
+    assert runner.num_free_blocks() == runner.num_blocks
+
+
+def test_sampler_gets_seed_and_draw_index_per_request():
+    seen = []
+
+    def sampler(logits, params, seeds, draws):
+        seen.append((list(seeds), list(draws), [p.temperature for p in params]))
+        return logits.argmax(dim=-1).tolist()
+
+    sched = make(FakeRunner(), sampler=sampler, base_seed=5)
+    sched.run_all([
+        Request(prompt(4, 0), SamplingParams(temperature=0.8, seed=1234), max_tokens=3),
+        Request(prompt(6, 1), SamplingParams(), max_tokens=2),
+    ])
+    assert seen[0][0][0] == 1234 and seen[0][1] == [0, 0] and seen[0][2] == [0.8, 0.0]
+    assert seen[1][1] == [1, 1] and seen[2][1] == [2]
+    assert seen[0][0][1] != 1234  # a request without a seed gets one of its own
+
+
+def test_engine_thread_runs_requests_and_stop_cancels():
+    sched = make(FakeRunner())
+    sched.start()
+    try:
+        result = sched.run(Request(prompt(9, 2), SamplingParams(), max_tokens=5))
+        assert result.tokens == expected_tokens(prompt(9, 2), 5)
+    finally:
+        sched.stop()
+    assert sched.runner.num_free_blocks() == sched.runner.num_blocks
+
+
+def test_out_of_memory_with_nothing_to_preempt_is_raised():
+    class Broken(FakeRunner):
+        def step(self, entries):
+            raise OutOfMemoryError("always")
+
+    sched = make(Broken())
+    handle = sched.submit(Request(prompt(4, 0), SamplingParams(), max_tokens=2))
+    sched.step()  # preempting the only request cancels it
+    assert handle.wait().finish_reason == "cancelled"
