@@ -1,7 +1,7 @@
 // True float32 matrix product for the 32-bit path: C[M,N] = A[M,K] * W[N,K]^T.
 // Plain FMA, no reduced-precision matrix mode.  Each output element is summed by
-// one thread over k = 0..K-1 in order, so a row's result does not depend on how
-// many other rows are in the batch or on where its tile lies.
+// one thread in a fixed order (16-deep slices, slice by slice), so a row's result
+// does not depend on how many other rows are in the batch or on where its tile lies.
 //
 // 64x64 output tile per 256-thread block, 16-deep K slices staged in LDS, 4x4
 // outputs per thread.  Any M, N, K; rows of A and W may have strides.
@@ -49,6 +49,13 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
         w_s[l_k + i][l_row] = (r < n && k0 + l_k + i < k) ? src[i] : 0.f;
     }
     __syncthreads();
+    // two-level sum: each 16-deep slice is summed on its own, then added to the total,
+    // which keeps the rounding error of long rows (K in the thousands) small
+    float part[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) part[i][j] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < BK; ++kk) {
       float av[4], wv[4];
@@ -59,8 +66,12 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        for (int j = 0; j < 4; ++j) part[i][j] = fmaf(av[i], wv[j], part[i][j]);
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] += part[i][j];
     __syncthreads();
   }
 

@@ -34,6 +34,8 @@ class Registry(Generic[T]):
 
     def lookup(self, name: str) -> T:
         if name not in self._entries:
+            _load_builtins()
+        if name not in self._entries:
             raise ValueError(
                 f"no {self.what} named {name!r}; supported: {sorted(self._entries)}"
             )
@@ -47,6 +49,12 @@ class Registry(Generic[T]):
 
     def __contains__(self, name: str) -> bool:
         return name in self._entries
+
+
+def _load_builtins() -> None:
+    """Import the packages whose import registers the built-in parts and architecture."""
+    import mini_infer_amd.models  # noqa: F401
+    import mini_infer_amd.parts  # noqa: F401
 
 
 # name in config.json's `architectures[0]` -> Architecture (models/architecture.py)

@@ -1,0 +1,485 @@
+"""The engine above the kernels: parts alone, generation through the entry points,
+the replay program, long decoding, first tokens, order lists, windows, and a toy
+mixer with state of its own registered from outside the package."""
+
+import json
+import math
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as pl
+import replay_util as ru
+import tiny
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DTYPES = ["float32", "bfloat16"]
+TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def _folder(tmp_path, name, seed):
+    cfg, block = tiny.CONFIGS[name]
+    weights = tiny.make_weights(cfg, seed)
+    return cfg, block, weights, tiny.write_model_dir(tmp_path / f"model{name}{seed}", cfg, weights)
+
+
+def _plain_greedy(cfg, weights, prompt, count):
+    sequence = list(prompt)
+    for _ in range(count):
+        sequence.append(pl.greedy(pl.llama_logits(cfg, weights, np.array(sequence))[-1]))
+    return sequence[len(prompt):]
+
+
+# -- parts alone -----------------------------------------------------------------
+
+
+def _context(positions, cu, seq_lens, slot_mapping=None, block_table=None, page_size=4):
+    from mini_infer_amd.parts import StepContext
+
+    t = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)  # noqa: E731
+    token_request = [b for b in range(len(cu) - 1) for _ in range(cu[b + 1] - cu[b])]
+    return StepContext(
+        num_tokens=len(positions), num_requests=len(cu) - 1, page_size=page_size, token_ids=t([0] * len(positions)),
+        positions=t(positions), token_request=t(token_request), cu_seqlens_q=t(cu), seq_lens=t(seq_lens),
+        state_slots=t(list(range(len(cu) - 1))), logit_rows=t([]),
+        slot_mapping=[t(slot_mapping)] if slot_mapping is not None else [],
+        block_tables=[t(block_table)] if block_table is not None else [],
+        max_q_len=max(cu[b + 1] - cu[b] for b in range(len(cu) - 1)), max_seq_len=max(seq_lens),
+        host_cu_seqlens_q=cu, host_seq_lens=seq_lens, host_state_slots=list(range(len(cu) - 1)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_norm_part(dtype):
+    from mini_infer_amd.registry import NORMS
+
+    norm = NORMS.lookup("rms_norm")({"kind": "rms_norm", "hidden_size": 100, "eps": 2e-6}, TORCH[dtype], DEV)
+    assert list(norm.param_specs("x.")) == ["x.weight"]
+    w = torch.rand(100) + 0.5
+    norm.load_params("x.", lambda name: w.to(TORCH[dtype]).to(DEV))
+    residual = torch.randn(3, 100, device=DEV)
+    delta = torch.randn(3, 100, device=DEV).to(TORCH[dtype])
+    expected = pl.rms_norm((residual.double() + delta.double()).cpu().numpy(),
+                           w.to(TORCH[dtype]).double().numpy(), 2e-6)
+    out = norm.forward(delta, residual)
+    assert np.abs(out.float().cpu().numpy() - expected).max() < (1e-5 if dtype == "float32" else 4e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_feed_forward_part(dtype):
+    from mini_infer_amd.registry import FEED_FORWARDS
+
+    ffn = FEED_FORWARDS.lookup("swiglu")(
+        {"kind": "swiglu", "hidden_size": 90, "intermediate_size": 130}, TORCH[dtype], DEV)
+    assert sorted(ffn.param_specs("m.")) == ["m.down_proj.weight", "m.gate_proj.weight", "m.up_proj.weight"]
+    rng = np.random.default_rng(0)
+    w = {"m.gate_proj.weight": rng.standard_normal((130, 90)) / 9, "m.up_proj.weight": rng.standard_normal((130, 90)) / 9,
+         "m.down_proj.weight": rng.standard_normal((90, 130)) / 11}
+    w = {k: tiny.bf16_round(v) for k, v in w.items()}
+    ffn.load_params("m.", lambda name: torch.from_numpy(w[name]).to(TORCH[dtype]).to(DEV))
+    x = torch.from_numpy(tiny.bf16_round(rng.standard_normal((5, 90)))).to(DEV)
+    expected = pl.swiglu(x.cpu().numpy(), w["m.gate_proj.weight"], w["m.up_proj.weight"], w["m.down_proj.weight"])
+    out = ffn.forward(x.to(TORCH[dtype]), None)
+    assert np.abs(out.float().cpu().numpy() - expected).max() < (1e-5 if dtype == "float32" else 4e-2)
+    with pytest.raises(NotImplementedError):
+        FEED_FORWARDS.lookup("swiglu")({"kind": "swiglu", "hidden_size": 8, "intermediate_size": 8,
+                                        "activation": "gelu"}, TORCH[dtype], DEV)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [None, 5])
+def test_attention_part_in_two_portions(dtype, window):
+    """The mixer alone: a sequence fed as 7 + 4 tokens through its own little cache."""
+    from mini_infer_amd.parts import LayerCache
+    from mini_infer_amd.registry import MIXERS
+
+    hidden, heads, kv_heads, head_dim, page = 40, 6, 2, 16, 4
+    desc = {"kind": "gqa_attention", "hidden_size": hidden, "num_heads": heads, "num_kv_heads": kv_heads,
+            "head_dim": head_dim, "window": window,
+            "position": {"kind": "rotary", "head_dim": head_dim, "theta": 100.0}}
+    mixer = MIXERS.lookup("gqa_attention")(desc, TORCH[dtype], DEV, {})
+    needs = mixer.cache_needs()
+    assert (needs.pages.num_kv_heads, needs.pages.head_dim, needs.pages.window) == (kv_heads, head_dim, window)
+    rng = np.random.default_rng(1)
+    w = {f"a.{n}_proj.weight": tiny.bf16_round(rng.standard_normal(s) / 6) for n, s in
+         (("q", (96, 40)), ("k", (32, 40)), ("v", (32, 40)), ("o", (40, 96)))}
+    mixer.load_params("a.", lambda name: torch.from_numpy(w[name]).to(TORCH[dtype]).to(DEV))
+    x = tiny.bf16_round(rng.standard_normal((11, hidden)))
+    cos, sin = pl.rope_tables(np.arange(11), pl.inv_freq_default(head_dim, 100.0))
+    expected, _ = pl.attention_layer(x, w["a.q_proj.weight"], w["a.k_proj.weight"], w["a.v_proj.weight"],
+                                     w["a.o_proj.weight"], cos, sin, heads, kv_heads, head_dim, window)
+    cache = LayerCache(group=0, k_pages=torch.zeros((5, kv_heads, page, head_dim), dtype=TORCH[dtype], device=DEV),
+                       v_pages=torch.zeros((5, kv_heads, page, head_dim), dtype=TORCH[dtype], device=DEV))
+    table = [[3, 0, 4]]
+    slots = [table[0][p // page] * page + p % page for p in range(11)]
+    xt = torch.from_numpy(x).to(TORCH[dtype]).to(DEV)
+    first = mixer.forward(xt[:7], _context(list(range(7)), [0, 7], [7], slots[:7], table), cache)
+    second = mixer.forward(xt[7:], _context(list(range(7, 11)), [0, 4], [11], slots[7:], table), cache)
+    got = torch.cat([first, second]).float().cpu().numpy()
+    assert np.abs(got - expected).max() < (2e-5 if dtype == "float32" else 4e-2)
+
+
+# -- generation through the entry points ---------------------------------------------
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_llm(tmp_path, name):
+    """Tiny A: 3 requests (5, 17, 32 tokens), 8 greedy tokens each, block size 4.
+    Tiny B: 4 requests (1, 40, 97, 150 tokens) under a 32-token budget, block size 16."""
+    from mini_infer_amd.engine.llm import LLM
+
+    cfg, block, weights, folder = _folder(tmp_path, name, 50)
+    lengths, new_tokens = ((5, 17, 32), 8) if name == "A" else ((1, 40, 97, 150), 12)
+    prompts = [tiny.random_tokens(cfg, n, seed=n) for n in lengths]
+    llm = LLM(folder, dtype="float32", num_blocks=96, block_size=block, max_num_batched_tokens=32, chunk_size=32)
+    results = llm.generate(prompts, max_tokens=new_tokens)
+    for prompt, result in zip(prompts, results):
+        assert result.tokens == _plain_greedy(cfg, weights, prompt, new_tokens)
+        assert result.finish_reason == "length" and result.prompt_tokens == len(prompt)
+    assert llm.runner.num_free_blocks() == 96
+    assert max(len(s) for s in [llm.scheduler.stats]) >= 1
+
+
+def test_greedy_generation_in_bfloat16_stays_on_near_maxima(tmp_path):
+    """bfloat16 may pick another token where two logits nearly tie; every token it picks
+    must be within rounding of the plain model's maximum given the engine's own prefix."""
+    from mini_infer_amd.engine.llm import LLM
+
+    cfg, block, weights, folder = _folder(tmp_path, "B", 51)
+    prompts = [tiny.random_tokens(cfg, n, seed=n) for n in (3, 40)]
+    llm = LLM(folder, dtype="bfloat16", num_blocks=32, block_size=block)
+    for prompt, result in zip(prompts, llm.generate(prompts, max_tokens=10)):
+        sequence = list(prompt)
+        for token in result.tokens:
+            logits = pl.llama_logits(cfg, weights, np.array(sequence))[-1]
+            assert logits[token] > logits.max() - 2 * ru.BF16_REL_TOL * max(1.0, np.abs(logits).max())
+            sequence.append(token)
+
+
+def test_seeded_temperature_generation_is_reproducible_and_independent_of_batching(tmp_path):
+    """Two greedy and two sampled requests (temperature 0.8): the sampled ones give the
+    same tokens alone, batched, and under another chunking."""
+    from mini_infer_amd.engine.llm import LLM
+    from mini_infer_amd.sampling import SamplingParams
+
+    cfg, block, weights, folder = _folder(tmp_path, "B", 52)
+    prompts = [tiny.random_tokens(cfg, n, seed=n) for n in (1, 40, 97, 150)]
+    params = [SamplingParams(), SamplingParams(temperature=0.8, seed=7), SamplingParams(),
+              SamplingParams(temperature=0.8, seed=8, top_k=50, top_p=0.9)]
+    batched = LLM(folder, dtype="float32", num_blocks=96, block_size=block, max_num_batched_tokens=32,
+                  chunk_size=32).generate(prompts, params, max_tokens=12)
+    other = LLM(folder, dtype="float32", num_blocks=96, block_size=block, max_num_batched_tokens=512,
+                max_concurrent=2).generate(prompts, params, max_tokens=12)
+    assert [r.tokens for r in batched] == [r.tokens for r in other]
+    alone = LLM(folder, dtype="float32", num_blocks=96, block_size=block).generate([prompts[3]], [params[3]], max_tokens=12)
+    assert alone[0].tokens == batched[3].tokens
+    assert batched[0].tokens == _plain_greedy(cfg, weights, prompts[0], 12)
+    reseeded = LLM(folder, dtype="float32", num_blocks=96, block_size=block).generate(
+        [prompts[1]], [SamplingParams(temperature=0.8, seed=9)], max_tokens=12)
+    assert reseeded[0].tokens != batched[1].tokens
+
+
+def test_preemption_on_the_real_engine_keeps_outputs(tmp_path):
+    from mini_infer_amd.engine.llm import LLM
+
+    cfg, block, weights, folder = _folder(tmp_path, "A", 53)
+    prompts = [tiny.random_tokens(cfg, 12, seed=s) for s in (1, 2, 3)]
+    llm = LLM(folder, dtype="float32", num_blocks=14, block_size=block, decode_headroom_blocks=0)
+    results = llm.generate(prompts, max_tokens=14)
+    assert llm.scheduler.stats["preemptions"] >= 1
+    for prompt, result in zip(prompts, results):
+        assert result.tokens == _plain_greedy(cfg, weights, prompt, 14)
+    assert llm.runner.num_free_blocks() == 14
+
+
+def test_command_line_generates(tmp_path):
+    cfg, block, weights, folder = _folder(tmp_path, "A", 54)
+    prompt = tiny.random_tokens(cfg, 6, seed=1)
+    done = subprocess.run(
+        [sys.executable, "-m", "mini_infer_amd", "generate", "--model", str(folder), "--prompt-ids",
+         " ".join(map(str, prompt)), "--max-tokens", "5", "--dtype", "float32", "--block-size", str(block),
+         "--num-blocks", "32"],
+        cwd=ROOT, capture_output=True, text=True, timeout=110)
+    assert done.returncode == 0, done.stderr[-2000:]
+    record = json.loads(done.stdout.strip().splitlines()[-1])
+    assert record["tokens"] == _plain_greedy(cfg, weights, prompt, 5) and record["finish_reason"] == "length"
+
+
+# -- the replay program ----------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_run_program(tmp_path, dtype):
+    """bin/trace_run as a user runs it: JSON steps on stdin, <step>.f32 files, `done <step>` lines."""
+    cfg, block, weights, folder = _folder(tmp_path, "B", 55)
+    requests = {f"r{i}": tiny.random_tokens(cfg, n, seed=i) for i, n in enumerate((40, 70, 33, 64, 50))}
+    expected = {rid: pl.llama_logits(cfg, weights, np.array(t)) for rid, t in requests.items()}
+    schedule = ru.schedule_mixed(requests, seed=5)
+    # each request's count rounded up to a multiple of 64
+    fed = {rid: 0 for rid in requests}
+    live, peak = set(), 0
+    lines, wanted = [], []
+    for number, step in enumerate(schedule):
+        entries = []
+        for rid, count in step["feed"].items():
+            want = [count - 1] if count > 1 else [0]
+            entries.append({"id": rid, "tokens": requests[rid][fed[rid]: fed[rid] + count], "want": want})
+            wanted.append((number, rid, fed[rid] + want[0]))
+            fed[rid] += count
+            live.add(rid)
+        peak = max(peak, sum(-(-fed[r] // 64) * 64 for r in live))
+        live -= set(step["end"])
+        lines.append(json.dumps({"step": number, "entries": entries, "end": step["end"]}))
+    out_dir = tmp_path / "out"
+    done = subprocess.run(
+        [os.path.join(ROOT, "bin", "trace_run"), "--model", str(folder), "--dtype", dtype, "--out", str(out_dir),
+         "--max-tokens", str(peak)],
+        input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=110)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert done.stdout.split("\n")[:-1] == [f"done {n}" for n in range(len(schedule))]
+    at = {}
+    for number, rid, position in wanted:
+        rows = np.fromfile(out_dir / f"{number}.f32", dtype="<f4").reshape(-1, cfg["vocab_size"])
+        row = rows[at.get(number, 0)]
+        at[number] = at.get(number, 0) + 1
+        ru.assert_close(row[None], expected[rid][position][None], dtype, f"step {number} {rid}@{position}")
+
+
+# -- long decoding, first tokens -----------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(tmp_path, dtype):
+    """A short prompt and 380 tokens one by one: far past the rope's original length
+    (64 for this configuration), across many pages."""
+    from mini_infer_amd.engine import ModelRunner
+
+    cfg, block, weights, folder = _folder(tmp_path, "B", 56)
+    requests = {"long": tiny.random_tokens(cfg, 400, seed=9)}
+    expected = {"long": pl.llama_logits(cfg, weights, np.array(requests["long"]))}
+    schedule = ru.schedule_prefill_then_decode(requests, tail=380)
+    runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=26, block_size=block)
+    got = ru.run_schedule(runner, requests, schedule)
+    ru.assert_close(got["long"], expected["long"], dtype, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_first_tokens_of_a_sequence(tmp_path, name, dtype):
+    from mini_infer_amd.engine import ModelRunner
+
+    cfg, block, weights, folder = _folder(tmp_path, name, 57)
+    runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=16, block_size=block)
+    for length in (1, 2, 3):
+        requests = {f"s{length}": tiny.random_tokens(cfg, length, seed=length)}
+        expected = pl.llama_logits(cfg, weights, np.array(requests[f"s{length}"]))
+        token_by_token = [{"feed": {f"s{length}": 1}} for _ in range(length)]
+        token_by_token[-1]["end"] = [f"s{length}"]
+        got = ru.run_schedule(runner, requests, token_by_token)
+        ru.assert_close(got[f"s{length}"], expected, dtype, f"{name} first {length} tokens")
+
+
+def test_step_refuses_bad_batches(tmp_path):
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.exceptions import OutOfMemoryError
+
+    cfg, block, weights, folder = _folder(tmp_path, "A", 58)
+    runner = ModelRunner.from_pretrained(folder, dtype="float32", num_blocks=4, block_size=block)
+    with pytest.raises(ValueError, match="token ids"):
+        runner.step([StepEntry("a", [cfg["vocab_size"]], [0])])
+    with pytest.raises(ValueError, match="twice"):
+        runner.step([StepEntry("a", [1], [0]), StepEntry("a", [2], [0])])
+    with pytest.raises(ValueError, match="outside"):
+        runner.step([StepEntry("a", [1, 2], [2])])
+    with pytest.raises(OutOfMemoryError):
+        runner.step([StepEntry("a", [1] * 17, [])])
+    assert not runner.has_request("a") and runner.num_free_blocks() == 4  # nothing changed
+    assert runner.step([StepEntry("a", [1, 2, 3], [])]).shape == (0, cfg["vocab_size"])
+    assert runner.cache.length("a") == 3
+
+
+# -- the model as data: order lists, windows, a toy mixer from outside -----------------------
+
+
+def _register_variant(name, transform):
+    """An architecture defined here: Llama's spec with `transform` applied to it."""
+    from mini_infer_amd.config import ModelConfig
+    from mini_infer_amd.models.llama import llama_spec
+    from mini_infer_amd.models.spec import Architecture
+    from mini_infer_amd.registry import ARCHITECTURES
+
+    ARCHITECTURES.register(name, Architecture(name, ModelConfig.from_dict, lambda cfg: transform(llama_spec(cfg))))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_order_list_names_a_layer_twice_and_reads_another_cache(tmp_path, dtype):
+    import dataclasses
+
+    from mini_infer_amd.engine import ModelRunner
+    from mini_infer_amd.models.spec import LayerCall
+    from mini_infer_amd.registry import ARCHITECTURES
+
+    order = [LayerCall(0), LayerCall(1), LayerCall(0), LayerCall(1, reads_cache_of=1)]
+    _register_variant("LoopedTestLM", lambda spec: dataclasses.replace(spec, order=order))
+    try:
+        cfg = dict(tiny.TINY_A, architectures=["LoopedTestLM"])
+        weights = tiny.make_weights(cfg, 60)
+        folder = tiny.write_model_dir(tmp_path / "looped", cfg, weights)
+        requests = {"x": tiny.random_tokens(cfg, 45, 1), "y": tiny.random_tokens(cfg, 30, 2)}
+        plain_order = [(0, None), (1, None), (0, None), (1, 1)]
+        expected = {r: pl.llama_logits(cfg, weights, np.array(t), order=plain_order) for r, t in requests.items()}
+        runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=24, block_size=4)
+        assert len(runner.cache.groups) == 1 and runner.cache.groups[0].calls == [0, 1, 2]
+        got = ru.run_schedule(runner, requests, ru.schedule_mixed(requests, seed=2, tail=8))
+        for rid in requests:
+            ru.assert_close(got[rid], expected[rid], dtype, f"looped {rid}")
+    finally:
+        ARCHITECTURES.unregister("LoopedTestLM")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_layers_with_and_without_a_window_have_page_groups_of_their_own(tmp_path, dtype):
+    import copy
+    import dataclasses
+
+    from mini_infer_amd.cache import RELEASED
+    from mini_infer_amd.engine import ModelRunner
+    from mini_infer_amd.models.spec import LayerSpec
+    from mini_infer_amd.registry import ARCHITECTURES
+
+    def windowed(spec):
+        layers = []
+        for i, layer in enumerate(spec.layers):
+            block = copy.deepcopy(layer.block)
+            block["mixer"]["window"] = 6 if i % 2 == 0 else None
+            layers.append(LayerSpec(layer.prefix, block))
+        return dataclasses.replace(spec, layers=layers)
+
+    _register_variant("WindowedTestLM", windowed)
+    try:
+        cfg = dict(tiny.TINY_B, architectures=["WindowedTestLM"])
+        weights = tiny.make_weights(cfg, 61)
+        folder = tiny.write_model_dir(tmp_path / "windowed", cfg, weights)
+        requests = {"x": tiny.random_tokens(cfg, 61, 1), "y": tiny.random_tokens(cfg, 38, 2)}
+        expected = {r: pl.llama_logits(cfg, weights, np.array(t), window=[6, None, 6]) for r, t in requests.items()}
+        runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=10, block_size=4)
+        groups = {g.window: g for g in runner.cache.groups}
+        assert sorted(groups, key=str) == [6, None] and groups[6].calls == [0, 2] and groups[None].calls == [1]
+        from mini_infer_amd.engine import StepEntry
+
+        # x alone first: after 30 tokens the windowed group has given back all but two or three pages
+        logits = runner.step([StepEntry("x", requests["x"][:30], list(range(30)))]).cpu().numpy()
+        ru.assert_close(logits, expected["x"][:30], dtype, "windowed x[:30]")
+        assert groups[6].tables["x"][:6] == [RELEASED] * 6
+        assert groups[6].pool.num_free == 10 - 2 and groups[None].pool.num_free == 10 - 8
+        rest = {"x": requests["x"][30:], "y": requests["y"]}
+        # the full group has 2 pages left: y must wait there, so feed y in the windowed order only after x ends
+        got_x = runner.step([StepEntry("x", rest["x"][:8], list(range(8)))]).cpu().numpy()
+        ru.assert_close(got_x, expected["x"][30:38], dtype, "windowed x[30:38]")
+        runner.free_request("x")
+        got = ru.run_schedule(runner, {"y": requests["y"]}, ru.schedule_portions({"y": requests["y"]}, seed=1))
+        ru.assert_close(got["y"], expected["y"], dtype, "windowed y")
+        runner.cache.check()
+        assert all(g.pool.num_free == 10 for g in runner.cache.groups)
+    finally:
+        ARCHITECTURES.unregister("WindowedTestLM")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path, dtype):
+    """A mixer defined here, with state of fixed size per request (a decaying sum of its
+    inputs) and no pages, is registered, built from a layer description, loaded from a
+    checkpoint by name, and stepped in portions and mixed batches: no framework file changes."""
+    import copy
+    import dataclasses
+
+    from mini_infer_amd.engine import ModelRunner
+    from mini_infer_amd.models.spec import LayerSpec
+    from mini_infer_amd.parts import CacheNeeds, Mixer, ParamSpec, StateNeeds
+    from mini_infer_amd.registry import ARCHITECTURES, MIXERS
+
+    hidden = tiny.TINY_A["hidden_size"]
+    decay = 0.75
+
+    class DecayingSum(Mixer):
+        def param_specs(self, prefix):
+            return {prefix + "mix.weight": ParamSpec((hidden, hidden))}
+
+        def load_params(self, prefix, get):
+            self.weight = get(prefix + "mix.weight")
+
+        def cache_needs(self):
+            return CacheNeeds(state=StateNeeds((hidden,), torch.float32))
+
+        def forward(self, x, ctx, cache, writes_cache=True):
+            out = torch.empty_like(x)
+            for b, slot in enumerate(ctx.host_state_slots):
+                state = cache.state[slot]
+                for t in range(ctx.host_cu_seqlens_q[b], ctx.host_cu_seqlens_q[b + 1]):
+                    state = decay * state + x[t].float()
+                    out[t] = (self.weight.float() @ state).to(x.dtype)
+                cache.state[slot] = state
+            return out
+
+    MIXERS.register("decaying_sum", lambda desc, dtype_, device, shared=None: DecayingSum(dtype_, device))
+
+    def with_toy(spec):
+        layers = list(spec.layers)
+        block = copy.deepcopy(layers[1].block)
+        block["mixer"] = {"kind": "decaying_sum"}
+        layers[1] = LayerSpec(layers[1].prefix, block)
+        return dataclasses.replace(spec, layers=layers)
+
+    _register_variant("ToyStateTestLM", with_toy)
+    try:
+        cfg = dict(tiny.TINY_A, architectures=["ToyStateTestLM"])
+        weights = tiny.make_weights(cfg, 62)
+        for n in "qkvo":
+            del weights[f"model.layers.1.self_attn.{n}_proj.weight"]
+        rng = np.random.default_rng(3)
+        weights["model.layers.1.self_attn.mix.weight"] = tiny.bf16_round(rng.standard_normal((hidden, hidden)) / 16)
+        folder = tiny.write_model_dir(tmp_path / "toy", cfg, weights)
+
+        def plain(tokens):
+            """Layer 0 as Llama's, layer 1 with the decaying sum in place of attention."""
+            eps = cfg["rms_norm_eps"]
+            r = pl.embedding(weights["model.embed_tokens.weight"], np.array(tokens))
+            cos, sin = pl.rope_tables(np.arange(len(tokens)), pl.config_inv_freq(cfg))
+            p = "model.layers.0."
+            a, _ = pl.attention_layer(
+                pl.rms_norm(r, weights[p + "input_layernorm.weight"], eps),
+                *(weights[p + f"self_attn.{n}_proj.weight"] for n in "qkvo"), cos, sin, 4, 2, 16)
+            r = r + a
+            r = r + pl.swiglu(pl.rms_norm(r, weights[p + "post_attention_layernorm.weight"], eps),
+                              *(weights[p + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            p = "model.layers.1."
+            h = pl.rms_norm(r, weights[p + "input_layernorm.weight"], eps)
+            if dtype == "bfloat16":
+                h = tiny.bf16_round(h).astype(np.float64)
+            state, mixed = np.zeros(hidden), []
+            for row in h:
+                state = decay * state + row
+                mixed.append(weights[p + "self_attn.mix.weight"].astype(np.float64) @ state)
+            r = r + np.array(mixed)
+            r = r + pl.swiglu(pl.rms_norm(r, weights[p + "post_attention_layernorm.weight"], eps),
+                              *(weights[p + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            return pl.rms_norm(r, weights["model.norm.weight"], eps) @ weights["model.embed_tokens.weight"].astype(np.float64).T
+
+        requests = {f"t{i}": tiny.random_tokens(cfg, n, seed=i) for i, n in enumerate((20, 9, 14, 11, 17))}
+        expected = {rid: plain(t) for rid, t in requests.items()}
+        runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=24, block_size=4, max_concurrent=4)
+        caches = runner.cache.layer_caches()
+        assert caches[1].state.shape == (4, hidden) and caches[1].k_pages is None and caches[0].state is None
+        got = ru.run_schedule(runner, requests, ru.schedule_mixed(requests, seed=4, tail=5))
+        for rid in requests:
+            ru.assert_close(got[rid], expected[rid], dtype, f"toy {rid}")
+        runner.cache.check()
+        assert runner.cache.states.num_free == 4
+    finally:
+        ARCHITECTURES.unregister("ToyStateTestLM")
+        MIXERS.unregister("decaying_sum")

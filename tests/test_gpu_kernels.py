@@ -1,0 +1,305 @@
+"""Each HIP kernel alone against a plain reference, at other sizes than the engine's tiny models."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as pl
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _tol(dtype, scale=1.0):
+    return (2e-5 if dtype == torch.float32 else 2e-2) * scale
+
+
+def _rand(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,vocab", [(4096, 1000), (100, 301), (90, 17)])
+def test_embed_gather(dtype, hidden, vocab):
+    from mini_infer_amd import ops
+
+    table = _rand(vocab, hidden, dtype=dtype)
+    ids = torch.tensor([0, vocab - 1, 5, 5, vocab // 2], dtype=torch.int32, device=DEV)
+    out = ops.embed_gather(table, ids)
+    assert out.dtype == torch.float32
+    assert torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [4096, 100, 90, 9000])
+def test_add_rmsnorm(dtype, hidden):
+    from mini_infer_amd import ops
+
+    tokens, eps = 7, 3e-6
+    residual = _rand(tokens, hidden, seed=1, scale=2.0)
+    delta = _rand(tokens, hidden, dtype=dtype, seed=2)
+    weight = (_rand(hidden, seed=3) * 0.2 + 1.0).to(dtype)
+    expected_sum = residual.double() + delta.double()
+    expected = pl.rms_norm(expected_sum.cpu().numpy(), weight.double().cpu().numpy(), eps)
+
+    res = residual.clone()
+    out = ops.add_rmsnorm(delta, res, weight, eps)
+    assert torch.allclose(res, expected_sum.float(), atol=1e-6)  # the sum is stored, in float32
+    assert np.abs(out.float().cpu().numpy() - expected).max() < _tol(dtype, 4)
+
+    # first layer: nothing to add, residual untouched
+    res = residual.clone()
+    out = ops.add_rmsnorm(None, res, weight, eps)
+    assert torch.equal(res, residual)
+    plain = pl.rms_norm(residual.double().cpu().numpy(), weight.double().cpu().numpy(), eps)
+    assert np.abs(out.float().cpu().numpy() - plain).max() < _tol(dtype, 4)
+
+    # chosen rows only: the residual stays as it was
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    res = residual.clone()
+    out = ops.add_rmsnorm(delta, res, weight, eps, rows)
+    assert torch.equal(res, residual) and out.shape == (3, hidden)
+    assert np.abs(out.float().cpu().numpy() - expected[[5, 0, 5]]).max() < _tol(dtype, 4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("inter", [14336, 130, 7])
+def test_silu_mul(dtype, inter):
+    from mini_infer_amd import ops
+
+    gate_up = _rand(5, 2 * inter, dtype=dtype, seed=4, scale=3.0)
+    gate_up[0, 0] = 0.0
+    gate_up[0, 1 % inter] = 80.0
+    gate_up[1, 0] = -80.0
+    out = ops.silu_mul(gate_up).float().cpu().numpy()
+    g = gate_up[:, :inter].double().cpu().numpy()
+    u = gate_up[:, inter:].double().cpu().numpy()
+    expected = pl.silu(g) * u
+    assert np.isfinite(out).all()
+    assert np.abs(out - expected).max() < _tol(dtype, max(1.0, np.abs(expected).max()))
+    assert out[0, 0] == 0.0
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (7, 130, 90), (65, 301, 259), (300, 96, 4096), (33, 1, 5)])
+def test_gemm_f32_is_true_float32(m, n, k):
+    from mini_infer_amd import ops
+
+    a, w = _rand(m, k, seed=5), _rand(n, k, seed=6)
+    out = ops.gemm_f32(a, w)
+    expected = a.double() @ w.double().T
+    # float32 rounding of a K-long sum; a reduced-precision matrix mode (10-bit or
+    # 7-bit mantissas) would miss this bound by a factor of ten or more
+    assert (out.double() - expected).abs().max() < 6e-8 * math.sqrt(k) * float(expected.abs().max()) * 4
+    # a row's result does not depend on the other rows in the batch
+    alone = ops.gemm_f32(a[m // 2 : m // 2 + 1].contiguous(), w)
+    assert torch.equal(alone[0], out[m // 2])
+    # strided rows
+    wide = _rand(m, k + 3, seed=7)
+    assert torch.equal(ops.gemm_f32(wide[:, :k], w), ops.gemm_f32(wide[:, :k].contiguous(), w))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize(
+    "q_heads,kv_heads,head_dim,rotary_dim,interleaved",
+    [(32, 8, 128, 128, False), (3, 1, 32, 32, False), (6, 3, 48, 16, False), (4, 2, 64, 64, True), (2, 2, 16, 0, False)],
+)
+def test_rope_kv_write(dtype, q_heads, kv_heads, head_dim, rotary_dim, interleaved):
+    from mini_infer_amd import ops
+
+    tokens, page_size, num_pages = 9, 4, 11
+    width = (q_heads + 2 * kv_heads) * head_dim
+    qkv = _rand(tokens, width, dtype=dtype, seed=8)
+    original = qkv.clone()
+    positions = torch.tensor([0, 1, 2, 3, 700, 701, 5, 6, 131071], dtype=torch.int32, device=DEV)
+    half = rotary_dim // 2
+    if half:
+        inv_freq = torch.from_numpy(pl.inv_freq_default(rotary_dim, 500000.0)).to(DEV)
+        cos, sin = ops.rope_table(positions, inv_freq)
+        angle = positions.float().cpu().numpy()[:, None] * inv_freq.cpu().numpy()[None, :]
+        assert np.abs(cos.cpu().numpy() - np.cos(angle.astype(np.float64))).max() < 2e-6
+        assert np.abs(sin.cpu().numpy() - np.sin(angle.astype(np.float64))).max() < 2e-6
+    else:
+        cos = sin = torch.empty((tokens, 0), dtype=torch.float32, device=DEV)
+    # scattered slots, one token not written at all
+    slots = torch.tensor([40, 3, 17, 16, 0, 43, -1, 9, 22], dtype=torch.int32, device=DEV)
+    k_pages = torch.zeros((num_pages, kv_heads, page_size, head_dim), dtype=dtype, device=DEV)
+    v_pages = torch.zeros_like(k_pages)
+    ops.rope_kv_write(qkv, cos, sin, slots, k_pages, v_pages, q_heads=q_heads, kv_heads=kv_heads,
+                      head_dim=head_dim, rotary_dim=rotary_dim, interleaved=interleaved)
+
+    def rotate(x):  # x [T, heads, D] float64
+        if not half:
+            return x
+        c, s = cos.double().cpu().numpy()[:, None, :], sin.double().cpu().numpy()[:, None, :]
+        out = x.copy()
+        if interleaved:
+            x0, x1 = x[..., 0:rotary_dim:2], x[..., 1:rotary_dim:2]
+            out[..., 0:rotary_dim:2], out[..., 1:rotary_dim:2] = x0 * c - x1 * s, x1 * c + x0 * s
+        else:
+            x0, x1 = x[..., :half], x[..., half:rotary_dim]
+            out[..., :half], out[..., half:rotary_dim] = x0 * c - x1 * s, x1 * c + x0 * s
+        return out
+
+    src = original.double().cpu().numpy()
+    q_in = src[:, : q_heads * head_dim].reshape(tokens, q_heads, head_dim)
+    k_in = src[:, q_heads * head_dim : (q_heads + kv_heads) * head_dim].reshape(tokens, kv_heads, head_dim)
+    v_in = src[:, (q_heads + kv_heads) * head_dim :].reshape(tokens, kv_heads, head_dim)
+    got_q = qkv[:, : q_heads * head_dim].double().cpu().numpy().reshape(tokens, q_heads, head_dim)
+    assert np.abs(got_q - rotate(q_in)).max() < _tol(dtype, 4)
+    assert torch.equal(qkv[:, q_heads * head_dim :], original[:, q_heads * head_dim :])  # k, v inputs untouched
+    expect_k = np.zeros(k_pages.shape)
+    expect_v = np.zeros(v_pages.shape)
+    rk = rotate(k_in)
+    for t, slot in enumerate(slots.tolist()):
+        if slot >= 0:
+            expect_k[slot // page_size, :, slot % page_size] = rk[t]
+            expect_v[slot // page_size, :, slot % page_size] = v_in[t]
+    assert np.abs(k_pages.double().cpu().numpy() - expect_k).max() < _tol(dtype, 4)
+    assert np.array_equal(v_pages.double().cpu().numpy(), expect_v)  # values copied bit for bit, other slots still zero
+    if half:
+        # position 0 leaves q as it was
+        assert torch.equal(qkv[0, : q_heads * head_dim], original[0, : q_heads * head_dim])
+
+
+def _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=0):
+    """Random keys/values scattered over shuffled pages; queries are the last q_len positions."""
+    rng = np.random.default_rng(seed)
+    num_requests = len(lengths)
+    pages_per = [-(-n // page_size) for n in lengths]
+    num_pages = sum(pages_per) + 3
+    order = rng.permutation(num_pages)
+    max_blocks = max(pages_per)
+    table = np.full((num_requests, max_blocks), -1, dtype=np.int32)
+    k_pages = torch.zeros((num_pages, kv_heads, page_size, head_dim), dtype=dtype)
+    v_pages = torch.zeros_like(k_pages)
+    ks, vs, qs, token_request, positions = [], [], [], [], []
+    at = 0
+    for b, n in enumerate(lengths):
+        table[b, : pages_per[b]] = order[at : at + pages_per[b]]
+        at += pages_per[b]
+        k = torch.from_numpy(rng.standard_normal((n, kv_heads, head_dim))).to(dtype)
+        v = torch.from_numpy(rng.standard_normal((n, kv_heads, head_dim))).to(dtype)
+        for p in range(n):
+            k_pages[table[b, p // page_size], :, p % page_size] = k[p]
+            v_pages[table[b, p // page_size], :, p % page_size] = v[p]
+        q = torch.from_numpy(rng.standard_normal((q_lens[b], q_heads, head_dim))).to(dtype)
+        ks.append(k), vs.append(v), qs.append(q)
+        token_request += [b] * q_lens[b]
+        positions += list(range(n - q_lens[b], n))
+    return dict(
+        q=torch.cat(qs).reshape(-1, q_heads * head_dim).to(DEV), qs=qs, ks=ks, vs=vs,
+        k_pages=k_pages.to(DEV), v_pages=v_pages.to(DEV),
+        block_table=torch.from_numpy(table).to(DEV),
+        token_request=torch.tensor(token_request, dtype=torch.int32, device=DEV),
+        positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
+    )
+
+
+def _attention_expected(case, scale, window):
+    outs = []
+    for q, k, v in zip(case["qs"], case["ks"], case["vs"]):
+        out = pl.causal_attention(q.double().numpy(), k.double().numpy(), v.double().numpy(), scale, window)
+        outs.append(out.reshape(out.shape[0], -1))
+    return np.concatenate(outs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize(
+    "q_heads,kv_heads,head_dim,page_size,window",
+    [
+        (32, 8, 128, 16, None),
+        (5, 5, 64, 1, None),
+        (7, 1, 16, 4, None),
+        (6, 2, 48, 8, 9),
+        (10, 2, 80, 64, None),
+        (4, 4, 256, 16, 40),
+        (12, 2, 112, 32, None),
+    ],
+)
+def test_paged_attention_mixed_batch(dtype, q_heads, kv_heads, head_dim, page_size, window):
+    """Portions of prompts beside single tokens, pages in shuffled order, GQA groups of 1 to 7."""
+    from mini_infer_amd import ops
+
+    lengths, q_lens = [70, 1, 33, 129, 64], [70, 1, 5, 1, 2]
+    case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=head_dim)
+    scale = 1.0 / math.sqrt(head_dim)
+    out = ops.paged_attention(
+        case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"],
+        case["positions"], q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale,
+        window=window, max_seq_len=max(lengths))
+    expected = _attention_expected(case, scale, window)
+    assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_long_decode_splits_keys(dtype):
+    """Few tokens over long contexts: the key range is split and recombined."""
+    from mini_infer_amd import ops
+
+    q_heads, kv_heads, head_dim, page_size = 8, 2, 128, 16
+    lengths, q_lens = [3000, 517, 1], [1, 1, 1]
+    assert ops.attention_splits(3, q_heads, kv_heads, max(lengths)) > 1
+    case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=1)
+    scale = 0.2
+    out = ops.paged_attention(
+        case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"],
+        case["positions"], q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale,
+        window=None, max_seq_len=max(lengths))
+    expected = _attention_expected(case, scale, None)
+    assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_finds_one_far_key_and_respects_edges(dtype):
+    """One key among a thousand is made to stand out; the output must be its value.
+    Placed at a page's first and last slot, at the causal edge and at the window's edge."""
+    from mini_infer_amd import ops
+
+    q_heads = kv_heads = 1
+    head_dim, page_size, length = 64, 16, 1000
+    for window, spots in ((None, [0, 15, 16, 511, 512, 999]), (100, [900, 901, 911, 912, 999])):
+        for spot in spots:
+            case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, [length], [1], seed=spot)
+            q = case["qs"][0][0, 0].float()
+            page = case["block_table"][0, spot // page_size].item()
+            case["k_pages"][page, 0, spot % page_size] = (q * 4.0).to(dtype).to(DEV)  # score >> all others
+            case["ks"][0][spot, 0] = (q * 4.0).to(dtype)
+            out = ops.paged_attention(
+                case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"],
+                case["positions"], q_heads=1, kv_heads=1, head_dim=head_dim, scale=1.0, window=window,
+                max_seq_len=length)
+            value = case["vs"][0][spot, 0].float()
+            assert (out[0].float().cpu() - value).abs().max() < 2e-2, (window, spot)
+    # a key just outside the window must not be seen
+    case = _paged_case(dtype, 1, 1, head_dim, page_size, [length], [1], seed=5)
+    q = case["qs"][0][0, 0].float()
+    spot = length - 100 - 1
+    page = case["block_table"][0, spot // page_size].item()
+    case["k_pages"][page, 0, spot % page_size] = (q * 4.0).to(dtype).to(DEV)
+    out = ops.paged_attention(
+        case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"],
+        case["positions"], q_heads=1, kv_heads=1, head_dim=head_dim, scale=1.0, window=100, max_seq_len=length)
+    expected = _attention_expected(case, 1.0, 100)  # `ks` was not changed: the plain model never sees that key
+    assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
+
+
+def test_kernels_refuse_what_they_do_not_take():
+    from mini_infer_amd import ops
+    from mini_infer_amd.exceptions import KernelShapeError
+
+    case = _paged_case(torch.float32, 4, 2, 24, 4, [5], [1])
+    with pytest.raises(KernelShapeError, match="multiple of 16"):
+        ops.paged_attention(case["q"], case["k_pages"], case["v_pages"], case["block_table"],
+                            case["token_request"], case["positions"], q_heads=4, kv_heads=2, head_dim=24,
+                            scale=1.0, window=None, max_seq_len=5)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.silu_mul(torch.zeros(2, 8))
+    with pytest.raises(KernelShapeError):
+        ops.add_rmsnorm(None, torch.zeros(2, 8, device=DEV), torch.ones(9, device=DEV), 1e-5)
+    with pytest.raises(KernelShapeError):
+        ops.gemm_f32(torch.zeros(2, 8, device=DEV), torch.zeros(3, 9, device=DEV))
