@@ -15,7 +15,9 @@ Life of a request:
                    the pages no future query can see
   free_request     every page and the state slot go back; ids are reused at once
 
-Storage layout per group: [calls, 2 (k, v), num_pages, kv_heads, page_size, head_dim].
+Storage layout per group: [calls, 2 (k, v), num_pages, kv_heads, page_size * head_dim];
+a key chunk is [page_size][head_dim]; a value chunk is the same, or transposed
+([head_dim][page_size]) where the matrix-core attention kernel will read it.
 """
 
 from __future__ import annotations
@@ -29,6 +31,7 @@ import torch
 from mini_infer_amd.cache.page_pool import PagePool
 from mini_infer_amd.cache.state_slots import StateSlots
 from mini_infer_amd.exceptions import OutOfMemoryError
+from mini_infer_amd.ops.kernels import mfma_attention_supported
 from mini_infer_amd.parts.base import CacheNeeds, LayerCache, StateNeeds
 
 RELEASED = -1  # block-table entry of a page a window has passed
@@ -43,6 +46,7 @@ class PageGroup:
     window: int | None
     pool: PagePool
     storage: torch.Tensor | None = None
+    v_transposed: bool = False  # values stored [head_dim][slot] inside a page (matrix-core attention)
     tables: dict[Hashable, list[int]] = dataclasses.field(default_factory=dict)
 
     def first_live_page(self, length: int, page_size: int) -> int:
@@ -111,10 +115,11 @@ class CacheManager:
                 self._group_of_call[call] = group.index
             if need.state is not None:
                 state_needs[call] = need.state
-        if allocate_storage:
-            for group in self.groups:
+        for group in self.groups:
+            group.v_transposed = mfma_attention_supported(dtype, group.head_dim, page_size)
+            if allocate_storage:
                 group.storage = torch.zeros(
-                    (len(group.calls), 2, num_pages, group.num_kv_heads, page_size, group.head_dim),
+                    (len(group.calls), 2, num_pages, group.num_kv_heads, page_size * group.head_dim),
                     dtype=dtype,
                     device=self.device,
                 )
@@ -278,9 +283,14 @@ class CacheManager:
         for group in self.groups:
             for i, call in enumerate(group.calls):
                 caches[call].group = group.index
+                caches[call].v_transposed = group.v_transposed
                 if group.storage is not None:
-                    caches[call].k_pages = group.storage[i, 0]
-                    caches[call].v_pages = group.storage[i, 1]
+                    pages, heads = self.num_pages, group.num_kv_heads
+                    caches[call].k_pages = group.storage[i, 0].view(pages, heads, self.page_size, group.head_dim)
+                    if group.v_transposed:
+                        caches[call].v_pages = group.storage[i, 1].view(pages, heads, group.head_dim, self.page_size)
+                    else:
+                        caches[call].v_pages = group.storage[i, 1].view(pages, heads, self.page_size, group.head_dim)
         for call, tensor in self.states.tensors.items():
             caches[call].state = tensor
         return caches

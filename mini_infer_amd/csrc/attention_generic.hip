@@ -242,3 +242,17 @@ extern "C" int mi_attn_generic(int dtype, const void* q, int64_t q_row_stride, c
                                      num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
                                      num_splits, stream);
 }
+
+// The combining step alone, for partials written by the matrix-core kernel.
+extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, void* out,
+                                   int64_t out_row_stride, int num_tokens, int q_heads,
+                                   int head_dim, int num_splits, hipStream_t stream) {
+  if (num_tokens == 0) return MI_OK;
+  MI_REQUIRE(q_heads <= 65535, "attn_reduce: too many heads");
+  dim3 rgrid(num_tokens, q_heads);
+  attn_reduce_kernel<bf16_t><<<rgrid, MI_WAVE, 0, stream>>>(part_acc, part_ml, (bf16_t*)out,
+                                                            out_row_stride, q_heads, head_dim,
+                                                            num_splits);
+  MI_CHECK_LAUNCH("attn_reduce");
+  return MI_OK;
+}

@@ -1,0 +1,311 @@
+// Paged causal attention on the matrix cores (bfloat16 in, float32 accumulate), for
+// prefill portions and decode tokens alike.  gfx950 MFMA 16x16x32.
+//
+// Rows of work are (query token, query head of one key/value group) pairs, so the
+// heads that share a key/value head share its loads.  A wave owns 16 such rows and
+// walks the keys 32 at a time, computing the TRANSPOSED score block
+//     S^T[key, row] = K[key, :] . Q[row, :]
+// with K as the A operand (each lane reads 16 contiguous bytes of a key row straight
+// from the cache page) and Q^T as the B operand (kept in registers).  The MFMA
+// result leaves every lane with 8 scores of ONE row (lane % 16), so the online
+// softmax needs two cross-lane steps, and the probabilities are already laid out
+// as the B operand of the second product
+//     O^T[dim, row] += V^T[dim, key] . P^T[key, row]
+// whose A operand wants, per lane, consecutive keys of one dim: the cache stores
+// values transposed inside each page ([page][head][dim][slot]) to make that a
+// contiguous load.  No LDS is used; waves of a block read the same keys and meet in
+// the cache hierarchy.
+//
+// A block is `WAVES` waves = 16*WAVES rows = one tile of consecutive tokens of one
+// request, times `heads_per_block` heads of one key/value group.  Keys of a tile
+// may be cut into `num_splits` ranges across blocks; the partial (max, sum,
+// accumulator) triples are combined by attn_reduce_kernel (attention_generic.hip).
+//
+// Semantics as in the reference's oracle (cache/packed_attention.py:296-338):
+// row at absolute position p sees keys 0..p, or p-window+1..p with a window.
+// Requires head_dim % 32 == 0 and page_size % 16 == 0; other sizes use the plain kernel.
+#include "common.h"
+
+#include <math.h>
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+#define LOG2E 1.4426950408889634f
+#define LN2 0.6931471805599453f
+
+template <int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void attn_mfma_kernel(
+    const bf16_t* __restrict__ q, int64_t q_row_stride, const bf16_t* __restrict__ k_pages,
+    const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ cu_seqlens_q, const int* __restrict__ positions, int num_requests,
+    bf16_t* __restrict__ out, int64_t out_row_stride, float* __restrict__ part_acc,
+    float* __restrict__ part_ml, int q_heads, int kv_heads, int page_size, float scale_log2,
+    int window, int num_splits, int heads_per_block, int tokens_per_tile) {
+  constexpr int KSTEPS = D / 32;  // MFMA k-steps over the head dim for S^T
+  constexpr int DBLOCKS = D / 16;  // 16-dim blocks of the output
+
+  // ---- which tile of which request ----------------------------------------
+  int req = -1, t0 = 0, n_tok = 0;
+  {
+    int tiles_before = 0;
+    for (int b = 0; b < num_requests; ++b) {
+      const int q_len = cu_seqlens_q[b + 1] - cu_seqlens_q[b];
+      const int n_tiles = (q_len + tokens_per_tile - 1) / tokens_per_tile;
+      if ((int)blockIdx.x < tiles_before + n_tiles) {
+        const int ti = blockIdx.x - tiles_before;
+        req = b;
+        t0 = cu_seqlens_q[b] + ti * tokens_per_tile;
+        n_tok = min(tokens_per_tile, q_len - ti * tokens_per_tile);
+        break;
+      }
+      tiles_before += n_tiles;
+    }
+  }
+  if (req < 0) return;
+
+  const int group = q_heads / kv_heads;
+  const int head_blocks = (group + heads_per_block - 1) / heads_per_block;
+  const int kvh = blockIdx.y / head_blocks;
+  const int g0 = (blockIdx.y % head_blocks) * heads_per_block;
+  const int n_heads = min(heads_per_block, group - g0);
+  const int split = blockIdx.z;
+
+  const int wave = threadIdx.x / MI_WAVE;
+  const int lane = threadIdx.x % MI_WAVE;
+  const int col = lane % 16;  // this lane's row of work (a column of S^T and O^T)
+  const int quad = lane / 16;  // 0..3
+
+  // a wave whose 16 rows are all padding has nothing to do
+  if (wave * 16 >= n_tok * heads_per_block) return;
+
+  const int row = wave * 16 + col;
+  int tok_in_tile = row / heads_per_block;
+  int head_in_block = row % heads_per_block;
+  const bool row_valid = tok_in_tile < n_tok && head_in_block < n_heads;
+  tok_in_tile = min(tok_in_tile, n_tok - 1);  // padded rows repeat a real row and store nothing
+  head_in_block = min(head_in_block, n_heads - 1);
+  const int token = t0 + tok_in_tile;
+  const int head = kvh * group + g0 + head_in_block;
+  const int pos0 = positions[t0];  // tokens of a tile sit at consecutive positions
+  const int pos = pos0 + tok_in_tile;
+  const int lo_row = (window > 0) ? max(0, pos - window + 1) : 0;
+
+  // ---- key range of this block ------------------------------------------------
+  const int tile_lo = (window > 0) ? max(0, pos0 - window + 1) : 0;
+  const int tile_hi = pos0 + n_tok;  // exclusive
+  int chunk = (tile_hi - tile_lo + num_splits - 1) / num_splits;
+  chunk = (chunk + 31) / 32 * 32;
+  const int k_begin = tile_lo + split * chunk;
+  const int k_end = min(k_begin + chunk, tile_hi);
+  const int* bt = block_table + (int64_t)req * max_blocks;
+
+  // ---- Q^T operand: this lane's row, 8 consecutive dims per k-step --------------
+  bf16x8_t q_reg[KSTEPS];
+  {
+    const bf16_t* q_row = q + (int64_t)token * q_row_stride + (int64_t)head * D + quad * 8;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) q_reg[s] = *reinterpret_cast<const bf16x8_t*>(q_row + s * 32);
+  }
+
+  f32x4_t o_acc[DBLOCKS];
+#pragma unroll
+  for (int db = 0; db < DBLOCKS; ++db) o_acc[db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY;  // running maximum of this lane's row, in log2 units
+  float l_run = 0.f;  // running sum of exp2(score - m_run)
+
+  for (int kb = (k_begin / 32) * 32; kb < k_end; kb += 32) {
+    // the (page, head) chunk and first slot of the two 16-key halves (a half never
+    // straddles a page); K rows of a chunk are [slot][D], V^T rows are [D][slot]
+    int64_t chunk_off[2];
+    int slot0[2];
+#pragma unroll
+    for (int hlf = 0; hlf < 2; ++hlf) {
+      const int key0 = kb + 16 * hlf;
+      const int idx = key0 / page_size;
+      int page = (idx < max_blocks) ? bt[idx] : 0;
+      page = max(page, 0);  // released or unallocated: every key of it is masked below
+      chunk_off[hlf] = ((int64_t)page * kv_heads + kvh) * page_size * D;
+      slot0[hlf] = key0 % page_size;
+    }
+
+    // ---- S^T = K . Q^T for 32 keys ------------------------------------------------
+    f32x4_t s_acc[2];
+#pragma unroll
+    for (int hlf = 0; hlf < 2; ++hlf) {
+      const bf16_t* k_row = k_pages + chunk_off[hlf] + (int64_t)(slot0[hlf] + col) * D + quad * 8;
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        const bf16x8_t k_reg = *reinterpret_cast<const bf16x8_t*>(k_row + s * 32);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_reg, q_reg[s], acc, 0, 0, 0);
+      }
+      s_acc[hlf] = acc;
+    }
+
+    // ---- scale, mask, online softmax (lane holds keys kb + 16*hlf + 4*quad + r) -----
+    float sc[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int hlf = 0; hlf < 2; ++hlf) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = kb + 16 * hlf + 4 * quad + r;
+        const bool visible = key >= lo_row && key <= pos && key >= k_begin && key < k_end;
+        const float v = visible ? s_acc[hlf][r] * scale_log2 : -INFINITY;
+        sc[hlf * 4 + r] = v;
+        mx = fmaxf(mx, v);
+      }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, MI_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, MI_WAVE));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen nothing yet
+    const float alpha = exp2f(m_run - m_safe);  // exp2(-inf) = 0 on the first visible block
+    float sum = 0.f;
+    bf16x8_t p_reg;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float p = exp2f(sc[i] - m_safe);
+      sum += p;
+      p_reg[i] = (bf16_t)p;
+    }
+    sum += __shfl_xor(sum, 16, MI_WAVE);
+    sum += __shfl_xor(sum, 32, MI_WAVE);
+    l_run = l_run * alpha + sum;
+    m_run = m_new;
+
+    // ---- O^T = O^T * alpha + V^T . P^T ------------------------------------------------
+    const int64_t v_chunk0 = chunk_off[0], v_chunk1 = chunk_off[1];
+    const int v_slot0 = slot0[0] + 4 * quad, v_slot1 = slot0[1] + 4 * quad;
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) {
+      const int dim = db * 16 + col;
+      const bf16x4_t v0 =
+          *reinterpret_cast<const bf16x4_t*>(vt_pages + v_chunk0 + (int64_t)dim * page_size + v_slot0);
+      const bf16x4_t v1 =
+          *reinterpret_cast<const bf16x4_t*>(vt_pages + v_chunk1 + (int64_t)dim * page_size + v_slot1);
+      bf16x8_t v_reg;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v_reg[i] = v0[i];
+        v_reg[4 + i] = v1[i];
+      }
+      f32x4_t acc = o_acc[db];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[r] *= alpha;
+      o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_reg, p_reg, acc, 0, 0, 0);
+    }
+  }
+
+  // ---- write: lane holds O^T[dim = 16*db + 4*quad + r][its row] ------------------------
+  if (!row_valid) return;
+  if (num_splits == 1) {
+    const float inv = 1.f / l_run;
+    bf16_t* o = out + (int64_t)token * out_row_stride + (int64_t)head * D + quad * 4;
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) {
+      bf16x4_t packed;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) packed[r] = (bf16_t)(o_acc[db][r] * inv);
+      *reinterpret_cast<bf16x4_t*>(o + db * 16) = packed;
+    }
+  } else {
+    const int64_t slot = ((int64_t)token * q_heads + head) * num_splits + split;
+    float* pa = part_acc + slot * D + quad * 4;
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) {
+      *reinterpret_cast<f32x4_t*>(pa + db * 16) = o_acc[db];
+    }
+    if (quad == 0) {
+      part_ml[slot * 2] = m_run * LN2;  // natural-log units, as the combining kernel expects
+      part_ml[slot * 2 + 1] = l_run;
+    }
+  }
+}
+
+extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, void* out,
+                                   int64_t out_row_stride, int num_tokens, int q_heads,
+                                   int head_dim, int num_splits, hipStream_t stream);
+
+static int heads_per_block_for(int group, int rows) { return group < rows ? group : rows; }
+
+// Tiling the Python side needs to size the grid: tokens per tile for a group size.
+extern "C" int mi_attn_mfma_tokens_per_tile(int q_heads, int kv_heads, int decode_only) {
+  if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return 0;
+  const int rows = decode_only ? 16 : 64;
+  const int hb = heads_per_block_for(q_heads / kv_heads, rows);
+  const int t = rows / hb;
+  return t < 1 ? 1 : t;
+}
+
+extern "C" int mi_attn_mfma_supported(int head_dim, int page_size) {
+  const bool d_ok = head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128 ||
+                    head_dim == 192 || head_dim == 256;
+  return (d_ok && page_size > 0 && page_size % 16 == 0) ? 1 : 0;
+}
+
+// `num_tiles` = sum over requests of ceil(q_len / tokens_per_tile), computed by the
+// caller from the host copy of cu_seqlens_q (a larger number is harmless).
+// With num_splits > 1, part_acc holds num_tokens*q_heads*num_splits*head_dim floats
+// and part_ml num_tokens*q_heads*num_splits*2.
+extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_pages,
+                            const void* vt_pages, const int* block_table, int max_blocks,
+                            const int* cu_seqlens_q, const int* positions, int num_requests,
+                            int num_tokens, int num_tiles, void* out, int64_t out_row_stride,
+                            float* part_acc, float* part_ml, int q_heads, int kv_heads,
+                            int head_dim, int page_size, int num_pages, float scale, int window,
+                            int num_splits, int decode_only, hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && num_requests >= 0 && num_tiles >= 0,
+             "attn_mfma: bad sizes tokens=%d requests=%d tiles=%d", num_tokens, num_requests, num_tiles);
+  MI_REQUIRE(q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
+             "attn_mfma: q_heads=%d is not a multiple of kv_heads=%d", q_heads, kv_heads);
+  MI_REQUIRE(mi_attn_mfma_supported(head_dim, page_size),
+             "attn_mfma: head_dim=%d (32, 64, 96, 128, 192 or 256) or page_size=%d (multiple of 16) not taken",
+             head_dim, page_size);
+  MI_REQUIRE(num_pages > 0 && max_blocks > 0, "attn_mfma: bad page counts num_pages=%d max_blocks=%d",
+             num_pages, max_blocks);
+  MI_REQUIRE(window >= 0, "attn_mfma: window=%d must be 0 (none) or positive", window);
+  MI_REQUIRE(num_splits >= 1 && num_splits <= 65535, "attn_mfma: num_splits=%d out of range", num_splits);
+  MI_REQUIRE(num_splits == 1 || (part_acc && part_ml), "attn_mfma: split keys need partial buffers");
+  MI_REQUIRE(q_row_stride >= (int64_t)q_heads * head_dim && out_row_stride >= (int64_t)q_heads * head_dim,
+             "attn_mfma: row strides shorter than q_heads*head_dim");
+  MI_REQUIRE(q_row_stride % 8 == 0 && out_row_stride % 4 == 0,
+             "attn_mfma: row strides must keep 16-byte (q) and 8-byte (out) alignment");
+  if (num_tokens == 0 || num_tiles == 0) return MI_OK;
+
+  const int group = q_heads / kv_heads;
+  const int rows = decode_only ? 16 : 64;
+  const int hb = heads_per_block_for(group, rows);
+  const int tq = mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, decode_only);
+  const int head_blocks = ceil_div(group, hb);
+  MI_REQUIRE(kv_heads * head_blocks <= 65535, "attn_mfma: too many heads");
+  dim3 grid(num_tiles, kv_heads * head_blocks, num_splits);
+  const float scale_log2 = scale * LOG2E;
+
+#define MI_LAUNCH(DD, WW)                                                                         \
+  attn_mfma_kernel<DD, WW><<<grid, 64 * WW, 0, stream>>>(                                         \
+      (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)vt_pages,            \
+      block_table, max_blocks, cu_seqlens_q, positions, num_requests, (bf16_t*)out,               \
+      out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, scale_log2, window,        \
+      num_splits, hb, tq)
+#define MI_LAUNCH_D(DD)            \
+  if (decode_only) MI_LAUNCH(DD, 1); \
+  else MI_LAUNCH(DD, 4)
+  switch (head_dim) {
+    case 32: MI_LAUNCH_D(32); break;
+    case 64: MI_LAUNCH_D(64); break;
+    case 96: MI_LAUNCH_D(96); break;
+    case 128: MI_LAUNCH_D(128); break;
+    case 192: MI_LAUNCH_D(192); break;
+    default: MI_LAUNCH_D(256); break;
+  }
+#undef MI_LAUNCH_D
+#undef MI_LAUNCH
+  MI_CHECK_LAUNCH("attn_mfma");
+  if (num_splits > 1)
+    return mi_attn_reduce_bf16(part_acc, part_ml, out, out_row_stride, num_tokens, q_heads,
+                               head_dim, num_splits, stream);
+  return MI_OK;
+}

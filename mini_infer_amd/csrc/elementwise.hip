@@ -207,7 +207,8 @@ extern "C" int mi_rope_table(const int* positions, const float* inv_freq, float*
 //   pairing: half rotation pairs dim j with j + rotary_dim/2; interleaved pairs
 //   2j with 2j+1.  Dims at and beyond rotary_dim pass through.
 //   pages: [num_pages, kv_heads, page_size, head_dim]; slot = page*page_size + offset;
-//   a negative slot writes nothing.
+//   a negative slot writes nothing.  With v_transposed, values are stored
+//   [num_pages, kv_heads, head_dim, page_size] (what the matrix-core attention reads).
 // ---------------------------------------------------------------------------
 
 template <typename T>
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     T* __restrict__ qkv, int64_t row_stride, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const int* __restrict__ slot_mapping, T* __restrict__ k_pages,
     T* __restrict__ v_pages, int q_heads, int kv_heads, int head_dim, int rotary_dim,
-    int interleaved, int page_size) {
+    int interleaved, int page_size, int v_transposed) {
   const int t = blockIdx.x;
   const int half = rotary_dim / 2;
   T* row = qkv + (int64_t)t * row_stride;
@@ -256,7 +257,9 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   }
   for (int e = threadIdx.x; e < kv_heads * head_dim; e += blockDim.x) {
     const int h = e / head_dim, d = e % head_dim;
-    v_pages[(((int64_t)page * kv_heads + h) * page_size + off) * head_dim + d] = v_row[h * head_dim + d];
+    const int64_t chunk = ((int64_t)page * kv_heads + h) * page_size * head_dim;
+    const int64_t at = v_transposed ? chunk + (int64_t)d * page_size + off : chunk + (int64_t)off * head_dim + d;
+    v_pages[at] = v_row[h * head_dim + d];
   }
 }
 
@@ -264,7 +267,7 @@ extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const 
                                 const float* sin_t, const int* slot_mapping, void* k_pages,
                                 void* v_pages, int num_tokens, int q_heads, int kv_heads,
                                 int head_dim, int rotary_dim, int interleaved, int page_size,
-                                int num_pages, hipStream_t stream) {
+                                int num_pages, int v_transposed, hipStream_t stream) {
   MI_REQUIRE(num_tokens >= 0 && q_heads >= 0 && kv_heads >= 0 && head_dim > 0,
              "rope_kv_write: bad sizes tokens=%d q_heads=%d kv_heads=%d head_dim=%d", num_tokens,
              q_heads, kv_heads, head_dim);
@@ -279,11 +282,11 @@ extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const 
   if (dtype == MI_F32) {
     rope_kv_write_kernel<float><<<num_tokens, 256, 0, stream>>>(
         (float*)qkv, row_stride, cos_t, sin_t, slot_mapping, (float*)k_pages, (float*)v_pages,
-        q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size);
+        q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size, v_transposed);
   } else {
     rope_kv_write_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, cos_t, sin_t, slot_mapping, (bf16_t*)k_pages, (bf16_t*)v_pages,
-        q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size);
+        q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size, v_transposed);
   }
   MI_CHECK_LAUNCH("rope_kv_write");
   return MI_OK;

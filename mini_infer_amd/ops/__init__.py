@@ -6,6 +6,7 @@ from mini_infer_amd.ops.kernels import (
     embed_gather,
     gemm_f32,
     linear,
+    mfma_attention_supported,
     paged_attention,
     rope_kv_write,
     rope_table,
@@ -19,6 +20,7 @@ __all__ = [
     "embed_gather",
     "gemm_f32",
     "linear",
+    "mfma_attention_supported",
     "paged_attention",
     "rope_kv_write",
     "rope_table",

@@ -44,6 +44,26 @@ def _need_int32(name: str, t: torch.Tensor | None) -> None:
         raise KernelShapeError(f"{name} must be int32, got {t.dtype}")
 
 
+def _check_v_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, v_transposed: bool) -> None:
+    pages, heads, page_size, head_dim = k_pages.shape
+    expected = (pages, heads, head_dim, page_size) if v_transposed else (pages, heads, page_size, head_dim)
+    if tuple(v_pages.shape) != expected:
+        raise KernelShapeError(
+            f"v_pages has shape {tuple(v_pages.shape)}, expected {expected} (v_transposed={v_transposed})"
+        )
+
+
+MFMA_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
+
+
+def mfma_attention_supported(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
+    """Whether the matrix-core attention kernel takes this cache shape (else the plain kernel runs).
+
+    Caches it takes store their values transposed inside each page.
+    """
+    return dtype == torch.bfloat16 and head_dim in MFMA_HEAD_DIMS and page_size % 16 == 0
+
+
 def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
@@ -143,11 +163,14 @@ def rope_kv_write(
     head_dim: int,
     rotary_dim: int,
     interleaved: bool = False,
+    v_transposed: bool = False,
 ) -> None:
     """Rotate q in place inside `qkv`; rotate k and write k, v into their page slots.
 
     `qkv` is [T, (q_heads + 2*kv_heads) * head_dim] (rows may be strided); pages are
-    [num_pages, kv_heads, page_size, head_dim].  `kv_heads=0` rotates q only.
+    [num_pages, kv_heads, page_size, head_dim], value pages
+    [num_pages, kv_heads, head_dim, page_size] with `v_transposed`.  `kv_heads=0`
+    rotates q only.
     """
     _need_cuda(qkv, cos, sin, slot_mapping, k_pages, v_pages)
     _need_contiguous("cos", cos)
@@ -178,8 +201,7 @@ def rope_kv_write(
             raise KernelShapeError(
                 f"pages must be [num_pages, {kv_heads}, page_size, {head_dim}], got {tuple(k_pages.shape)}"
             )
-        if v_pages.shape != k_pages.shape:
-            raise KernelShapeError("k_pages and v_pages differ in shape")
+        _check_v_pages(k_pages, v_pages, v_transposed)
         if slot_mapping.numel() != tokens:
             raise KernelShapeError(f"slot_mapping has {slot_mapping.numel()} entries for {tokens} tokens")
         num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
@@ -188,7 +210,7 @@ def rope_kv_write(
         lib.mi_rope_kv_write(
             _dtype_code(qkv), _ptr(qkv), qkv.stride(0), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
             _ptr(k_pages), _ptr(v_pages), tokens, q_heads, kv_heads, head_dim, rotary_dim,
-            int(interleaved), page_size, num_pages, _stream(),
+            int(interleaved), page_size, num_pages, int(v_transposed), _stream(),
         )
     )
 
@@ -240,13 +262,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return torch.matmul(x, weight.t())
 
 
-def attention_splits(num_tokens: int, q_heads: int, kv_heads: int, max_seq_len: int) -> int:
-    """How many key ranges each (token, head group) is cut into to fill the GPU."""
-    group = q_heads // kv_heads
-    work_items = max(1, num_tokens * kv_heads * math.ceil(group / 4))
-    target = 2048  # waves wanted in flight: 256 CUs x 8
-    by_fill = max(1, target // work_items)
-    by_len = max(1, max_seq_len // 256)
+def attention_splits(work_items: int, max_seq_len: int, target: int = 2048, min_keys: int = 256) -> int:
+    """How many key ranges each work item is cut into so that the GPU is full.
+
+    `work_items` blocks would run without splitting; `target` are wanted; a split
+    keeps at least `min_keys` keys.
+    """
+    by_fill = max(1, target // max(1, work_items))
+    by_len = max(1, max_seq_len // min_keys)
     return int(min(by_fill, by_len, 64))
 
 
@@ -257,6 +280,8 @@ def paged_attention(
     block_table: torch.Tensor,
     token_request: torch.Tensor,
     positions: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    host_cu_seqlens_q: list[int],
     *,
     q_heads: int,
     kv_heads: int,
@@ -264,18 +289,25 @@ def paged_attention(
     scale: float,
     window: int | None,
     max_seq_len: int,
+    v_transposed: bool = False,
+    force_plain: bool = False,
 ) -> torch.Tensor:
     """Causal attention of every token over its request's pages; returns [T, q_heads*head_dim].
 
     `q` is [T, >= q_heads*head_dim] with the rotated queries in its first columns
     (rows may be strided, so the merged projection's buffer can be passed as it is).
+    Tokens of a request are consecutive and sit at consecutive positions;
+    `cu_seqlens_q` (device) and `host_cu_seqlens_q` give the request boundaries.
+    bfloat16 caches with transposed values run on the matrix cores; everything else
+    (float32, other head or page sizes) runs the plain kernel.
     """
-    _need_cuda(q, k_pages, v_pages, block_table, token_request, positions)
+    _need_cuda(q, k_pages, v_pages, block_table, token_request, positions, cu_seqlens_q)
     for name, t in (("k_pages", k_pages), ("v_pages", v_pages), ("block_table", block_table),
-                    ("token_request", token_request), ("positions", positions)):
+                    ("token_request", token_request), ("positions", positions),
+                    ("cu_seqlens_q", cu_seqlens_q)):
         _need_contiguous(name, t)
     for name, t in (("block_table", block_table), ("token_request", token_request),
-                    ("positions", positions)):
+                    ("positions", positions), ("cu_seqlens_q", cu_seqlens_q)):
         _need_int32(name, t)
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < q_heads * head_dim:
         raise KernelShapeError(f"q must be [T, >= {q_heads * head_dim}] with unit inner stride")
@@ -285,21 +317,64 @@ def paged_attention(
         raise KernelShapeError(
             f"pages must be [num_pages, {kv_heads}, page_size, {head_dim}], got {tuple(k_pages.shape)}"
         )
-    if v_pages.shape != k_pages.shape:
-        raise KernelShapeError("k_pages and v_pages differ in shape")
+    _check_v_pages(k_pages, v_pages, v_transposed)
     tokens = q.shape[0]
     if token_request.numel() != tokens or positions.numel() != tokens:
         raise KernelShapeError("token_request and positions need one entry per token")
     if block_table.dim() != 2:
         raise KernelShapeError("block_table must be [requests, max_blocks]")
+    num_requests = block_table.shape[0]
+    if cu_seqlens_q.numel() != num_requests + 1 or len(host_cu_seqlens_q) != num_requests + 1:
+        raise KernelShapeError("cu_seqlens_q needs one more entry than there are requests")
+    if host_cu_seqlens_q[-1] != tokens:
+        raise KernelShapeError(f"cu_seqlens_q ends at {host_cu_seqlens_q[-1]}, but there are {tokens} tokens")
     num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
     out = torch.empty((tokens, q_heads * head_dim), dtype=q.dtype, device=q.device)
-    splits = attention_splits(tokens, q_heads, kv_heads, max_seq_len)
-    part_acc = part_ml = None
-    if splits > 1:
-        part_acc = torch.empty((tokens * q_heads * splits, head_dim), dtype=torch.float32, device=q.device)
-        part_ml = torch.empty((tokens * q_heads * splits, 2), dtype=torch.float32, device=q.device)
     lib = library.load()
+    group = q_heads // kv_heads
+
+    use_mfma = v_transposed and not force_plain
+    if v_transposed and not mfma_attention_supported(q.dtype, head_dim, page_size):
+        raise KernelShapeError(
+            f"transposed value pages need the matrix-core kernel, which does not take "
+            f"{q.dtype}, head_dim={head_dim}, page_size={page_size}"
+        )
+    if v_transposed and force_plain:
+        raise KernelShapeError("the plain attention kernel reads value pages that are not transposed")
+
+    def partials(splits: int) -> tuple[torch.Tensor | None, torch.Tensor | None]:
+        if splits == 1:
+            return None, None
+        return (
+            torch.empty((tokens * q_heads * splits, head_dim), dtype=torch.float32, device=q.device),
+            torch.empty((tokens * q_heads * splits, 2), dtype=torch.float32, device=q.device),
+        )
+
+    if use_mfma:
+        q_lens = [host_cu_seqlens_q[b + 1] - host_cu_seqlens_q[b] for b in range(num_requests)]
+        decode_only = max(q_lens) <= 1
+        tokens_per_tile = lib.mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, int(decode_only))
+        num_tiles = sum(-(-n // tokens_per_tile) for n in q_lens)
+        rows = 16 if decode_only else 64
+        head_blocks = -(-group // min(group, rows))
+        splits = attention_splits(
+            num_tiles * kv_heads * head_blocks, max_seq_len,
+            target=2048 if decode_only else 1024, min_keys=128,
+        )
+        part_acc, part_ml = partials(splits)
+        library.check(
+            lib.mi_attn_mfma(
+                _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+                block_table.shape[1], _ptr(cu_seqlens_q), _ptr(positions), num_requests, tokens,
+                num_tiles, _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads,
+                head_dim, page_size, num_pages, float(scale), int(window or 0), splits,
+                int(decode_only), _stream(),
+            )
+        )
+        return out
+
+    splits = attention_splits(tokens * kv_heads * math.ceil(group / 4), max_seq_len)
+    part_acc, part_ml = partials(splits)
     library.check(
         lib.mi_attn_generic(
             _dtype_code(q), _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),

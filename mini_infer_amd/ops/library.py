@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -26,7 +26,7 @@ _SIGNATURES: dict[str, list] = {
     "mi_rope_table": [_P, _P, _P, _P, c_int, c_int, _P],
     "mi_rope_kv_write": [
         c_int, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-        c_int, _P,
+        c_int, c_int, _P,
     ],
     "mi_silu_mul": [c_int, _P, _P, c_int, c_int, _P],
     "mi_gemm_f32": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
@@ -34,6 +34,12 @@ _SIGNATURES: dict[str, list] = {
         c_int, _P, c_int64, _P, _P, _P, c_int, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int,
         c_int, c_int, c_int, c_float, c_int, c_int, _P,
     ],
+    "mi_attn_mfma": [
+        _P, c_int64, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, _P, c_int64, _P, _P, c_int,
+        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P,
+    ],
+    "mi_attn_mfma_tokens_per_tile": [c_int, c_int, c_int],
+    "mi_attn_mfma_supported": [c_int, c_int],
     "mi_sample": [c_int, _P, c_int64, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P],
 }
 

@@ -88,19 +88,20 @@ class GQAttention(Mixer):
                 qkv, cos, sin, slots, cache.k_pages, cache.v_pages,
                 q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
                 rotary_dim=self.position.rotary_dim, interleaved=self.position.interleaved,
+                v_transposed=cache.v_transposed,
             )
         else:
             empty = torch.empty((ctx.num_tokens, 0), dtype=torch.float32, device=x.device)
             ops.rope_kv_write(
                 qkv, empty, empty, slots, cache.k_pages, cache.v_pages,
                 q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
-                rotary_dim=0, interleaved=False,
+                rotary_dim=0, interleaved=False, v_transposed=cache.v_transposed,
             )
         attended = ops.paged_attention(
             qkv, cache.k_pages, cache.v_pages, ctx.block_tables[cache.group], ctx.token_request,
-            ctx.positions, q_heads=self.num_heads, kv_heads=self.num_kv_heads,
-            head_dim=self.head_dim, scale=self.scale, window=self.window,
-            max_seq_len=ctx.max_seq_len,
+            ctx.positions, ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=self.num_heads,
+            kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
+            max_seq_len=ctx.max_seq_len, v_transposed=cache.v_transposed,
         )
         return self.out.forward(attended)
 

@@ -85,7 +85,8 @@ class LayerCache:
 
     group: int | None = None  # which page group's block table and write slots apply
     k_pages: torch.Tensor | None = None  # [num_pages, kv_heads, page_size, head_dim]
-    v_pages: torch.Tensor | None = None
+    v_pages: torch.Tensor | None = None  # same, or [num_pages, kv_heads, head_dim, page_size] if transposed
+    v_transposed: bool = False
     state: torch.Tensor | None = None  # [max_requests, *state shape]
 
 

@@ -131,6 +131,12 @@ def test_rope_kv_write(dtype, q_heads, kv_heads, head_dim, rotary_dim, interleav
     v_pages = torch.zeros_like(k_pages)
     ops.rope_kv_write(qkv, cos, sin, slots, k_pages, v_pages, q_heads=q_heads, kv_heads=kv_heads,
                       head_dim=head_dim, rotary_dim=rotary_dim, interleaved=interleaved)
+    # the same write with values transposed inside each page
+    vt_pages = torch.zeros((num_pages, kv_heads, head_dim, page_size), dtype=dtype, device=DEV)
+    ops.rope_kv_write(original.clone(), cos, sin, slots, torch.zeros_like(k_pages), vt_pages, q_heads=q_heads,
+                      kv_heads=kv_heads, head_dim=head_dim, rotary_dim=rotary_dim, interleaved=interleaved,
+                      v_transposed=True)
+    assert torch.equal(vt_pages.transpose(2, 3), v_pages)
 
     def rotate(x):  # x [T, heads, D] float64
         if not half:
@@ -166,7 +172,7 @@ def test_rope_kv_write(dtype, q_heads, kv_heads, head_dim, rotary_dim, interleav
         assert torch.equal(qkv[0, : q_heads * head_dim], original[0, : q_heads * head_dim])
 
 
-def _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=0):
+def _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=0, v_transposed=False):
     """Random keys/values scattered over shuffled pages; queries are the last q_len positions."""
     rng = np.random.default_rng(seed)
     num_requests = len(lengths)
@@ -191,13 +197,29 @@ def _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, 
         ks.append(k), vs.append(v), qs.append(q)
         token_request += [b] * q_lens[b]
         positions += list(range(n - q_lens[b], n))
+    cu = [0]
+    for n in q_lens:
+        cu.append(cu[-1] + n)
+    if v_transposed:
+        v_pages = v_pages.transpose(2, 3).contiguous()
     return dict(
         q=torch.cat(qs).reshape(-1, q_heads * head_dim).to(DEV), qs=qs, ks=ks, vs=vs,
-        k_pages=k_pages.to(DEV), v_pages=v_pages.to(DEV),
+        k_pages=k_pages.to(DEV), v_pages=v_pages.to(DEV), v_transposed=v_transposed,
+        cu=torch.tensor(cu, dtype=torch.int32, device=DEV), host_cu=cu,
         block_table=torch.from_numpy(table).to(DEV),
         token_request=torch.tensor(token_request, dtype=torch.int32, device=DEV),
         positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
     )
+
+
+def _attend(case, q_heads, kv_heads, head_dim, scale, window, max_seq_len):
+    from mini_infer_amd import ops
+
+    return ops.paged_attention(
+        case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"],
+        case["positions"], case["cu"], case["host_cu"], q_heads=q_heads, kv_heads=kv_heads,
+        head_dim=head_dim, scale=scale, window=window, max_seq_len=max_seq_len,
+        v_transposed=case["v_transposed"])
 
 
 def _attention_expected(case, scale, window):
@@ -208,84 +230,102 @@ def _attention_expected(case, scale, window):
     return np.concatenate(outs)
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize(
-    "q_heads,kv_heads,head_dim,page_size,window",
-    [
-        (32, 8, 128, 16, None),
-        (5, 5, 64, 1, None),
-        (7, 1, 16, 4, None),
-        (6, 2, 48, 8, 9),
-        (10, 2, 80, 64, None),
-        (4, 4, 256, 16, 40),
-        (12, 2, 112, 32, None),
-    ],
-)
-def test_paged_attention_mixed_batch(dtype, q_heads, kv_heads, head_dim, page_size, window):
-    """Portions of prompts beside single tokens, pages in shuffled order, GQA groups of 1 to 7."""
-    from mini_infer_amd import ops
+ATTENTION_MODES = [("plain", torch.float32), ("plain", torch.bfloat16), ("mfma", torch.bfloat16)]
+PLAIN_SHAPES = [
+    (32, 8, 128, 16, None),
+    (5, 5, 64, 1, None),
+    (7, 1, 16, 4, None),
+    (6, 2, 48, 8, 9),
+    (10, 2, 80, 64, None),
+    (4, 4, 256, 16, 40),
+    (12, 2, 112, 32, None),
+]
+MFMA_SHAPES = [
+    (32, 8, 128, 16, None),
+    (3, 1, 32, 16, None),
+    (7, 1, 64, 32, None),
+    (6, 2, 96, 16, 9),
+    (40, 2, 64, 16, None),
+    (8, 2, 256, 64, 40),
+    (12, 4, 192, 16, None),
+    (5, 5, 128, 48, 70),
+]
 
-    lengths, q_lens = [70, 1, 33, 129, 64], [70, 1, 5, 1, 2]
-    case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=head_dim)
+
+def _attention_cases():
+    for mode, dtype in ATTENTION_MODES:
+        for shape in MFMA_SHAPES if mode == "mfma" else PLAIN_SHAPES:
+            yield pytest.param(mode, dtype, *shape, id=f"{mode}-{str(dtype)[6:]}-" + "-".join(map(str, shape)))
+
+
+@pytest.mark.parametrize("mode,dtype,q_heads,kv_heads,head_dim,page_size,window", list(_attention_cases()))
+def test_paged_attention_mixed_batch(mode, dtype, q_heads, kv_heads, head_dim, page_size, window):
+    """Portions of prompts beside single tokens, pages in shuffled order, groups of 1 to 20 heads."""
+    lengths, q_lens = [70, 1, 33, 129, 64, 200], [70, 1, 5, 1, 2, 37]
+    case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=head_dim,
+                       v_transposed=mode == "mfma")
     scale = 1.0 / math.sqrt(head_dim)
-    out = ops.paged_attention(
-        case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"],
-        case["positions"], q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale,
-        window=window, max_seq_len=max(lengths))
+    out = _attend(case, q_heads, kv_heads, head_dim, scale, window, max(lengths))
     expected = _attention_expected(case, scale, window)
     assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_paged_attention_long_decode_splits_keys(dtype):
-    """Few tokens over long contexts: the key range is split and recombined."""
+@pytest.mark.parametrize("mode,dtype", ATTENTION_MODES)
+@pytest.mark.parametrize("q_heads,kv_heads,window", [(8, 2, None), (40, 2, None), (4, 4, 1000)])
+def test_paged_attention_decode_only_splits_keys(mode, dtype, q_heads, kv_heads, window):
+    """Single tokens over long contexts: the key range is split over blocks and recombined."""
     from mini_infer_amd import ops
 
-    q_heads, kv_heads, head_dim, page_size = 8, 2, 128, 16
-    lengths, q_lens = [3000, 517, 1], [1, 1, 1]
-    assert ops.attention_splits(3, q_heads, kv_heads, max(lengths)) > 1
-    case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=1)
+    head_dim, page_size = 128, 16
+    lengths, q_lens = [3000, 517, 1, 64, 2049], [1, 1, 1, 1, 1]
+    assert ops.attention_splits(5 * kv_heads, max(lengths)) > 1
+    case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=1,
+                       v_transposed=mode == "mfma")
     scale = 0.2
-    out = ops.paged_attention(
-        case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"],
-        case["positions"], q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale,
-        window=None, max_seq_len=max(lengths))
-    expected = _attention_expected(case, scale, None)
+    out = _attend(case, q_heads, kv_heads, head_dim, scale, window, max(lengths))
+    expected = _attention_expected(case, scale, window)
     assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_paged_attention_finds_one_far_key_and_respects_edges(dtype):
+@pytest.mark.parametrize("mode,dtype", ATTENTION_MODES)
+def test_paged_attention_portion_over_long_context_splits_keys(mode, dtype):
+    """A short portion late in a long prompt: few tiles, so keys are split there too."""
+    q_heads, kv_heads, head_dim, page_size = 8, 2, 64, 16
+    lengths, q_lens = [2500, 900], [40, 3]
+    case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=2,
+                       v_transposed=mode == "mfma")
+    out = _attend(case, q_heads, kv_heads, head_dim, 0.15, None, max(lengths))
+    expected = _attention_expected(case, 0.15, None)
+    assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
+
+
+@pytest.mark.parametrize("mode,dtype", ATTENTION_MODES)
+def test_paged_attention_finds_one_far_key_and_respects_edges(mode, dtype):
     """One key among a thousand is made to stand out; the output must be its value.
     Placed at a page's first and last slot, at the causal edge and at the window's edge."""
-    from mini_infer_amd import ops
-
-    q_heads = kv_heads = 1
     head_dim, page_size, length = 64, 16, 1000
-    for window, spots in ((None, [0, 15, 16, 511, 512, 999]), (100, [900, 901, 911, 912, 999])):
+    transposed = mode == "mfma"
+
+    def plant(case, spot):
+        q = case["qs"][0][0, 0].float()
+        page = case["block_table"][0, spot // page_size].item()
+        case["k_pages"][page, 0, spot % page_size] = (q * 4.0).to(dtype).to(DEV)  # score >> all others
+
+    for window, spots in ((None, [0, 15, 16, 31, 32, 511, 512, 999]), (100, [900, 901, 911, 912, 927, 928, 999])):
         for spot in spots:
-            case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, [length], [1], seed=spot)
-            q = case["qs"][0][0, 0].float()
-            page = case["block_table"][0, spot // page_size].item()
-            case["k_pages"][page, 0, spot % page_size] = (q * 4.0).to(dtype).to(DEV)  # score >> all others
-            case["ks"][0][spot, 0] = (q * 4.0).to(dtype)
-            out = ops.paged_attention(
-                case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"],
-                case["positions"], q_heads=1, kv_heads=1, head_dim=head_dim, scale=1.0, window=window,
-                max_seq_len=length)
+            case = _paged_case(dtype, 1, 1, head_dim, page_size, [length], [1], seed=spot, v_transposed=transposed)
+            plant(case, spot)
+            out = _attend(case, 1, 1, head_dim, 1.0, window, length)
             value = case["vs"][0][spot, 0].float()
             assert (out[0].float().cpu() - value).abs().max() < 2e-2, (window, spot)
-    # a key just outside the window must not be seen
-    case = _paged_case(dtype, 1, 1, head_dim, page_size, [length], [1], seed=5)
-    q = case["qs"][0][0, 0].float()
-    spot = length - 100 - 1
-    page = case["block_table"][0, spot // page_size].item()
-    case["k_pages"][page, 0, spot % page_size] = (q * 4.0).to(dtype).to(DEV)
-    out = ops.paged_attention(
-        case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"],
-        case["positions"], q_heads=1, kv_heads=1, head_dim=head_dim, scale=1.0, window=100, max_seq_len=length)
-    expected = _attention_expected(case, 1.0, 100)  # `ks` was not changed: the plain model never sees that key
-    assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
+    # a key just outside the window must not be seen, nor one after the query
+    for spot, q_len in ((length - 100 - 1, 1), (length - 1, 2)):
+        case = _paged_case(dtype, 1, 1, head_dim, page_size, [length], [q_len], seed=5, v_transposed=transposed)
+        plant(case, spot)  # `ks` is not changed: the plain model never sees that key
+        out = _attend(case, 1, 1, head_dim, 1.0, 100, length)
+        expected = _attention_expected(case, 1.0, 100)
+        rows = slice(0, 1)  # the first query (position length - q_len) must not see the planted key
+        assert np.abs(out.double().cpu().numpy() - expected)[rows].max() < _tol(dtype, 2)
 
 
 def test_kernels_refuse_what_they_do_not_take():
@@ -294,9 +334,15 @@ def test_kernels_refuse_what_they_do_not_take():
 
     case = _paged_case(torch.float32, 4, 2, 24, 4, [5], [1])
     with pytest.raises(KernelShapeError, match="multiple of 16"):
-        ops.paged_attention(case["q"], case["k_pages"], case["v_pages"], case["block_table"],
-                            case["token_request"], case["positions"], q_heads=4, kv_heads=2, head_dim=24,
-                            scale=1.0, window=None, max_seq_len=5)
+        _attend(case, 4, 2, 24, 1.0, None, 5)
+    # transposed value pages belong to the matrix-core kernel, which takes bfloat16 only
+    case = _paged_case(torch.float32, 4, 2, 32, 16, [5], [1], v_transposed=True)
+    with pytest.raises(KernelShapeError, match="matrix-core"):
+        _attend(case, 4, 2, 32, 1.0, None, 5)
+    assert ops.mfma_attention_supported(torch.bfloat16, 128, 16)
+    assert not ops.mfma_attention_supported(torch.bfloat16, 48, 16)
+    assert not ops.mfma_attention_supported(torch.bfloat16, 128, 8)
+    assert not ops.mfma_attention_supported(torch.float32, 128, 16)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         ops.silu_mul(torch.zeros(2, 8))
     with pytest.raises(KernelShapeError):
