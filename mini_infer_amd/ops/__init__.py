@@ -5,6 +5,7 @@ from mini_infer_amd.ops.kernels import (
     attention_splits,
     embed_gather,
     gemm_f32,
+    gemm_skinny_bf16,
     linear,
     mfma_attention_supported,
     paged_attention,
@@ -19,6 +20,7 @@ __all__ = [
     "attention_splits",
     "embed_gather",
     "gemm_f32",
+    "gemm_skinny_bf16",
     "linear",
     "mfma_attention_supported",
     "paged_attention",

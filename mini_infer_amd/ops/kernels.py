@@ -249,16 +249,51 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return c
 
 
+SKINNY_MAX_ROWS = 16
+
+
+def gemm_skinny_bf16(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """`a @ w.T` for at most 16 rows of bfloat16: a [M, K], w [N, K] -> [M, N], K % 32 == 0."""
+    _need_cuda(a, w)
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelShapeError(f"gemm_skinny_bf16 takes bfloat16, got {a.dtype} and {w.dtype}")
+    if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
+        raise KernelShapeError(f"gemm_skinny_bf16: shapes {tuple(a.shape)} and {tuple(w.shape)} do not fit")
+    if a.stride(1) != 1 or w.stride(1) != 1:
+        raise KernelShapeError("gemm_skinny_bf16: rows must have unit inner stride")
+    m, k = a.shape
+    n = w.shape[0]
+    c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    lib = library.load()
+    library.check(
+        lib.mi_gemm_skinny_bf16(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(c), c.stride(0), m, n, k, _stream())
+    )
+    return c
+
+
+def skinny_gemm_takes(m: int, k: int, lda: int, ldw: int) -> bool:
+    return 1 <= m <= SKINNY_MAX_ROWS and k >= 32 and k % 32 == 0 and lda % 8 == 0 and ldw % 8 == 0
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """`x @ weight.T` without bias.
 
-    float32 runs the hand-written true-float32 kernel.  bfloat16 goes to the
-    vendor GEMM library through torch, as the reference's engine does
+    float32 runs the hand-written true-float32 kernel.  bfloat16 with at most 16
+    rows (decode) runs the hand-written weight-streaming kernel; more rows go to
+    the vendor GEMM library through torch, as the reference's engine does
     (distributed/linear.py:167, `F.linear` -> the vendor BLAS).
     """
     if x.dtype == torch.float32:
         return gemm_f32(x, weight)
     _need_cuda(x, weight)
+    if (
+        x.dtype == torch.bfloat16
+        and x.dim() == 2
+        and x.stride(1) == 1
+        and weight.stride(1) == 1
+        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), weight.stride(0))
+    ):
+        return gemm_skinny_bf16(x, weight)
     return torch.matmul(x, weight.t())
 
 

@@ -103,6 +103,42 @@ def test_gemm_f32_is_true_float32(m, n, k):
     assert torch.equal(ops.gemm_f32(wide[:, :k], w), ops.gemm_f32(wide[:, :k].contiguous(), w))
 
 
+@pytest.mark.parametrize(
+    "m,n,k",
+    [(1, 4096, 4096), (8, 6144, 4096), (16, 96, 64), (7, 301, 96), (13, 130, 160), (16, 1000, 14336),
+     (5, 128256, 256), (3, 7, 32), (9, 28672, 4096), (2, 16400, 1056)],
+)
+def test_gemm_skinny_bf16(m, n, k):
+    from mini_infer_amd import ops
+
+    a, w = _rand(m, k, dtype=torch.bfloat16, seed=9), _rand(n, k, dtype=torch.bfloat16, seed=10, scale=0.05)
+    out = ops.gemm_skinny_bf16(a, w)
+    expected = a.double() @ w.double().T
+    # float32 accumulation of exact bfloat16 products, one rounding to bfloat16 at the end
+    assert (out.double() - expected).abs().max() < 2.0 ** -8 * float(expected.abs().max()) + 1e-6
+    # a row's result does not depend on the other rows in the batch
+    alone = ops.gemm_skinny_bf16(a[m // 2 : m // 2 + 1].contiguous(), w)
+    assert torch.equal(alone[0], out[m // 2])
+    # strided activations (a slice of a wider buffer), and the dispatch in `linear`
+    wide = _rand(m, k + 8, dtype=torch.bfloat16, seed=11)
+    assert torch.equal(ops.gemm_skinny_bf16(wide[:, :k], w), ops.gemm_skinny_bf16(wide[:, :k].contiguous(), w))
+    assert torch.equal(ops.linear(a, w), out)
+
+
+def test_linear_falls_back_to_the_library_where_the_skinny_kernel_does_not_apply():
+    from mini_infer_amd import ops
+    from mini_infer_amd.exceptions import KernelShapeError
+
+    a, w = _rand(5, 90, dtype=torch.bfloat16), _rand(40, 90, dtype=torch.bfloat16, seed=1)
+    assert (ops.linear(a, w).double() - a.double() @ w.double().T).abs().max() < 0.2
+    big = _rand(100, 64, dtype=torch.bfloat16)
+    assert ops.linear(big, _rand(32, 64, dtype=torch.bfloat16, seed=2)).shape == (100, 32)
+    with pytest.raises(KernelShapeError, match="m <= 16"):
+        ops.gemm_skinny_bf16(big, _rand(32, 64, dtype=torch.bfloat16, seed=2))
+    with pytest.raises(KernelShapeError):
+        ops.gemm_skinny_bf16(a, w)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize(
     "q_heads,kv_heads,head_dim,rotary_dim,interleaved",
