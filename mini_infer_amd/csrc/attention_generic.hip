@@ -153,25 +153,34 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
   }
 }
 
-// Combine the splits of one (token, head) in a fixed order.
+// Combine the splits of one (token, head): one wave; lanes first share the work of
+// reading the splits' (max, sum) pairs, then own output dims.  The order of the sums
+// is fixed, so the result does not depend on timing.
 template <typename T>
 __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict__ part_acc,
                                                          const float* __restrict__ part_ml,
                                                          T* __restrict__ out, int64_t out_row_stride,
                                                          int q_heads, int head_dim, int num_splits) {
   const int t = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x;
   const int64_t base = ((int64_t)t * q_heads + h) * num_splits;
-  float m_all = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) m_all = fmaxf(m_all, part_ml[(base + s) * 2]);
+  // num_splits <= 64: lane s holds split s
+  const float m_s = (lane < num_splits) ? part_ml[(base + lane) * 2] : -INFINITY;
+  const float l_s = (lane < num_splits) ? part_ml[(base + lane) * 2 + 1] : 0.f;
+  const float m_all = wave_max(m_s);
+  const float w_s = (lane < num_splits) ? expf(m_s - m_all) : 0.f;
   float l_all = 0.f;
-  for (int s = 0; s < num_splits; ++s)
-    l_all += part_ml[(base + s) * 2 + 1] * expf(part_ml[(base + s) * 2] - m_all);
+  for (int s = 0; s < num_splits; ++s) l_all += __shfl(l_s * w_s, s, MI_WAVE);
   const float inv = 1.f / l_all;
-  for (int d = threadIdx.x; d < head_dim; d += MI_WAVE) {
+  for (int d0 = 0; d0 < head_dim; d0 += MI_WAVE) {  // all lanes stay in the loop for the shuffles
+    const int d = d0 + lane;
+    const bool active = d < head_dim;
     float o = 0.f;
-    for (int s = 0; s < num_splits; ++s)
-      o += part_acc[(base + s) * head_dim + d] * expf(part_ml[(base + s) * 2] - m_all);
-    out[(int64_t)t * out_row_stride + (int64_t)h * head_dim + d] = from_f32<T>(o * inv);
+    for (int s = 0; s < num_splits; ++s) {
+      const float w = __shfl(w_s, s, MI_WAVE);
+      if (active) o += part_acc[(base + s) * head_dim + d] * w;
+    }
+    if (active) out[(int64_t)t * out_row_stride + (int64_t)h * head_dim + d] = from_f32<T>(o * inv);
   }
 }
 
@@ -225,7 +234,7 @@ extern "C" int mi_attn_generic(int dtype, const void* q, int64_t q_row_stride, c
   MI_REQUIRE((int64_t)num_pages * kv_heads * page_size < (int64_t)1 << 31,
              "attn_generic: the cache has too many key rows for 32-bit row indices");
   MI_REQUIRE(window >= 0, "attn_generic: window=%d must be 0 (none) or positive", window);
-  MI_REQUIRE(num_splits >= 1 && num_splits <= 65535, "attn_generic: num_splits=%d out of range", num_splits);
+  MI_REQUIRE(num_splits >= 1 && num_splits <= 64, "attn_generic: num_splits=%d must be 1..64", num_splits);
   MI_REQUIRE(num_splits == 1 || (part_acc && part_ml), "attn_generic: split keys need partial buffers");
   MI_REQUIRE(q_row_stride >= (int64_t)q_heads * head_dim && out_row_stride >= (int64_t)q_heads * head_dim,
              "attn_generic: row strides shorter than q_heads*head_dim");

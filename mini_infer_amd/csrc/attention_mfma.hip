@@ -16,10 +16,13 @@
 // contiguous load.  No LDS is used; waves of a block read the same keys and meet in
 // the cache hierarchy.
 //
-// A block is `WAVES` waves = 16*WAVES rows = one tile of consecutive tokens of one
-// request, times `heads_per_block` heads of one key/value group.  Keys of a tile
-// may be cut into `num_splits` ranges across blocks; the partial (max, sum,
-// accumulator) triples are combined by attn_reduce_kernel (attention_generic.hip).
+// A block is `WAVES` row groups = 16*WAVES rows = one tile of consecutive tokens of
+// one request, times `heads_per_block` heads of one key/value group.  For decode
+// (one row group) `KW` waves share the rows, each taking every KW-th block of keys,
+// and merge through LDS: more waves in flight per byte of partial results.  Keys of
+// a tile may also be cut into `num_splits` ranges across blocks; those partial
+// (max, sum, accumulator) triples are combined by attn_reduce_kernel
+// (attention_generic.hip).
 //
 // Semantics as in the reference's oracle (cache/packed_attention.py:296-338):
 // row at absolute position p sees keys 0..p, or p-window+1..p with a window.
@@ -35,35 +38,59 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define LOG2E 1.4426950408889634f
 #define LN2 0.6931471805599453f
 
-template <int D, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void attn_mfma_kernel(
+template <int D, int WAVES, int KW>
+__global__ __launch_bounds__(64 * WAVES * KW) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_row_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ positions, int num_requests,
     bf16_t* __restrict__ out, int64_t out_row_stride, float* __restrict__ part_acc,
     float* __restrict__ part_ml, int q_heads, int kv_heads, int page_size, float scale_log2,
-    int window, int num_splits, int heads_per_block, int tokens_per_tile) {
+    int window, int num_splits, int heads_per_block, int tokens_per_tile, int one_tile_per_request) {
   constexpr int KSTEPS = D / 32;  // MFMA k-steps over the head dim for S^T
   constexpr int DBLOCKS = D / 16;  // 16-dim blocks of the output
 
   // ---- which tile of which request ----------------------------------------
+  // Every wave finds it on its own.  With at most one tile per request (decode, short
+  // portions) the tile IS the request; otherwise the lanes share the search: each takes
+  // a request, a prefix sum over the requests' tile counts locates the tile.
   int req = -1, t0 = 0, n_tok = 0;
-  {
+  if (one_tile_per_request) {
+    if ((int)blockIdx.x < num_requests) {
+      req = blockIdx.x;
+      t0 = cu_seqlens_q[req];
+      n_tok = cu_seqlens_q[req + 1] - t0;
+    }
+  } else {
+    const int search_lane = threadIdx.x % MI_WAVE;
     int tiles_before = 0;
-    for (int b = 0; b < num_requests; ++b) {
-      const int q_len = cu_seqlens_q[b + 1] - cu_seqlens_q[b];
+    for (int b0 = 0; b0 < num_requests && req < 0; b0 += MI_WAVE) {
+      const int b = b0 + search_lane;
+      const int start = (b < num_requests) ? cu_seqlens_q[b] : 0;
+      const int q_len = (b < num_requests) ? cu_seqlens_q[b + 1] - start : 0;
       const int n_tiles = (q_len + tokens_per_tile - 1) / tokens_per_tile;
-      if ((int)blockIdx.x < tiles_before + n_tiles) {
-        const int ti = blockIdx.x - tiles_before;
-        req = b;
-        t0 = cu_seqlens_q[b] + ti * tokens_per_tile;
-        n_tok = min(tokens_per_tile, q_len - ti * tokens_per_tile);
-        break;
+      int inclusive = n_tiles;
+#pragma unroll
+      for (int off = 1; off < MI_WAVE; off <<= 1) {
+        const int up = __shfl_up(inclusive, off, MI_WAVE);
+        if (search_lane >= off) inclusive += up;
       }
-      tiles_before += n_tiles;
+      const int first = tiles_before + inclusive - n_tiles;
+      const bool mine = n_tiles > 0 && (int)blockIdx.x >= first && (int)blockIdx.x < first + n_tiles;
+      const unsigned long long owners = __ballot(mine);
+      if (owners) {
+        const int src = __ffsll((long long)owners) - 1;
+        const int ti = blockIdx.x - __shfl(first, src, MI_WAVE);
+        req = b0 + src;
+        t0 = __shfl(start, src, MI_WAVE) + ti * tokens_per_tile;
+        n_tok = min(tokens_per_tile, __shfl(q_len, src, MI_WAVE) - ti * tokens_per_tile);
+      }
+      tiles_before += __shfl(inclusive, MI_WAVE - 1, MI_WAVE);
     }
   }
-  if (req < 0) return;
+  if (req < 0 || n_tok <= 0) return;
+  req = __builtin_amdgcn_readfirstlane(req);
+  t0 = __builtin_amdgcn_readfirstlane(t0);
+  n_tok = __builtin_amdgcn_readfirstlane(n_tok);
 
   const int group = q_heads / kv_heads;
   const int head_blocks = (group + heads_per_block - 1) / heads_per_block;
@@ -72,13 +99,19 @@ __global__ __launch_bounds__(64 * WAVES) void attn_mfma_kernel(
   const int n_heads = min(heads_per_block, group - g0);
   const int split = blockIdx.z;
 
-  const int wave = threadIdx.x / MI_WAVE;
+  static_assert(WAVES == 1 || KW == 1, "key-splitting waves are for single-row-group blocks");
+  // WAVES row groups of 16 rows; KW waves share a row group and take every KW-th key block
+  // (made wave-uniform for the compiler, so that key block numbers and with them the
+  // block-table reads are scalar and do not wait on the vector loads in flight)
+  const int wave_id = __builtin_amdgcn_readfirstlane(threadIdx.x / MI_WAVE);
+  const int wave = wave_id / KW;
+  const int key_wave = wave_id % KW;
   const int lane = threadIdx.x % MI_WAVE;
   const int col = lane % 16;  // this lane's row of work (a column of S^T and O^T)
   const int quad = lane / 16;  // 0..3
 
   // a wave whose 16 rows are all padding has nothing to do
-  if (wave * 16 >= n_tok * heads_per_block) return;
+  if (KW == 1 && wave * 16 >= n_tok * heads_per_block) return;
 
   const int row = wave * 16 + col;
   int tok_in_tile = row / heads_per_block;
@@ -115,9 +148,15 @@ __global__ __launch_bounds__(64 * WAVES) void attn_mfma_kernel(
   float m_run = -INFINITY;  // running maximum of this lane's row, in log2 units
   float l_run = 0.f;  // running sum of exp2(score - m_run)
 
-  for (int kb = (k_begin / 32) * 32; kb < k_end; kb += 32) {
-    // the (page, head) chunk and first slot of the two 16-key halves (a half never
-    // straddles a page); K rows of a chunk are [slot][D], V^T rows are [D][slot]
+  // One 32-key block: the K operands of its two 16-key halves and the V^T operands of
+  // all dim blocks.  A half never straddles a page; K rows of a (page, head) chunk are
+  // [slot][D], V^T rows are [D][slot].  Released or unallocated pages read page 0:
+  // every key of them is masked in the compute step.
+  struct KVBlock {
+    bf16x8_t k[2][KSTEPS];
+    bf16x8_t v[DBLOCKS];
+  };
+  auto load_block = [&](int kb, KVBlock& blk) {
     int64_t chunk_off[2];
     int slot0[2];
 #pragma unroll
@@ -125,25 +164,42 @@ __global__ __launch_bounds__(64 * WAVES) void attn_mfma_kernel(
       const int key0 = kb + 16 * hlf;
       const int idx = key0 / page_size;
       int page = (idx < max_blocks) ? bt[idx] : 0;
-      page = max(page, 0);  // released or unallocated: every key of it is masked below
+      page = max(page, 0);
       chunk_off[hlf] = ((int64_t)page * kv_heads + kvh) * page_size * D;
       slot0[hlf] = key0 % page_size;
     }
+#pragma unroll
+    for (int hlf = 0; hlf < 2; ++hlf) {
+      const bf16_t* k_row = k_pages + chunk_off[hlf] + (int64_t)(slot0[hlf] + col) * D + quad * 8;
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) blk.k[hlf][s] = *reinterpret_cast<const bf16x8_t*>(k_row + s * 32);
+    }
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) {
+      const int dim = db * 16 + col;
+      const bf16x4_t v0 = *reinterpret_cast<const bf16x4_t*>(
+          vt_pages + chunk_off[0] + (int64_t)dim * page_size + slot0[0] + 4 * quad);
+      const bf16x4_t v1 = *reinterpret_cast<const bf16x4_t*>(
+          vt_pages + chunk_off[1] + (int64_t)dim * page_size + slot0[1] + 4 * quad);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        blk.v[db][i] = v0[i];
+        blk.v[db][4 + i] = v1[i];
+      }
+    }
+  };
 
+  auto compute_block = [&](int kb, const KVBlock& blk) {
     // ---- S^T = K . Q^T for 32 keys ------------------------------------------------
     f32x4_t s_acc[2];
 #pragma unroll
     for (int hlf = 0; hlf < 2; ++hlf) {
-      const bf16_t* k_row = k_pages + chunk_off[hlf] + (int64_t)(slot0[hlf] + col) * D + quad * 8;
       f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < KSTEPS; ++s) {
-        const bf16x8_t k_reg = *reinterpret_cast<const bf16x8_t*>(k_row + s * 32);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_reg, q_reg[s], acc, 0, 0, 0);
-      }
+      for (int s = 0; s < KSTEPS; ++s)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[hlf][s], q_reg[s], acc, 0, 0, 0);
       s_acc[hlf] = acc;
     }
-
     // ---- scale, mask, online softmax (lane holds keys kb + 16*hlf + 4*quad + r) -----
     float sc[8];
     float mx = -INFINITY;
@@ -175,27 +231,70 @@ __global__ __launch_bounds__(64 * WAVES) void attn_mfma_kernel(
     sum += __shfl_xor(sum, 32, MI_WAVE);
     l_run = l_run * alpha + sum;
     m_run = m_new;
-
     // ---- O^T = O^T * alpha + V^T . P^T ------------------------------------------------
-    const int64_t v_chunk0 = chunk_off[0], v_chunk1 = chunk_off[1];
-    const int v_slot0 = slot0[0] + 4 * quad, v_slot1 = slot0[1] + 4 * quad;
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db) {
-      const int dim = db * 16 + col;
-      const bf16x4_t v0 =
-          *reinterpret_cast<const bf16x4_t*>(vt_pages + v_chunk0 + (int64_t)dim * page_size + v_slot0);
-      const bf16x4_t v1 =
-          *reinterpret_cast<const bf16x4_t*>(vt_pages + v_chunk1 + (int64_t)dim * page_size + v_slot1);
-      bf16x8_t v_reg;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        v_reg[i] = v0[i];
-        v_reg[4 + i] = v1[i];
-      }
       f32x4_t acc = o_acc[db];
 #pragma unroll
       for (int r = 0; r < 4; ++r) acc[r] *= alpha;
-      o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_reg, p_reg, acc, 0, 0, 0);
+      o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.v[db], p_reg, acc, 0, 0, 0);
+    }
+  };
+
+  // Software pipeline: the loads of the next block are in flight while this one is
+  // computed (two register sets, the loop advances two blocks a turn).
+  {
+    // The prefetch is unconditional (past the end it re-reads this wave's last block),
+    // so the compiler can count outstanding loads exactly instead of draining them all.
+    constexpr int STEP = 32 * KW;
+    KVBlock blk_a, blk_b;
+    int kb = (k_begin / 32) * 32 + 32 * key_wave;
+    if (kb < k_end) {
+      const int kb_last = kb + (k_end - 1 - kb) / STEP * STEP;
+      load_block(kb, blk_a);
+      while (true) {
+        load_block(min(kb + STEP, kb_last), blk_b);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_block(kb, blk_a);
+        __builtin_amdgcn_sched_barrier(0);
+        kb += STEP;
+        if (kb >= k_end) break;
+        load_block(min(kb + STEP, kb_last), blk_a);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_block(kb, blk_b);
+        __builtin_amdgcn_sched_barrier(0);
+        kb += STEP;
+        if (kb >= k_end) break;
+      }
+    }
+  }
+
+  // ---- waves that shared the rows merge their (max, sum, accumulator) in a fixed order ----
+  if (KW > 1) {
+    __shared__ float merge_o[KW > 1 ? KW - 1 : 1][DBLOCKS * 4][MI_WAVE];
+    __shared__ float merge_ml[KW > 1 ? KW - 1 : 1][2][MI_WAVE];
+    if (key_wave > 0) {
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) merge_o[key_wave - 1][db * 4 + r][lane] = o_acc[db][r];
+      merge_ml[key_wave - 1][0][lane] = m_run;
+      merge_ml[key_wave - 1][1][lane] = l_run;
+    }
+    __syncthreads();
+    if (key_wave > 0) return;
+    for (int other = 0; other < KW - 1; ++other) {
+      const float m_o = merge_ml[other][0][lane];
+      const float l_o = merge_ml[other][1][lane];
+      const float m_new = fmaxf(m_run, m_o);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float a = exp2f(m_run - m_safe), b = exp2f(m_o - m_safe);
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o_acc[db][r] = o_acc[db][r] * a + merge_o[other][db * 4 + r][lane] * b;
+      l_run = l_run * a + l_o * b;
+      m_run = m_new;
     }
   }
 
@@ -248,6 +347,8 @@ extern "C" int mi_attn_mfma_supported(int head_dim, int page_size) {
 
 // `num_tiles` = sum over requests of ceil(q_len / tokens_per_tile), computed by the
 // caller from the host copy of cu_seqlens_q (a larger number is harmless).
+// `one_tile_per_request` promises that no request has more than tokens_per_tile
+// tokens in this step; then num_tiles must be num_requests.
 // With num_splits > 1, part_acc holds num_tokens*q_heads*num_splits*head_dim floats
 // and part_ml num_tokens*q_heads*num_splits*2.
 extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_pages,
@@ -256,7 +357,8 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
                             int num_tokens, int num_tiles, void* out, int64_t out_row_stride,
                             float* part_acc, float* part_ml, int q_heads, int kv_heads,
                             int head_dim, int page_size, int num_pages, float scale, int window,
-                            int num_splits, int decode_only, hipStream_t stream) {
+                            int num_splits, int decode_only, int one_tile_per_request,
+                            hipStream_t stream) {
   MI_REQUIRE(num_tokens >= 0 && num_requests >= 0 && num_tiles >= 0,
              "attn_mfma: bad sizes tokens=%d requests=%d tiles=%d", num_tokens, num_requests, num_tiles);
   MI_REQUIRE(q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
@@ -267,12 +369,14 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
   MI_REQUIRE(num_pages > 0 && max_blocks > 0, "attn_mfma: bad page counts num_pages=%d max_blocks=%d",
              num_pages, max_blocks);
   MI_REQUIRE(window >= 0, "attn_mfma: window=%d must be 0 (none) or positive", window);
-  MI_REQUIRE(num_splits >= 1 && num_splits <= 65535, "attn_mfma: num_splits=%d out of range", num_splits);
+  MI_REQUIRE(num_splits >= 1 && num_splits <= 64, "attn_mfma: num_splits=%d must be 1..64", num_splits);
   MI_REQUIRE(num_splits == 1 || (part_acc && part_ml), "attn_mfma: split keys need partial buffers");
   MI_REQUIRE(q_row_stride >= (int64_t)q_heads * head_dim && out_row_stride >= (int64_t)q_heads * head_dim,
              "attn_mfma: row strides shorter than q_heads*head_dim");
   MI_REQUIRE(q_row_stride % 8 == 0 && out_row_stride % 4 == 0,
              "attn_mfma: row strides must keep 16-byte (q) and 8-byte (out) alignment");
+  MI_REQUIRE(!one_tile_per_request || num_tiles == num_requests,
+             "attn_mfma: one tile per request needs num_tiles == num_requests");
   if (num_tokens == 0 || num_tiles == 0) return MI_OK;
 
   const int group = q_heads / kv_heads;
@@ -284,15 +388,15 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
   dim3 grid(num_tiles, kv_heads * head_blocks, num_splits);
   const float scale_log2 = scale * LOG2E;
 
-#define MI_LAUNCH(DD, WW)                                                                         \
-  attn_mfma_kernel<DD, WW><<<grid, 64 * WW, 0, stream>>>(                                         \
+#define MI_LAUNCH(DD, WW, KK)                                                                     \
+  attn_mfma_kernel<DD, WW, KK><<<grid, 64 * WW * KK, 0, stream>>>(                                \
       (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)vt_pages,            \
       block_table, max_blocks, cu_seqlens_q, positions, num_requests, (bf16_t*)out,               \
       out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, scale_log2, window,        \
-      num_splits, hb, tq)
+      num_splits, hb, tq, one_tile_per_request)
 #define MI_LAUNCH_D(DD)            \
-  if (decode_only) MI_LAUNCH(DD, 1); \
-  else MI_LAUNCH(DD, 4)
+  if (decode_only) MI_LAUNCH(DD, 1, 4); \
+  else MI_LAUNCH(DD, 4, 1)
   switch (head_dim) {
     case 32: MI_LAUNCH_D(32); break;
     case 64: MI_LAUNCH_D(64); break;

@@ -19,6 +19,7 @@ import torch
 from mini_infer_amd.cache.manager import CacheManager
 from mini_infer_amd.config import DEFAULT_BLOCK_SIZE, DEFAULT_NUM_BLOCKS, read_config_json
 from mini_infer_amd.engine.batch import StepEntry
+from mini_infer_amd.engine.decode_graph import DecodeGraphs
 from mini_infer_amd.models import DecoderModel, architecture_for
 from mini_infer_amd.parts.base import StepContext
 from mini_infer_amd.weights import load_checkpoint
@@ -58,6 +59,7 @@ class ModelRunner:
         num_blocks: int = DEFAULT_NUM_BLOCKS,
         block_size: int = DEFAULT_BLOCK_SIZE,
         max_concurrent: int = 16,
+        cuda_graph: bool = True,
     ) -> None:
         self.model = model
         self.config = config
@@ -75,6 +77,8 @@ class ModelRunner:
             device=model.device,
         )
         self._layer_caches = self.cache.layer_caches()
+        # decode steps are replayed as HIP graphs where every part of the model allows it
+        self.decode_graphs = DecodeGraphs(self, max_batch=64) if cuda_graph and model.graph_safe else None
 
     # -- construction -----------------------------------------------------------
 
@@ -88,6 +92,7 @@ class ModelRunner:
         num_blocks: int = DEFAULT_NUM_BLOCKS,
         block_size: int = DEFAULT_BLOCK_SIZE,
         max_concurrent: int = 16,
+        cuda_graph: bool = True,
     ) -> "ModelRunner":
         """Load the model folder `model_name` (config.json + safetensors) and build its cache."""
         dev = require_gpu(device)
@@ -96,7 +101,8 @@ class ModelRunner:
         config = arch.parse_config(raw)
         model = DecoderModel(arch.build_spec(config), resolve_dtype(dtype), dev)
         load_checkpoint(model, model_name)
-        return cls(model, config, num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent)
+        return cls(model, config, num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent,
+                   cuda_graph=cuda_graph)
 
     @classmethod
     def from_random(
@@ -111,6 +117,7 @@ class ModelRunner:
         max_concurrent: int = 16,
         std: float = 0.02,
         norm_jitter: float = 0.0,
+        cuda_graph: bool = True,
     ) -> "ModelRunner":
         """Random weights made on the device (no file): for sizes too large to write out."""
         dev = require_gpu(device)
@@ -118,7 +125,8 @@ class ModelRunner:
         config = arch.parse_config(raw_config)
         model = DecoderModel(arch.build_spec(config), resolve_dtype(dtype), dev)
         fill_random_on_device(model, seed, std=std, norm_jitter=norm_jitter)
-        return cls(model, config, num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent)
+        return cls(model, config, num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent,
+                   cuda_graph=cuda_graph)
 
     # -- requests ---------------------------------------------------------------
 
@@ -140,7 +148,8 @@ class ModelRunner:
         """Run the given tokens as one batch from the cache; logits [wanted, vocab] float32.
 
         Rows come in the order of `entries` and, within an entry, of its `want`.
-        Requests seen for the first time are admitted.  Raises `OutOfMemoryError`
+        The tensor may be reused by the next step: read or copy it before calling
+        `step` again.  Requests seen for the first time are admitted.  Raises `OutOfMemoryError`
         before anything changes if the pages for this step are not there.
         """
         entries = [e for e in entries if len(e.tokens) > 0]
@@ -178,8 +187,11 @@ class ModelRunner:
             (int(index.cu_seqlens_q[b]) + w for b, e in enumerate(entries) for w in e.want),
             dtype=np.int32,
         )
-        ctx = self._to_device(token_ids.astype(np.int32), rows, index)
-        logits = self.model.forward(ctx, self._layer_caches)
+        token_ids = token_ids.astype(np.int32)
+        if self.decode_graphs is not None and self.decode_graphs.takes(index, rows):
+            logits = self.decode_graphs.run(token_ids, index)
+        else:
+            logits = self.model.forward(self._to_device(token_ids, rows, index), self._layer_caches)
         self.cache.commit(extents)
         return logits
 

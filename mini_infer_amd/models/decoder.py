@@ -46,6 +46,12 @@ class DecoderModel:
             tied_to=self.embedding if spec.tie_word_embeddings else None,
         )
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a decode step of this model can be recorded as a HIP graph."""
+        parts = [self.embedding, self.final_norm, self.head, *self.blocks]
+        return all(part.graph_safe for part in parts)
+
     # -- weights --------------------------------------------------------------
 
     def param_specs(self) -> dict[str, ParamSpec]:

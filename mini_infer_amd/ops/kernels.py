@@ -389,13 +389,13 @@ def paged_attention(
         q_lens = [host_cu_seqlens_q[b + 1] - host_cu_seqlens_q[b] for b in range(num_requests)]
         decode_only = max(q_lens) <= 1
         tokens_per_tile = lib.mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, int(decode_only))
-        num_tiles = sum(-(-n // tokens_per_tile) for n in q_lens)
+        one_tile_per_request = max(q_lens) <= tokens_per_tile
+        num_tiles = num_requests if one_tile_per_request else sum(-(-n // tokens_per_tile) for n in q_lens)
         rows = 16 if decode_only else 64
         head_blocks = -(-group // min(group, rows))
-        splits = attention_splits(
-            num_tiles * kv_heads * head_blocks, max_seq_len,
-            target=2048 if decode_only else 1024, min_keys=128,
-        )
+        # the kernel's blocks are register-heavy (one per CU at a time): about one
+        # block per CU measured best at batch 1, 8 and 64 and for short portions
+        splits = min(16, attention_splits(num_tiles * kv_heads * head_blocks, max_seq_len, target=256, min_keys=128))
         part_acc, part_ml = partials(splits)
         library.check(
             lib.mi_attn_mfma(
@@ -403,7 +403,7 @@ def paged_attention(
                 block_table.shape[1], _ptr(cu_seqlens_q), _ptr(positions), num_requests, tokens,
                 num_tiles, _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads,
                 head_dim, page_size, num_pages, float(scale), int(window or 0), splits,
-                int(decode_only), _stream(),
+                int(decode_only), int(one_tile_per_request), _stream(),
             )
         )
         return out

@@ -30,6 +30,8 @@ from mini_infer_amd.registry import POSITION_ENCODINGS, register_mixer
 
 
 class GQAttention(Mixer):
+    graph_safe = True
+
     def __init__(
         self,
         hidden_size: int,

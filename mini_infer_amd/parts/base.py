@@ -37,7 +37,15 @@ TensorGetter = Callable[[str], torch.Tensor]
 
 
 class Part:
-    """Base of all parts.  `dtype` is the compute dtype, float32 or bfloat16."""
+    """Base of all parts.  `dtype` is the compute dtype, float32 or bfloat16.
+
+    `graph_safe` says that `forward` only launches device work that depends on the
+    step through device tensors (not through host lists or Python loops over
+    requests), so a decode step containing the part can be recorded once as a HIP
+    graph and replayed.  Parts are not graph-safe unless they say so.
+    """
+
+    graph_safe = False
 
     def __init__(self, dtype: torch.dtype, device: torch.device | str) -> None:
         self.dtype = dtype

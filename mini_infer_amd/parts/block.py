@@ -41,6 +41,10 @@ class PreNormBlock(Block):
         self.feed_forward = feed_forward
         self.names = names  # part -> its prefix inside the layer, e.g. "self_attn."
 
+    @property
+    def graph_safe(self) -> bool:  # type: ignore[override]
+        return all(part.graph_safe for _, part in self._children())
+
     def _children(self):
         return (
             (self.names["mixer_norm"], self.mixer_norm),

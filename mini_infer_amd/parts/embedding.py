@@ -15,6 +15,8 @@ from mini_infer_amd.parts.base import ParamSpec, Part, TensorGetter
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int, name: str, dtype: torch.dtype, device) -> None:
         super().__init__(dtype, device)
         self.vocab_size = vocab_size
@@ -34,6 +36,8 @@ class TokenEmbedding(Part):
 
 
 class OutputHead(Part):
+    graph_safe = True
+
     def __init__(
         self,
         hidden_size: int,

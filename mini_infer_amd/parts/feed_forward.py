@@ -17,6 +17,8 @@ from mini_infer_amd.registry import register_feed_forward
 
 
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, dtype: torch.dtype, device) -> None:
         super().__init__(dtype, device)
         self.hidden_size = hidden_size

@@ -16,6 +16,8 @@ from mini_infer_amd.parts.base import ParamSpec, Part, TensorGetter
 
 
 class Linear(Part):
+    graph_safe = True
+
     def __init__(
         self,
         in_features: int,

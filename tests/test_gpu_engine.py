@@ -284,6 +284,50 @@ def test_first_tokens_of_a_sequence(tmp_path, name, dtype):
         ru.assert_close(got[f"s{length}"], expected, dtype, f"{name} first {length} tokens")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_graph_replays_equal_eager_steps_with_eager_work_between(tmp_path, dtype):
+    """Decode steps replayed as HIP graphs give the logits of the same steps run eagerly,
+    on every replay, with prompt portions (eager work) and synchronizations in between,
+    for batches that fill a bucket and batches that are padded."""
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+
+    cfg, block, weights, folder = _folder(tmp_path, "B", 59)
+    graphed = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=64, block_size=block, cuda_graph=True)
+    eager = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=64, block_size=block, cuda_graph=False)
+    assert graphed.decode_graphs is not None and eager.decode_graphs is None
+    rng = np.random.default_rng(0)
+    live: list[str] = []
+    limit = 2e-5 if dtype == "float32" else 0.05
+    for round_ in range(6):
+        # eager work: a new request's prompt in two portions, beside nothing else
+        rid = f"g{round_}"
+        prompt = tiny.random_tokens(cfg, int(rng.integers(20, 60)), seed=round_)
+        for runner in (graphed, eager):
+            runner.step([StepEntry(rid, prompt[:7], [])])
+            runner.step([StepEntry(rid, prompt[7:], [len(prompt) - 8])])
+        live.append(rid)
+        # several decode steps of all live requests (1, 2, 3, ... rows: padded buckets too)
+        for _ in range(5):
+            tokens = {r: int(rng.integers(0, cfg["vocab_size"])) for r in live}
+            outs = []
+            for runner in (graphed, eager):
+                logits = runner.step([StepEntry(r, [tokens[r]], [0]) for r in live])
+                outs.append(logits.cpu().numpy().copy())
+            torch.cuda.synchronize()
+            assert np.abs(outs[0] - outs[1]).max() < limit, f"round {round_}"
+    assert graphed.decode_graphs.replays == 30 and len(graphed.decode_graphs.graphs) >= 3
+    for runner in (graphed, eager):
+        for rid in live:
+            runner.free_request(rid)
+        runner.cache.check()
+
+
+def test_model_with_a_host_looping_part_is_not_graphed(tmp_path):
+    from mini_infer_amd.parts import Mixer
+
+    assert Mixer.graph_safe is False
+
+
 def test_step_refuses_bad_batches(tmp_path):
     from mini_infer_amd.engine import ModelRunner, StepEntry
     from mini_infer_amd.exceptions import OutOfMemoryError
