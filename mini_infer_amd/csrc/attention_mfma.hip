@@ -35,11 +35,30 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
+#define RESCALE_SLACK 8.0f
 #define LOG2E 1.4426950408889634f
 #define LN2 0.6931471805599453f
 
-template <int D, int WAVES, int KW>
-__global__ __launch_bounds__(64 * WAVES * KW) void attn_mfma_kernel(
+// Reductions over the 4 lanes that hold one row's scores (lane, lane^16, lane^32, lane^48)
+// with the gfx950 lane-swap instructions: no trip through the LDS crossbar.
+__device__ __forceinline__ float quad_max(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_sum(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+// VPF: value operands are prefetched a block ahead like the keys (more registers), or
+// loaded at the start of the block that uses them (fewer registers, so OCC waves of
+// different blocks can share a SIMD and fill each other's stalls).
+template <int D, int WAVES, int KW, int RG, bool VPF, int OCC>
+__global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_row_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ positions, int num_requests,
@@ -61,6 +80,9 @@ __global__ __launch_bounds__(64 * WAVES * KW) void attn_mfma_kernel(
       n_tok = cu_seqlens_q[req + 1] - t0;
     }
   } else {
+    // Tiles are handed out last first: under the causal mask a request's later tiles
+    // have more keys, and starting the long ones first keeps the GPU's tail short.
+    const int tile_index = (int)gridDim.x - 1 - (int)blockIdx.x;
     const int search_lane = threadIdx.x % MI_WAVE;
     int tiles_before = 0;
     for (int b0 = 0; b0 < num_requests && req < 0; b0 += MI_WAVE) {
@@ -75,11 +97,11 @@ __global__ __launch_bounds__(64 * WAVES * KW) void attn_mfma_kernel(
         if (search_lane >= off) inclusive += up;
       }
       const int first = tiles_before + inclusive - n_tiles;
-      const bool mine = n_tiles > 0 && (int)blockIdx.x >= first && (int)blockIdx.x < first + n_tiles;
+      const bool mine = n_tiles > 0 && tile_index >= first && tile_index < first + n_tiles;
       const unsigned long long owners = __ballot(mine);
       if (owners) {
         const int src = __ffsll((long long)owners) - 1;
-        const int ti = blockIdx.x - __shfl(first, src, MI_WAVE);
+        const int ti = tile_index - __shfl(first, src, MI_WAVE);
         req = b0 + src;
         t0 = __shfl(start, src, MI_WAVE) + ti * tokens_per_tile;
         n_tok = min(tokens_per_tile, __shfl(q_len, src, MI_WAVE) - ti * tokens_per_tile);
@@ -100,30 +122,51 @@ __global__ __launch_bounds__(64 * WAVES * KW) void attn_mfma_kernel(
   const int split = blockIdx.z;
 
   static_assert(WAVES == 1 || KW == 1, "key-splitting waves are for single-row-group blocks");
-  // WAVES row groups of 16 rows; KW waves share a row group and take every KW-th key block
-  // (made wave-uniform for the compiler, so that key block numbers and with them the
-  // block-table reads are scalar and do not wait on the vector loads in flight)
+  // WAVES wave slots of RG row groups (16 rows each); KW waves share a slot's rows and
+  // take every KW-th key block.  (Wave numbers are made uniform for the compiler, so
+  // that key block numbers and with them the block-table reads are scalar and do not
+  // wait on the vector loads in flight.)
   const int wave_id = __builtin_amdgcn_readfirstlane(threadIdx.x / MI_WAVE);
   const int wave = wave_id / KW;
   const int key_wave = wave_id % KW;
   const int lane = threadIdx.x % MI_WAVE;
-  const int col = lane % 16;  // this lane's row of work (a column of S^T and O^T)
+  const int col = lane % 16;  // this lane's row of work within a row group
   const int quad = lane / 16;  // 0..3
 
-  // a wave whose 16 rows are all padding has nothing to do
-  if (KW == 1 && wave * 16 >= n_tok * heads_per_block) return;
+  // a wave whose rows are all padding has nothing to do
+  if (KW == 1 && wave * 16 * RG >= n_tok * heads_per_block) return;
 
-  const int row = wave * 16 + col;
-  int tok_in_tile = row / heads_per_block;
-  int head_in_block = row % heads_per_block;
-  const bool row_valid = tok_in_tile < n_tok && head_in_block < n_heads;
-  tok_in_tile = min(tok_in_tile, n_tok - 1);  // padded rows repeat a real row and store nothing
-  head_in_block = min(head_in_block, n_heads - 1);
-  const int token = t0 + tok_in_tile;
-  const int head = kvh * group + g0 + head_in_block;
   const int pos0 = positions[t0];  // tokens of a tile sit at consecutive positions
-  const int pos = pos0 + tok_in_tile;
-  const int lo_row = (window > 0) ? max(0, pos - window + 1) : 0;
+  int token[RG], head[RG], pos[RG], lo_row[RG];
+  bool row_valid[RG];
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg) {
+    const int row = (wave * RG + rg) * 16 + col;
+    int tok_in_tile = row / heads_per_block;
+    int head_in_block = row % heads_per_block;
+    row_valid[rg] = tok_in_tile < n_tok && head_in_block < n_heads;
+    tok_in_tile = min(tok_in_tile, n_tok - 1);  // padded rows repeat a real row and store nothing
+    head_in_block = min(head_in_block, n_heads - 1);
+    token[rg] = t0 + tok_in_tile;
+    head[rg] = kvh * group + g0 + head_in_block;
+    pos[rg] = pos0 + tok_in_tile;
+    lo_row[rg] = (window > 0) ? max(0, pos[rg] - window + 1) : 0;
+  }
+
+  // smallest position and largest window start among this wave's rows (for the mask-free test)
+  int wave_pos_min = pos[0], wave_lo_max = lo_row[0];
+#pragma unroll
+  for (int rg = 1; rg < RG; ++rg) {
+    wave_pos_min = min(wave_pos_min, pos[rg]);
+    wave_lo_max = max(wave_lo_max, lo_row[rg]);
+  }
+#pragma unroll
+  for (int off = 1; off < 16; off <<= 1) {
+    wave_pos_min = min(wave_pos_min, __shfl_xor(wave_pos_min, off, MI_WAVE));
+    wave_lo_max = max(wave_lo_max, __shfl_xor(wave_lo_max, off, MI_WAVE));
+  }
+  wave_pos_min = __builtin_amdgcn_readfirstlane(wave_pos_min);
+  wave_lo_max = __builtin_amdgcn_readfirstlane(wave_lo_max);
 
   // ---- key range of this block ------------------------------------------------
   const int tile_lo = (window > 0) ? max(0, pos0 - window + 1) : 0;
@@ -134,19 +177,24 @@ __global__ __launch_bounds__(64 * WAVES * KW) void attn_mfma_kernel(
   const int k_end = min(k_begin + chunk, tile_hi);
   const int* bt = block_table + (int64_t)req * max_blocks;
 
-  // ---- Q^T operand: this lane's row, 8 consecutive dims per k-step --------------
-  bf16x8_t q_reg[KSTEPS];
-  {
-    const bf16_t* q_row = q + (int64_t)token * q_row_stride + (int64_t)head * D + quad * 8;
+  // ---- Q^T operands: this lane's rows, 8 consecutive dims per k-step --------------
+  bf16x8_t q_reg[RG][KSTEPS];
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) q_reg[s] = *reinterpret_cast<const bf16x8_t*>(q_row + s * 32);
+  for (int rg = 0; rg < RG; ++rg) {
+    const bf16_t* q_row = q + (int64_t)token[rg] * q_row_stride + (int64_t)head[rg] * D + quad * 8;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) q_reg[rg][s] = *reinterpret_cast<const bf16x8_t*>(q_row + s * 32);
   }
 
-  f32x4_t o_acc[DBLOCKS];
+  f32x4_t o_acc[RG][DBLOCKS];
+  float m_run[RG], l_run[RG];  // running maximum (log2 units) and sum of exp2(score - max)
 #pragma unroll
-  for (int db = 0; db < DBLOCKS; ++db) o_acc[db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY;  // running maximum of this lane's row, in log2 units
-  float l_run = 0.f;  // running sum of exp2(score - m_run)
+  for (int rg = 0; rg < RG; ++rg) {
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) o_acc[rg][db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    m_run[rg] = -INFINITY;
+    l_run[rg] = 0.f;
+  }
 
   // One 32-key block: the K operands of its two 16-key halves and the V^T operands of
   // all dim blocks.  A half never straddles a page; K rows of a (page, head) chunk are
@@ -154,90 +202,141 @@ __global__ __launch_bounds__(64 * WAVES * KW) void attn_mfma_kernel(
   // every key of them is masked in the compute step.
   struct KVBlock {
     bf16x8_t k[2][KSTEPS];
-    bf16x8_t v[DBLOCKS];
+    bf16x8_t v[VPF ? DBLOCKS : 1];
+    const bf16_t* v_base[2];
+  };
+  // Addresses are a wave-uniform base (page, head, first slot: scalar registers) plus a
+  // per-lane 32-bit offset that never changes, so a load costs no vector arithmetic.
+  // Page ids come from a register: lane j of `page_vec` holds block-table entry
+  // page_base + j, refilled every 64 pages, so the walk over the keys does not wait on a
+  // block-table read per step.
+  int page_vec = 0;
+  int page_base = -(1 << 30);
+  auto page_of = [&](int idx) -> int {  // idx is wave-uniform
+    if (idx < page_base || idx - page_base >= MI_WAVE) {
+      page_base = idx;
+      const int j = idx + lane;
+      page_vec = (j < max_blocks) ? bt[j] : 0;
+    }
+    return __builtin_amdgcn_readlane(page_vec, idx - page_base);
+  };
+  const unsigned k_lane_off = (unsigned)(col * D + quad * 8);
+  const unsigned v_lane_off = (unsigned)(col * page_size + 4 * quad);
+  auto load_values = [&](const bf16_t* const v_base[2], bf16x8_t* v) {
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) {
+      const unsigned off = v_lane_off + (unsigned)(db * 16) * (unsigned)page_size;
+      const bf16x4_t v0 = *reinterpret_cast<const bf16x4_t*>(v_base[0] + off);
+      const bf16x4_t v1 = *reinterpret_cast<const bf16x4_t*>(v_base[1] + off);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[db][i] = v0[i];
+        v[db][4 + i] = v1[i];
+      }
+    }
   };
   auto load_block = [&](int kb, KVBlock& blk) {
-    int64_t chunk_off[2];
-    int slot0[2];
+    const bf16_t* k_base[2];
 #pragma unroll
     for (int hlf = 0; hlf < 2; ++hlf) {
       const int key0 = kb + 16 * hlf;
       const int idx = key0 / page_size;
-      int page = (idx < max_blocks) ? bt[idx] : 0;
-      page = max(page, 0);
-      chunk_off[hlf] = ((int64_t)page * kv_heads + kvh) * page_size * D;
-      slot0[hlf] = key0 % page_size;
+      const int page = max(page_of(idx), 0);
+      const int64_t chunk_off = ((int64_t)page * kv_heads + kvh) * page_size * D;
+      const int slot0 = key0 % page_size;
+      k_base[hlf] = k_pages + chunk_off + (int64_t)slot0 * D;
+      blk.v_base[hlf] = vt_pages + chunk_off + slot0;
     }
 #pragma unroll
     for (int hlf = 0; hlf < 2; ++hlf) {
-      const bf16_t* k_row = k_pages + chunk_off[hlf] + (int64_t)(slot0[hlf] + col) * D + quad * 8;
-#pragma unroll
-      for (int s = 0; s < KSTEPS; ++s) blk.k[hlf][s] = *reinterpret_cast<const bf16x8_t*>(k_row + s * 32);
-    }
-#pragma unroll
-    for (int db = 0; db < DBLOCKS; ++db) {
-      const int dim = db * 16 + col;
-      const bf16x4_t v0 = *reinterpret_cast<const bf16x4_t*>(
-          vt_pages + chunk_off[0] + (int64_t)dim * page_size + slot0[0] + 4 * quad);
-      const bf16x4_t v1 = *reinterpret_cast<const bf16x4_t*>(
-          vt_pages + chunk_off[1] + (int64_t)dim * page_size + slot0[1] + 4 * quad);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        blk.v[db][i] = v0[i];
-        blk.v[db][4 + i] = v1[i];
-      }
-    }
-  };
-
-  auto compute_block = [&](int kb, const KVBlock& blk) {
-    // ---- S^T = K . Q^T for 32 keys ------------------------------------------------
-    f32x4_t s_acc[2];
-#pragma unroll
-    for (int hlf = 0; hlf < 2; ++hlf) {
-      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[hlf][s], q_reg[s], acc, 0, 0, 0);
-      s_acc[hlf] = acc;
+        blk.k[hlf][s] = *reinterpret_cast<const bf16x8_t*>(k_base[hlf] + (k_lane_off + s * 32));
     }
-    // ---- scale, mask, online softmax (lane holds keys kb + 16*hlf + 4*quad + r) -----
-    float sc[8];
-    float mx = -INFINITY;
+    if (VPF) load_values(blk.v_base, blk.v);
+  };
+
+  // The three phases run over all row groups of the wave in turn (scores for every
+  // group, then every group's softmax, then every group's value product): the groups
+  // are independent, so one group's vector work overlaps another's matrix work.
+  auto compute_block = [&](int kb, KVBlock& blk) {
+    bf16x8_t v_late[VPF ? 1 : DBLOCKS];
+    if (!VPF) load_values(blk.v_base, v_late);  // in flight during the scores and the softmax
+    const bf16x8_t* v_op = VPF ? blk.v : v_late;
+    // ---- S^T = K . Q^T for 32 keys ------------------------------------------------
+    f32x4_t s_acc[RG][2];
 #pragma unroll
-    for (int hlf = 0; hlf < 2; ++hlf) {
+    for (int rg = 0; rg < RG; ++rg) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int key = kb + 16 * hlf + 4 * quad + r;
-        const bool visible = key >= lo_row && key <= pos && key >= k_begin && key < k_end;
-        const float v = visible ? s_acc[hlf][r] * scale_log2 : -INFINITY;
-        sc[hlf * 4 + r] = v;
-        mx = fmaxf(mx, v);
+      for (int hlf = 0; hlf < 2; ++hlf) {
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[hlf][s], q_reg[rg][s], acc, 0, 0, 0);
+        s_acc[rg][hlf] = acc;
       }
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, MI_WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, MI_WAVE));
-    const float m_new = fmaxf(m_run, mx);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen nothing yet
-    const float alpha = exp2f(m_run - m_safe);  // exp2(-inf) = 0 on the first visible block
-    float sum = 0.f;
-    bf16x8_t p_reg;
+    // ---- scale, mask, online softmax (lane holds keys kb + 16*hlf + 4*quad + r) -----
+    // a block every row of this wave sees whole needs no mask (most blocks of a long prompt)
+    const bool interior = kb >= wave_lo_max && kb + 31 <= wave_pos_min && kb >= k_begin && kb + 32 <= k_end;
+    bf16x8_t p_reg[RG];
+    float alpha[RG];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float p = exp2f(sc[i] - m_safe);
-      sum += p;
-      p_reg[i] = (bf16_t)p;
+    for (int rg = 0; rg < RG; ++rg) {
+      float sc[8];
+      float mx = -INFINITY;
+      if (interior) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          sc[i] = s_acc[rg][i / 4][i % 4] * scale_log2;
+          mx = fmaxf(mx, sc[i]);
+        }
+      } else {
+#pragma unroll
+        for (int hlf = 0; hlf < 2; ++hlf) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int key = kb + 16 * hlf + 4 * quad + r;
+            const bool visible = key >= lo_row[rg] && key <= pos[rg] && key >= k_begin && key < k_end;
+            const float v = visible ? s_acc[rg][hlf][r] * scale_log2 : -INFINITY;
+            sc[hlf * 4 + r] = v;
+            mx = fmaxf(mx, v);
+          }
+        }
+      }
+      mx = quad_max(mx);
+      // The reference point of the exponentials follows the running maximum lazily: it
+      // moves only when the maximum grows by more than RESCALE_SLACK (in log2 units), so
+      // probabilities stay below 2^RESCALE_SLACK and the accumulator is rarely rescaled.
+      const float m_new = (mx > m_run[rg] + RESCALE_SLACK) ? mx : m_run[rg];
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen nothing yet
+      // arguments are bounded above: the hardware exp2 is exact enough, tiny results flush to 0
+      alpha[rg] = __builtin_amdgcn_exp2f(m_run[rg] - m_safe);  // 0 on the first visible block
+      float sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float p = __builtin_amdgcn_exp2f(sc[i] - m_safe);
+        sum += p;
+        p_reg[rg][i] = (bf16_t)p;
+      }
+      sum = quad_sum(sum);
+      l_run[rg] = l_run[rg] * alpha[rg] + sum;
+      m_run[rg] = m_new;
     }
-    sum += __shfl_xor(sum, 16, MI_WAVE);
-    sum += __shfl_xor(sum, 32, MI_WAVE);
-    l_run = l_run * alpha + sum;
-    m_run = m_new;
     // ---- O^T = O^T * alpha + V^T . P^T ------------------------------------------------
 #pragma unroll
-    for (int db = 0; db < DBLOCKS; ++db) {
-      f32x4_t acc = o_acc[db];
+    for (int rg = 0; rg < RG; ++rg) {
+      // alpha is 1 in every lane unless some row's reference point moved
+      // (one branch around the whole rescale, so that it is not turned into selects)
+      if (__ballot(alpha[rg] != 1.f) != 0ull) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) acc[r] *= alpha;
-      o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.v[db], p_reg, acc, 0, 0, 0);
+        for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o_acc[rg][db][r] *= alpha[rg];
+      }
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db)
+        o_acc[rg][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op[db], p_reg[rg], o_acc[rg][db], 0, 0, 0);
     }
   };
 
@@ -271,55 +370,65 @@ __global__ __launch_bounds__(64 * WAVES * KW) void attn_mfma_kernel(
 
   // ---- waves that shared the rows merge their (max, sum, accumulator) in a fixed order ----
   if (KW > 1) {
-    __shared__ float merge_o[KW > 1 ? KW - 1 : 1][DBLOCKS * 4][MI_WAVE];
-    __shared__ float merge_ml[KW > 1 ? KW - 1 : 1][2][MI_WAVE];
+    __shared__ float merge_o[KW > 1 ? KW - 1 : 1][RG * DBLOCKS * 4][MI_WAVE];
+    __shared__ float merge_ml[KW > 1 ? KW - 1 : 1][RG * 2][MI_WAVE];
     if (key_wave > 0) {
 #pragma unroll
-      for (int db = 0; db < DBLOCKS; ++db)
+      for (int rg = 0; rg < RG; ++rg) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) merge_o[key_wave - 1][db * 4 + r][lane] = o_acc[db][r];
-      merge_ml[key_wave - 1][0][lane] = m_run;
-      merge_ml[key_wave - 1][1][lane] = l_run;
+        for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) merge_o[key_wave - 1][(rg * DBLOCKS + db) * 4 + r][lane] = o_acc[rg][db][r];
+        merge_ml[key_wave - 1][rg * 2][lane] = m_run[rg];
+        merge_ml[key_wave - 1][rg * 2 + 1][lane] = l_run[rg];
+      }
     }
     __syncthreads();
     if (key_wave > 0) return;
     for (int other = 0; other < KW - 1; ++other) {
-      const float m_o = merge_ml[other][0][lane];
-      const float l_o = merge_ml[other][1][lane];
-      const float m_new = fmaxf(m_run, m_o);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float a = exp2f(m_run - m_safe), b = exp2f(m_o - m_safe);
 #pragma unroll
-      for (int db = 0; db < DBLOCKS; ++db)
+      for (int rg = 0; rg < RG; ++rg) {
+        const float m_o = merge_ml[other][rg * 2][lane];
+        const float l_o = merge_ml[other][rg * 2 + 1][lane];
+        const float m_new = fmaxf(m_run[rg], m_o);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float a = exp2f(m_run[rg] - m_safe), b = exp2f(m_o - m_safe);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o_acc[db][r] = o_acc[db][r] * a + merge_o[other][db * 4 + r][lane] * b;
-      l_run = l_run * a + l_o * b;
-      m_run = m_new;
+        for (int db = 0; db < DBLOCKS; ++db)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            o_acc[rg][db][r] = o_acc[rg][db][r] * a + merge_o[other][(rg * DBLOCKS + db) * 4 + r][lane] * b;
+        l_run[rg] = l_run[rg] * a + l_o * b;
+        m_run[rg] = m_new;
+      }
     }
   }
 
   // ---- write: lane holds O^T[dim = 16*db + 4*quad + r][its row] ------------------------
-  if (!row_valid) return;
-  if (num_splits == 1) {
-    const float inv = 1.f / l_run;
-    bf16_t* o = out + (int64_t)token * out_row_stride + (int64_t)head * D + quad * 4;
 #pragma unroll
-    for (int db = 0; db < DBLOCKS; ++db) {
-      bf16x4_t packed;
+  for (int rg = 0; rg < RG; ++rg) {
+    if (!row_valid[rg]) continue;
+    if (num_splits == 1) {
+      const float inv = 1.f / l_run[rg];
+      bf16_t* o = out + (int64_t)token[rg] * out_row_stride + (int64_t)head[rg] * D + quad * 4;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) packed[r] = (bf16_t)(o_acc[db][r] * inv);
-      *reinterpret_cast<bf16x4_t*>(o + db * 16) = packed;
-    }
-  } else {
-    const int64_t slot = ((int64_t)token * q_heads + head) * num_splits + split;
-    float* pa = part_acc + slot * D + quad * 4;
+      for (int db = 0; db < DBLOCKS; ++db) {
+        bf16x4_t packed;
 #pragma unroll
-    for (int db = 0; db < DBLOCKS; ++db) {
-      *reinterpret_cast<f32x4_t*>(pa + db * 16) = o_acc[db];
-    }
-    if (quad == 0) {
-      part_ml[slot * 2] = m_run * LN2;  // natural-log units, as the combining kernel expects
-      part_ml[slot * 2 + 1] = l_run;
+        for (int r = 0; r < 4; ++r) packed[r] = (bf16_t)(o_acc[rg][db][r] * inv);
+        *reinterpret_cast<bf16x4_t*>(o + db * 16) = packed;
+      }
+    } else {
+      const int64_t slot = ((int64_t)token[rg] * q_heads + head[rg]) * num_splits + split;
+      float* pa = part_acc + slot * D + quad * 4;
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db) {
+        *reinterpret_cast<f32x4_t*>(pa + db * 16) = o_acc[rg][db];
+      }
+      if (quad == 0) {
+        part_ml[slot * 2] = m_run[rg] * LN2;  // natural-log units, as the combining kernel expects
+        part_ml[slot * 2 + 1] = l_run[rg];
+      }
     }
   }
 }
@@ -331,9 +440,12 @@ extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, 
 static int heads_per_block_for(int group, int rows) { return group < rows ? group : rows; }
 
 // Tiling the Python side needs to size the grid: tokens per tile for a group size.
+#define MI_PREFILL_RG 2  // row groups (of 16 rows) per wave in the prefill shape
+#define MI_PREFILL_ROWS (64 * MI_PREFILL_RG)
+
 extern "C" int mi_attn_mfma_tokens_per_tile(int q_heads, int kv_heads, int decode_only) {
   if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return 0;
-  const int rows = decode_only ? 16 : 64;
+  const int rows = decode_only ? 16 : MI_PREFILL_ROWS;
   const int hb = heads_per_block_for(q_heads / kv_heads, rows);
   const int t = rows / hb;
   return t < 1 ? 1 : t;
@@ -380,7 +492,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
   if (num_tokens == 0 || num_tiles == 0) return MI_OK;
 
   const int group = q_heads / kv_heads;
-  const int rows = decode_only ? 16 : 64;
+  const int rows = decode_only ? 16 : MI_PREFILL_ROWS;
   const int hb = heads_per_block_for(group, rows);
   const int tq = mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, decode_only);
   const int head_blocks = ceil_div(group, hb);
@@ -388,15 +500,15 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
   dim3 grid(num_tiles, kv_heads * head_blocks, num_splits);
   const float scale_log2 = scale * LOG2E;
 
-#define MI_LAUNCH(DD, WW, KK)                                                                     \
-  attn_mfma_kernel<DD, WW, KK><<<grid, 64 * WW * KK, 0, stream>>>(                                \
+#define MI_LAUNCH(DD, WW, KK, RR, VV, OO)                                                         \
+  attn_mfma_kernel<DD, WW, KK, RR, VV, OO><<<grid, 64 * WW * KK, 0, stream>>>(                    \
       (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)vt_pages,            \
       block_table, max_blocks, cu_seqlens_q, positions, num_requests, (bf16_t*)out,               \
       out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, scale_log2, window,        \
       num_splits, hb, tq, one_tile_per_request)
 #define MI_LAUNCH_D(DD)            \
-  if (decode_only) MI_LAUNCH(DD, 1, 4); \
-  else MI_LAUNCH(DD, 4, 1)
+  if (decode_only) MI_LAUNCH(DD, 1, 4, 1, false, 2); \
+  else MI_LAUNCH(DD, 4, 1, MI_PREFILL_RG, false, 1)
   switch (head_dim) {
     case 32: MI_LAUNCH_D(32); break;
     case 64: MI_LAUNCH_D(64); break;

@@ -82,10 +82,10 @@ extern "C" int mi_embed_gather(int dtype, const void* table, const int* ids, flo
 // ---------------------------------------------------------------------------
 
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void add_rmsnorm_kernel(
+__global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
     const T* __restrict__ delta, float* __restrict__ residual, const T* __restrict__ weight,
     T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
-  __shared__ float scratch[4];
+  __shared__ float scratch[16];
   const int b = blockIdx.x;
   const int64_t r = rows ? rows[b] : b;
   float* res = residual + r * hidden;
@@ -152,7 +152,9 @@ static int add_rmsnorm_launch(const void* delta, float* residual, const void* we
                               hipStream_t stream) {
   if (num_out_rows == 0) return MI_OK;
   if (hidden % 4 == 0) {
-    add_rmsnorm_kernel<T, 4><<<num_out_rows, 256, 0, stream>>>(
+    // one vector of 4 per thread and pass where the row allows: fewer dependent steps
+    const int threads = min(1024, max(256, ceil_div(hidden / 4, 64) * 64));
+    add_rmsnorm_kernel<T, 4><<<num_out_rows, threads, 0, stream>>>(
         (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps);
   } else {
     add_rmsnorm_kernel<T, 1><<<num_out_rows, 256, 0, stream>>>(
@@ -218,12 +220,15 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     T* __restrict__ v_pages, int q_heads, int kv_heads, int head_dim, int rotary_dim,
     int interleaved, int page_size, int v_transposed) {
   const int t = blockIdx.x;
+  // the blocks along y share a token's work items
+  const int first = blockIdx.y * blockDim.x + threadIdx.x;
+  const int stride = blockDim.x * gridDim.y;
   const int half = rotary_dim / 2;
   T* row = qkv + (int64_t)t * row_stride;
   const float* c = cos_t + (int64_t)t * half;
   const float* s = sin_t + (int64_t)t * half;
 
-  for (int e = threadIdx.x; e < q_heads * half; e += blockDim.x) {
+  for (int e = first; e < q_heads * half; e += stride) {
     const int h = e / half, j = e % half;
     const int i0 = interleaved ? 2 * j : j;
     const int i1 = interleaved ? 2 * j + 1 : j + half;
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   const T* k_row = row + (int64_t)q_heads * head_dim;
   const T* v_row = k_row + (int64_t)kv_heads * head_dim;
 
-  for (int e = threadIdx.x; e < kv_heads * half; e += blockDim.x) {
+  for (int e = first; e < kv_heads * half; e += stride) {
     const int h = e / half, j = e % half;
     const int i0 = interleaved ? 2 * j : j;
     const int i1 = interleaved ? 2 * j + 1 : j + half;
@@ -251,11 +256,11 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     dst[i1] = from_f32<T>(x1 * c[j] + x0 * s[j]);
   }
   const int pass = head_dim - rotary_dim;
-  for (int e = threadIdx.x; e < kv_heads * pass; e += blockDim.x) {
+  for (int e = first; e < kv_heads * pass; e += stride) {
     const int h = e / pass, d = rotary_dim + e % pass;
     k_pages[(((int64_t)page * kv_heads + h) * page_size + off) * head_dim + d] = k_row[h * head_dim + d];
   }
-  for (int e = threadIdx.x; e < kv_heads * head_dim; e += blockDim.x) {
+  for (int e = first; e < kv_heads * head_dim; e += stride) {
     const int h = e / head_dim, d = e % head_dim;
     const int64_t chunk = ((int64_t)page * kv_heads + h) * page_size * head_dim;
     const int64_t at = v_transposed ? chunk + (int64_t)d * page_size + off : chunk + (int64_t)off * head_dim + d;
@@ -279,12 +284,16 @@ extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const 
              "rope_kv_write: pages are needed to write keys and values");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "rope_kv_write: unknown dtype %d", dtype);
   if (num_tokens == 0) return MI_OK;
+  // few tokens (decode): spread each token's heads over several blocks
+  const int items = max(q_heads * (rotary_dim / 2), kv_heads * head_dim);
+  const int blocks_y = (num_tokens >= 512) ? 1 : min(16, max(1, ceil_div(items, 256)));
+  dim3 grid(num_tokens, blocks_y);
   if (dtype == MI_F32) {
-    rope_kv_write_kernel<float><<<num_tokens, 256, 0, stream>>>(
+    rope_kv_write_kernel<float><<<grid, 256, 0, stream>>>(
         (float*)qkv, row_stride, cos_t, sin_t, slot_mapping, (float*)k_pages, (float*)v_pages,
         q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size, v_transposed);
   } else {
-    rope_kv_write_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
+    rope_kv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, cos_t, sin_t, slot_mapping, (bf16_t*)k_pages, (bf16_t*)v_pages,
         q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size, v_transposed);
   }

@@ -391,7 +391,7 @@ def paged_attention(
         tokens_per_tile = lib.mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, int(decode_only))
         one_tile_per_request = max(q_lens) <= tokens_per_tile
         num_tiles = num_requests if one_tile_per_request else sum(-(-n // tokens_per_tile) for n in q_lens)
-        rows = 16 if decode_only else 64
+        rows = 16 if decode_only else 128
         head_blocks = -(-group // min(group, rows))
         # the kernel's blocks are register-heavy (one per CU at a time): about one
         # block per CU measured best at batch 1, 8 and 64 and for short portions
