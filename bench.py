@@ -74,7 +74,8 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=256)
+    # defaults: 8 untimed steps, then every step up to 4,096 total positions
+    parser.add_argument("--steps", type=int, default=PROMPT_LEN - 8)
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--layers", type=int, default=FULL_LAYERS)
@@ -85,8 +86,8 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
-    if not 0 < args.steps <= PROMPT_LEN:
-        print(f"bench.py: --steps must be in 1..{PROMPT_LEN} (decoding runs from 2,048 to at most 4,096)")
+    if args.steps <= 0 or args.warmup < 0 or args.steps + args.warmup > PROMPT_LEN:
+        print(f"bench.py: --warmup + --steps must be at most {PROMPT_LEN} (decoding runs from 2,048 to at most 4,096)")
         return 2
 
     import numpy as np

@@ -286,7 +286,7 @@ extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const 
   if (num_tokens == 0) return MI_OK;
   // few tokens (decode): spread each token's heads over several blocks
   const int items = max(q_heads * (rotary_dim / 2), kv_heads * head_dim);
-  const int blocks_y = (num_tokens >= 512) ? 1 : min(16, max(1, ceil_div(items, 256)));
+  const int blocks_y = min((num_tokens >= 512) ? 4 : 16, max(1, ceil_div(items, 256)));
   dim3 grid(num_tokens, blocks_y);
   if (dtype == MI_F32) {
     rope_kv_write_kernel<float><<<grid, 256, 0, stream>>>(
