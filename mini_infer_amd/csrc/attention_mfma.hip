@@ -57,32 +57,50 @@ __device__ __forceinline__ float quad_sum(float v) {
 // VPF: value operands are prefetched a block ahead like the keys (more registers), or
 // loaded at the start of the block that uses them (fewer registers, so OCC waves of
 // different blocks can share a SIMD and fill each other's stalls).
-template <int D, int WAVES, int KW, int RG, bool VPF, int OCC>
+template <int D, int WAVES, int KW, int RG, bool VPF, int OCC, bool ONE_SET, int PS>
 __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_row_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ positions, int num_requests,
     bf16_t* __restrict__ out, int64_t out_row_stride, float* __restrict__ part_acc,
-    float* __restrict__ part_ml, int q_heads, int kv_heads, int page_size, float scale_log2,
+    float* __restrict__ part_ml, int q_heads, int kv_heads, int page_size_arg, unsigned page_magic, float scale_log2,
     int window, int num_splits, int heads_per_block, int tokens_per_tile, int one_tile_per_request) {
   constexpr int KSTEPS = D / 32;  // MFMA k-steps over the head dim for S^T
+  // PS != 0: the page size is this constant (divisions become shifts, value offsets
+  // immediates); PS == 0: any multiple of 16, divided by multiplying with
+  // page_magic = floor(2^32 / page_size) + 1 (exact for keys below 2^32 / page_size).
+  const int page_size = PS ? PS : page_size_arg;
+  auto page_index = [&](int key) -> int {
+    return PS ? key / PS : (int)__umulhi((unsigned)key, page_magic);
+  };
   constexpr int DBLOCKS = D / 16;  // 16-dim blocks of the output
 
   // ---- which tile of which request ----------------------------------------
   // Every wave finds it on its own.  With at most one tile per request (decode, short
   // portions) the tile IS the request; otherwise the lanes share the search: each takes
   // a request, a prefix sum over the requests' tile counts locates the tile.
+  // The grid is one-dimensional in (tile, head block) with the HEAD BLOCK running
+  // fastest: consecutive workgroups go to different XCDs (8, each with an L2 of its
+  // own), so with a multiple of 8 head blocks every XCD sees the keys and values of
+  // only its share of the heads, whatever the number of tiles, and they stay in its L2
+  // for all the tiles of a prompt.
+  const int group = q_heads / kv_heads;
+  const int head_blocks = (group + heads_per_block - 1) / heads_per_block;
+  const int head_slots = kv_heads * head_blocks;
+  const int grid_tile = (int)(blockIdx.x / (unsigned)head_slots);
+  const int grid_head = (int)(blockIdx.x % (unsigned)head_slots);
+  const int grid_tiles = (int)(gridDim.x / (unsigned)head_slots);
   int req = -1, t0 = 0, n_tok = 0;
   if (one_tile_per_request) {
-    if ((int)blockIdx.x < num_requests) {
-      req = blockIdx.x;
+    if (grid_tile < num_requests) {
+      req = grid_tile;
       t0 = cu_seqlens_q[req];
       n_tok = cu_seqlens_q[req + 1] - t0;
     }
   } else {
     // Tiles are handed out last first: under the causal mask a request's later tiles
     // have more keys, and starting the long ones first keeps the GPU's tail short.
-    const int tile_index = (int)gridDim.x - 1 - (int)blockIdx.x;
+    const int tile_index = grid_tiles - 1 - grid_tile;
     const int search_lane = threadIdx.x % MI_WAVE;
     int tiles_before = 0;
     for (int b0 = 0; b0 < num_requests && req < 0; b0 += MI_WAVE) {
@@ -114,10 +132,8 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   t0 = __builtin_amdgcn_readfirstlane(t0);
   n_tok = __builtin_amdgcn_readfirstlane(n_tok);
 
-  const int group = q_heads / kv_heads;
-  const int head_blocks = (group + heads_per_block - 1) / heads_per_block;
-  const int kvh = blockIdx.y / head_blocks;
-  const int g0 = (blockIdx.y % head_blocks) * heads_per_block;
+  const int kvh = grid_head / head_blocks;
+  const int g0 = (grid_head % head_blocks) * heads_per_block;
   const int n_heads = min(heads_per_block, group - g0);
   const int split = blockIdx.z;
 
@@ -207,19 +223,24 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   };
   // Addresses are a wave-uniform base (page, head, first slot: scalar registers) plus a
   // per-lane 32-bit offset that never changes, so a load costs no vector arithmetic.
-  // Page ids come from a register: lane j of `page_vec` holds block-table entry
-  // page_base + j, refilled every 64 pages, so the walk over the keys does not wait on a
-  // block-table read per step.
-  int page_vec = 0;
-  int page_base = -(1 << 30);
-  auto page_of = [&](int idx) -> int {  // idx is wave-uniform
-    if (idx < page_base || idx - page_base >= MI_WAVE) {
-      page_base = idx;
-      const int j = idx + lane;
-      page_vec = (j < max_blocks) ? bt[j] : 0;
-    }
-    return __builtin_amdgcn_readlane(page_vec, idx - page_base);
+  // Page ids are read with SCALAR loads (the key block number is wave-uniform and the
+  // block table is not written while the kernel runs) one block ahead of their use: they
+  // are counted apart from the vector loads, so waiting for a page id never waits for the
+  // keys and values in flight.
+  struct PageIds {
+    int page[2];  // of the two 16-key halves of a block
   };
+  auto fetch_pages = [&](int kb) -> PageIds {
+    PageIds ids;
+#pragma unroll
+    for (int hlf = 0; hlf < 2; ++hlf) {
+      // (past the table only for keys past the request's end, which are masked)
+      ids.page[hlf] = bt[min(page_index(kb + 16 * hlf), max_blocks - 1)];
+    }
+    return ids;
+  };
+  const int page_stride = kv_heads * page_size * D;  // elements from one page to the next
+  const int head_off = kvh * page_size * D;
   const unsigned k_lane_off = (unsigned)(col * D + quad * 8);
   const unsigned v_lane_off = (unsigned)(col * page_size + 4 * quad);
   auto load_values = [&](const bf16_t* const v_base[2], bf16x8_t* v) {
@@ -235,15 +256,14 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
       }
     }
   };
-  auto load_block = [&](int kb, KVBlock& blk) {
+  auto load_block = [&](int kb, const PageIds& ids, KVBlock& blk) {
     const bf16_t* k_base[2];
 #pragma unroll
     for (int hlf = 0; hlf < 2; ++hlf) {
       const int key0 = kb + 16 * hlf;
-      const int idx = key0 / page_size;
-      const int page = max(page_of(idx), 0);
-      const int64_t chunk_off = ((int64_t)page * kv_heads + kvh) * page_size * D;
-      const int slot0 = key0 % page_size;
+      const int page = max(ids.page[hlf], 0);
+      const int64_t chunk_off = (int64_t)page * page_stride + head_off;
+      const int slot0 = key0 - page_index(key0) * page_size;
       k_base[hlf] = k_pages + chunk_off + (int64_t)slot0 * D;
       blk.v_base[hlf] = vt_pages + chunk_off + slot0;
     }
@@ -259,12 +279,8 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   // The three phases run over all row groups of the wave in turn (scores for every
   // group, then every group's softmax, then every group's value product): the groups
   // are independent, so one group's vector work overlaps another's matrix work.
-  auto compute_block = [&](int kb, KVBlock& blk) {
-    bf16x8_t v_late[VPF ? 1 : DBLOCKS];
-    if (!VPF) load_values(blk.v_base, v_late);  // in flight during the scores and the softmax
-    const bf16x8_t* v_op = VPF ? blk.v : v_late;
-    // ---- S^T = K . Q^T for 32 keys ------------------------------------------------
-    f32x4_t s_acc[RG][2];
+  // ---- S^T = K . Q^T for 32 keys ------------------------------------------------
+  auto block_scores = [&](const KVBlock& blk, f32x4_t (&s_acc)[RG][2]) {
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) {
 #pragma unroll
@@ -276,11 +292,15 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
         s_acc[rg][hlf] = acc;
       }
     }
-    // ---- scale, mask, online softmax (lane holds keys kb + 16*hlf + 4*quad + r) -----
+  };
+  // ---- scale, mask, online softmax (lane holds keys kb + 16*hlf + 4*quad + r) -----
+  // Leaves the probabilities in p_reg (already the B operand of the value product) and
+  // the factor the old accumulator must be multiplied with in alpha; returns whether any
+  // row of the wave needs that multiplication (alpha != 1 somewhere).
+  auto block_softmax = [&](int kb, f32x4_t (&s_acc)[RG][2], bf16x8_t (&p_reg)[RG], float (&alpha)[RG]) -> bool {
     // a block every row of this wave sees whole needs no mask (most blocks of a long prompt)
     const bool interior = kb >= wave_lo_max && kb + 31 <= wave_pos_min && kb >= k_begin && kb + 32 <= k_end;
-    bf16x8_t p_reg[RG];
-    float alpha[RG];
+    bool moved = false;
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) {
       float sc[8];
@@ -310,8 +330,10 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
       // probabilities stay below 2^RESCALE_SLACK and the accumulator is rarely rescaled.
       const float m_new = (mx > m_run[rg] + RESCALE_SLACK) ? mx : m_run[rg];
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen nothing yet
+      // A row's first visible block moves the reference from -inf; its sum and accumulator
+      // are still zero, so nothing is to be rescaled (alpha 1, not exp2(-inf)).
       // arguments are bounded above: the hardware exp2 is exact enough, tiny results flush to 0
-      alpha[rg] = __builtin_amdgcn_exp2f(m_run[rg] - m_safe);  // 0 on the first visible block
+      alpha[rg] = (m_run[rg] == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[rg] - m_safe);
       float sum = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -322,43 +344,109 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
       sum = quad_sum(sum);
       l_run[rg] = l_run[rg] * alpha[rg] + sum;
       m_run[rg] = m_new;
+      moved = moved || (__ballot(alpha[rg] != 1.f) != 0ull);
     }
-    // ---- O^T = O^T * alpha + V^T . P^T ------------------------------------------------
+    return moved;
+  };
+  // ---- O^T *= alpha (only where block_softmax said so) ---------------------------------
+  auto rescale = [&](const float (&alpha)[RG]) {
 #pragma unroll
-    for (int rg = 0; rg < RG; ++rg) {
-      // alpha is 1 in every lane unless some row's reference point moved
-      // (one branch around the whole rescale, so that it is not turned into selects)
-      if (__ballot(alpha[rg] != 1.f) != 0ull) {
+    for (int rg = 0; rg < RG; ++rg)
 #pragma unroll
-        for (int db = 0; db < DBLOCKS; ++db)
+      for (int db = 0; db < DBLOCKS; ++db)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o_acc[rg][db][r] *= alpha[rg];
-      }
+        for (int r = 0; r < 4; ++r) o_acc[rg][db][r] *= alpha[rg];
+  };
+  // ---- O^T += V^T . P^T ------------------------------------------------------------------
+  auto block_values = [&](const bf16x8_t* v_op, const bf16x8_t (&p_reg)[RG]) {
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg)
 #pragma unroll
       for (int db = 0; db < DBLOCKS; ++db)
         o_acc[rg][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op[db], p_reg[rg], o_acc[rg][db], 0, 0, 0);
-    }
+  };
+  auto compute_block = [&](int kb, KVBlock& blk) {
+    bf16x8_t v_late[VPF ? 1 : DBLOCKS];
+    if (!VPF) load_values(blk.v_base, v_late);  // in flight during the scores and the softmax
+    f32x4_t s_acc[RG][2];
+    block_scores(blk, s_acc);
+    bf16x8_t p_reg[RG];
+    float alpha[RG];
+    // (one branch around the whole rescale, so that it is not turned into selects)
+    if (block_softmax(kb, s_acc, p_reg, alpha)) rescale(alpha);
+    block_values(VPF ? blk.v : v_late, p_reg);
   };
 
   // Software pipeline: the loads of the next block are in flight while this one is
   // computed (two register sets, the loop advances two blocks a turn).
-  {
+  constexpr int STEP = 32 * KW;
+  if constexpr (ONE_SET) {
+    // One register set: the values of a block are requested when its turn starts and
+    // used at its end; the keys of the NEXT block are requested as soon as the score
+    // products have consumed this block's.  Each load has over half a turn to arrive,
+    // and the registers saved keep the whole state out of the accumulation file.
+    static_assert(!VPF, "one register set loads values at the start of their block");
+    KVBlock blk;
+    int kb = (k_begin / 32) * 32 + 32 * key_wave;
+    if (kb < k_end) {
+      const int kb_last = kb + (k_end - 1 - kb) / STEP * STEP;
+      load_block(kb, fetch_pages(kb), blk);
+      PageIds ids_next = fetch_pages(min(kb + STEP, kb_last));
+      // Two loops in each other: the inner one runs while no row's reference point moves
+      // and touches the accumulator with matrix instructions only, so it stays in the
+      // accumulation registers; a block that moves a reference leaves the inner loop, has
+      // the accumulator rescaled out here, and the inner loop is entered again.
+      bf16x8_t v_now[DBLOCKS];
+      bf16x8_t p_reg[RG];
+      float alpha[RG];
+      bool more = true;
+      while (more) {
+        bool moved = false;
+        while (true) {
+          load_values(blk.v_base, v_now);
+          f32x4_t s_acc[RG][2];
+          block_scores(blk, s_acc);
+          __builtin_amdgcn_sched_barrier(0);
+          load_block(min(kb + STEP, kb_last), ids_next, blk);  // past the end: re-reads the last block
+          ids_next = fetch_pages(min(kb + 2 * STEP, kb_last));
+          __builtin_amdgcn_sched_barrier(0);
+          moved = block_softmax(kb, s_acc, p_reg, alpha);
+          if (moved) break;
+          block_values(v_now, p_reg);
+          __builtin_amdgcn_sched_barrier(0);
+          kb += STEP;
+          if (kb >= k_end) {
+            more = false;
+            break;
+          }
+        }
+        if (moved) {
+          rescale(alpha);
+          block_values(v_now, p_reg);
+          kb += STEP;
+          more = kb < k_end;
+        }
+      }
+    }
+  } else {
     // The prefetch is unconditional (past the end it re-reads this wave's last block),
     // so the compiler can count outstanding loads exactly instead of draining them all.
-    constexpr int STEP = 32 * KW;
     KVBlock blk_a, blk_b;
     int kb = (k_begin / 32) * 32 + 32 * key_wave;
     if (kb < k_end) {
       const int kb_last = kb + (k_end - 1 - kb) / STEP * STEP;
-      load_block(kb, blk_a);
+      load_block(kb, fetch_pages(kb), blk_a);
+      PageIds ids_next = fetch_pages(min(kb + STEP, kb_last));
       while (true) {
-        load_block(min(kb + STEP, kb_last), blk_b);
+        load_block(min(kb + STEP, kb_last), ids_next, blk_b);
+        ids_next = fetch_pages(min(kb + 2 * STEP, kb_last));
         __builtin_amdgcn_sched_barrier(0);
         compute_block(kb, blk_a);
         __builtin_amdgcn_sched_barrier(0);
         kb += STEP;
         if (kb >= k_end) break;
-        load_block(min(kb + STEP, kb_last), blk_a);
+        load_block(min(kb + STEP, kb_last), ids_next, blk_a);
+        ids_next = fetch_pages(min(kb + 2 * STEP, kb_last));
         __builtin_amdgcn_sched_barrier(0);
         compute_block(kb, blk_b);
         __builtin_amdgcn_sched_barrier(0);
@@ -440,8 +528,9 @@ extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, 
 static int heads_per_block_for(int group, int rows) { return group < rows ? group : rows; }
 
 // Tiling the Python side needs to size the grid: tokens per tile for a group size.
+#define MI_PREFILL_WAVES 4  // waves per block in the prefill shape
 #define MI_PREFILL_RG 2  // row groups (of 16 rows) per wave in the prefill shape
-#define MI_PREFILL_ROWS (64 * MI_PREFILL_RG)
+#define MI_PREFILL_ROWS (16 * MI_PREFILL_WAVES * MI_PREFILL_RG)
 
 extern "C" int mi_attn_mfma_tokens_per_tile(int q_heads, int kv_heads, int decode_only) {
   if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return 0;
@@ -496,19 +585,31 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
   const int hb = heads_per_block_for(group, rows);
   const int tq = mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, decode_only);
   const int head_blocks = ceil_div(group, hb);
-  MI_REQUIRE(kv_heads * head_blocks <= 65535, "attn_mfma: too many heads");
-  dim3 grid(num_tiles, kv_heads * head_blocks, num_splits);
+  MI_REQUIRE((int64_t)num_tiles * kv_heads * head_blocks < (1ll << 31), "attn_mfma: too many tiles x heads");
+  MI_REQUIRE(num_splits <= 65535, "attn_mfma: too many splits");
+  dim3 grid((unsigned)(num_tiles * kv_heads * head_blocks), 1, num_splits);
   const float scale_log2 = scale * LOG2E;
+  // keys reach max_blocks*page_size + 32 at most; the multiply-high division is exact below 2^32/page_size
+  MI_REQUIRE(((int64_t)max_blocks * page_size + 64) * page_size < (1ll << 32),
+             "attn_mfma: block table of %d pages of %d is too long for this kernel", max_blocks, page_size);
+  const unsigned page_magic = (unsigned)((1ull << 32) / (unsigned)page_size) + 1u;
 
-#define MI_LAUNCH(DD, WW, KK, RR, VV, OO)                                                         \
-  attn_mfma_kernel<DD, WW, KK, RR, VV, OO><<<grid, 64 * WW * KK, 0, stream>>>(                    \
+#define MI_LAUNCH(DD, WW, KK, RR, VV, OO, SS, PP)                                                 \
+  attn_mfma_kernel<DD, WW, KK, RR, VV, OO, SS, PP><<<grid, 64 * WW * KK, 0, stream>>>(                    \
       (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)vt_pages,            \
       block_table, max_blocks, cu_seqlens_q, positions, num_requests, (bf16_t*)out,               \
-      out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, scale_log2, window,        \
+      out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, page_magic, scale_log2,    \
+      window,                                                                                     \
       num_splits, hb, tq, one_tile_per_request)
-#define MI_LAUNCH_D(DD)            \
-  if (decode_only) MI_LAUNCH(DD, 1, 4, 1, false, 2); \
-  else MI_LAUNCH(DD, 4, 1, MI_PREFILL_RG, false, 1)
+#define MI_LAUNCH_P(DD, PP)                                              \
+  if (decode_only) MI_LAUNCH(DD, 1, 4, 1, false, 2, false, PP);          \
+  else MI_LAUNCH(DD, MI_PREFILL_WAVES, 1, MI_PREFILL_RG, false, 1, true, PP)
+#define MI_LAUNCH_D(DD)                 \
+  if (page_size == 16) {                \
+    MI_LAUNCH_P(DD, 16);                \
+  } else {                              \
+    MI_LAUNCH_P(DD, 0);                 \
+  }
   switch (head_dim) {
     case 32: MI_LAUNCH_D(32); break;
     case 64: MI_LAUNCH_D(64); break;
@@ -518,6 +619,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
     default: MI_LAUNCH_D(256); break;
   }
 #undef MI_LAUNCH_D
+#undef MI_LAUNCH_P
 #undef MI_LAUNCH
   MI_CHECK_LAUNCH("attn_mfma");
   if (num_splits > 1)
