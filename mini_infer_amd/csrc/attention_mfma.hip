@@ -528,6 +528,7 @@ extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, 
 static int heads_per_block_for(int group, int rows) { return group < rows ? group : rows; }
 
 // Tiling the Python side needs to size the grid: tokens per tile for a group size.
+#define MI_DECODE_KW 4  // waves that share a decode block's rows, each taking every KW-th key block
 #define MI_PREFILL_WAVES 4  // waves per block in the prefill shape
 #define MI_PREFILL_RG 2  // row groups (of 16 rows) per wave in the prefill shape
 #define MI_PREFILL_ROWS (16 * MI_PREFILL_WAVES * MI_PREFILL_RG)
@@ -602,7 +603,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
       window,                                                                                     \
       num_splits, hb, tq, one_tile_per_request)
 #define MI_LAUNCH_P(DD, PP)                                              \
-  if (decode_only) MI_LAUNCH(DD, 1, 4, 1, false, 2, false, PP);          \
+  if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, false, 2, false, PP); \
   else MI_LAUNCH(DD, MI_PREFILL_WAVES, 1, MI_PREFILL_RG, false, 1, true, PP)
 #define MI_LAUNCH_D(DD)                 \
   if (page_size == 16) {                \

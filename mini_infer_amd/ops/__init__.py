@@ -6,6 +6,7 @@ from mini_infer_amd.ops.kernels import (
     embed_gather,
     gemm_f32,
     gemm_skinny_bf16,
+    linear_swiglu,
     linear,
     mfma_attention_supported,
     paged_attention,
@@ -21,6 +22,7 @@ __all__ = [
     "embed_gather",
     "gemm_f32",
     "gemm_skinny_bf16",
+    "linear_swiglu",
     "linear",
     "mfma_attention_supported",
     "paged_attention",

@@ -297,6 +297,40 @@ def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return torch.matmul(x, weight.t())
 
 
+def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+    """`silu(x @ gate.T) * (x @ up.T)` with `gate_up_weight` = [gate; up] stacked, [2I, K].
+
+    bfloat16 with at most 16 rows runs as ONE hand-written kernel (the product with the
+    activation in its last step); otherwise the product and `silu_mul` run in turn.
+    Both ways round the two products to the element type before the activation, so a
+    token's result does not depend on which one ran.
+    """
+    rows, width = gate_up_weight.shape
+    if rows % 2:
+        raise KernelShapeError(f"linear_swiglu: stacked weight has an odd number of rows ({rows})")
+    if (
+        x.dtype == torch.bfloat16
+        and gate_up_weight.dtype == torch.bfloat16
+        and x.dim() == 2
+        and x.shape[1] == width
+        and x.stride(1) == 1
+        and gate_up_weight.stride(1) == 1
+        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), gate_up_weight.stride(0))
+    ):
+        _need_cuda(x, gate_up_weight)
+        m, n = x.shape[0], rows // 2
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+        lib = library.load()
+        library.check(
+            lib.mi_gemm_skinny_swiglu_bf16(
+                _ptr(x), x.stride(0), _ptr(gate_up_weight), gate_up_weight.stride(0), _ptr(out), out.stride(0),
+                m, n, width, _stream(),
+            )
+        )
+        return out
+    return silu_mul(linear(x, gate_up_weight))
+
+
 def attention_splits(work_items: int, max_seq_len: int, target: int = 2048, min_keys: int = 256) -> int:
     """How many key ranges each work item is cut into so that the GPU is full.
 

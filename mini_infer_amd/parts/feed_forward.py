@@ -2,8 +2,9 @@
 
 Formula: models/blocks/swiglu.py:44-46 and activations.py:36-45 of the
 reference.  Gate and up are two tensors in the checkpoint; they are stacked at
-load so one product yields [gate | up], and the activation kernel reads both
-halves (the reference runs two products and one fused SiLU*mul kernel).
+load so one product yields [gate | up], and the activation reads both halves
+(the reference runs two products and one fused SiLU*mul kernel); for few rows
+the product and the activation are one kernel.
 """
 
 from __future__ import annotations
@@ -36,7 +37,8 @@ class SwiGLU(FeedForward):
         self.down.load_params(prefix, get)
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        return self.down.forward(ops.silu_mul(self.gate_up.forward(x)))
+        assert self.gate_up.weight is not None, "SwiGLU used before its weights were loaded"
+        return self.down.forward(ops.linear_swiglu(x, self.gate_up.weight))
 
 
 @register_feed_forward("swiglu")

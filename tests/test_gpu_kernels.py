@@ -125,6 +125,33 @@ def test_gemm_skinny_bf16(m, n, k):
     assert torch.equal(ops.linear(a, w), out)
 
 
+@pytest.mark.parametrize(
+    "m,inter,k",
+    [(1, 14336, 4096), (8, 14336, 4096), (16, 160, 64), (7, 301, 96), (13, 4100, 160), (3, 5, 32), (9, 8192, 3072)],
+)
+def test_linear_swiglu_is_the_product_followed_by_the_activation(m, inter, k):
+    from mini_infer_amd import ops
+
+    a = _rand(m, k, dtype=torch.bfloat16, seed=12)
+    w = _rand(2 * inter, k, dtype=torch.bfloat16, seed=13, scale=0.08)
+    fused = ops.linear_swiglu(a, w)
+    assert fused.shape == (m, inter)
+    # the two-kernel path: the product (rounded to bfloat16), then the activation
+    assert torch.equal(fused, ops.silu_mul(ops.gemm_skinny_bf16(a, w)))
+    gate_up = (a.double() @ w.double().T).bfloat16().double()
+    gate, up = gate_up[:, :inter], gate_up[:, inter:]
+    expected = gate / (1 + torch.exp(-gate)) * up
+    assert (fused.double() - expected).abs().max() < 2.0 ** -7 * float(expected.abs().max()) + 1e-6
+    # more rows than the fused kernel takes: the same function, through the library product
+    many = _rand(40, k, dtype=torch.bfloat16, seed=14)
+    assert ops.linear_swiglu(many, w).shape == (40, inter)
+    # float32 goes through the true float32 product
+    got32 = ops.linear_swiglu(a.float(), w.float())
+    exact = a.double() @ w.double().T
+    exact = exact[:, :inter] / (1 + torch.exp(-exact[:, :inter])) * exact[:, inter:]
+    assert (got32.double() - exact).abs().max() < 1e-4 * float(exact.abs().max()) + 1e-6
+
+
 def test_linear_falls_back_to_the_library_where_the_skinny_kernel_does_not_apply():
     from mini_infer_amd import ops
     from mini_infer_amd.exceptions import KernelShapeError
