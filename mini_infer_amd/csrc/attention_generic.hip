@@ -172,13 +172,27 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
   float l_all = 0.f;
   for (int s = 0; s < num_splits; ++s) l_all += __shfl(l_s * w_s, s, MI_WAVE);
   const float inv = 1.f / l_all;
+  // The partial accumulators are read in batches of independent loads (a load per split
+  // issued one after the other's use would cost a memory latency per split) and added in
+  // split order.
+  constexpr int BATCH = 8;
   for (int d0 = 0; d0 < head_dim; d0 += MI_WAVE) {  // all lanes stay in the loop for the shuffles
     const int d = d0 + lane;
     const bool active = d < head_dim;
+    const float* src = part_acc + base * head_dim + (active ? d : 0);
     float o = 0.f;
-    for (int s = 0; s < num_splits; ++s) {
-      const float w = __shfl(w_s, s, MI_WAVE);
-      if (active) o += part_acc[(base + s) * head_dim + d] * w;
+    for (int s0 = 0; s0 < num_splits; s0 += BATCH) {
+      float v[BATCH];
+#pragma unroll
+      for (int i = 0; i < BATCH; ++i) {
+        const int sp = min(s0 + i, num_splits - 1);  // past the end: re-read the last split, weight 0 below
+        v[i] = src[(int64_t)sp * head_dim];
+      }
+#pragma unroll
+      for (int i = 0; i < BATCH; ++i) {
+        const float w = __shfl(w_s, min(s0 + i, MI_WAVE - 1), MI_WAVE);
+        if (s0 + i < num_splits) o += v[i] * w;
+      }
     }
     if (active) out[(int64_t)t * out_row_stride + (int64_t)h * head_dim + d] = from_f32<T>(o * inv);
   }

@@ -91,7 +91,15 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   const int grid_head = (int)(blockIdx.x % (unsigned)head_slots);
   const int grid_tiles = (int)(gridDim.x / (unsigned)head_slots);
   int req = -1, t0 = 0, n_tok = 0;
-  if (one_tile_per_request) {
+  if (one_tile_per_request == 2) {
+    // every request brings exactly one token (a decode step): token b belongs to request b,
+    // and nothing has to be read to know it
+    if (grid_tile < num_requests) {
+      req = grid_tile;
+      t0 = req;
+      n_tok = 1;
+    }
+  } else if (one_tile_per_request) {
     if (grid_tile < num_requests) {
       req = grid_tile;
       t0 = cu_seqlens_q[req];
@@ -549,8 +557,9 @@ extern "C" int mi_attn_mfma_supported(int head_dim, int page_size) {
 
 // `num_tiles` = sum over requests of ceil(q_len / tokens_per_tile), computed by the
 // caller from the host copy of cu_seqlens_q (a larger number is harmless).
-// `one_tile_per_request` promises that no request has more than tokens_per_tile
-// tokens in this step; then num_tiles must be num_requests.
+// `one_tile_per_request` = 1 promises that no request has more than tokens_per_tile
+// tokens in this step, 2 that every request has exactly one (then cu_seqlens_q is not
+// read); in both cases num_tiles must be num_requests.
 // With num_splits > 1, part_acc holds num_tokens*q_heads*num_splits*head_dim floats
 // and part_ml num_tokens*q_heads*num_splits*2.
 extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_pages,
@@ -577,6 +586,9 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
              "attn_mfma: row strides shorter than q_heads*head_dim");
   MI_REQUIRE(q_row_stride % 8 == 0 && out_row_stride % 4 == 0,
              "attn_mfma: row strides must keep 16-byte (q) and 8-byte (out) alignment");
+  MI_REQUIRE(one_tile_per_request >= 0 && one_tile_per_request <= 2, "attn_mfma: one_tile_per_request is 0, 1 or 2");
+  MI_REQUIRE(one_tile_per_request != 2 || num_tokens == num_requests,
+             "attn_mfma: one token per request needs num_tokens == num_requests");
   MI_REQUIRE(!one_tile_per_request || num_tiles == num_requests,
              "attn_mfma: one tile per request needs num_tiles == num_requests");
   if (num_tokens == 0 || num_tiles == 0) return MI_OK;

@@ -423,7 +423,8 @@ def paged_attention(
         q_lens = [host_cu_seqlens_q[b + 1] - host_cu_seqlens_q[b] for b in range(num_requests)]
         decode_only = max(q_lens) <= 1
         tokens_per_tile = lib.mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, int(decode_only))
-        one_tile_per_request = max(q_lens) <= tokens_per_tile
+        # 2: exactly one token per request (the kernel then needs no request boundaries)
+        one_tile_per_request = 2 if (decode_only and min(q_lens) == 1) else int(max(q_lens) <= tokens_per_tile)
         num_tiles = num_requests if one_tile_per_request else sum(-(-n // tokens_per_tile) for n in q_lens)
         rows = 16 if decode_only else 128
         head_blocks = -(-group // min(group, rows))
