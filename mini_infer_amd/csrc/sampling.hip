@@ -20,6 +20,7 @@
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_WAVES (SAMPLE_THREADS / MI_WAVE)
+#define SAMPLE_BATCH 16  // loads a thread has in flight
 #define MASS_ONE 1099511627776.0f  // 2^40
 
 __device__ __forceinline__ uint32_t order_key(float x) {
@@ -96,10 +97,21 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const float temp = temperature[row];
 
   if (temp == 0.f) {
+    // a thread's elements in batches of independent loads (one load per turn would cost a
+    // memory latency per element), visited in rising index order: ties go to the first
     ArgBest mine = {-INFINITY, 0x7fffffff};
-    for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
-      const float v = to_f32(x[i]);
-      if (v > mine.val || mine.idx == 0x7fffffff) { mine.val = v; mine.idx = i; }
+    for (int i0 = tid; i0 < vocab; i0 += SAMPLE_THREADS * SAMPLE_BATCH) {
+      float v[SAMPLE_BATCH];
+#pragma unroll
+      for (int u = 0; u < SAMPLE_BATCH; ++u) {
+        const int i = i0 + u * SAMPLE_THREADS;
+        v[u] = (i < vocab) ? to_f32(x[i]) : -INFINITY;
+      }
+#pragma unroll
+      for (int u = 0; u < SAMPLE_BATCH; ++u) {
+        const int i = i0 + u * SAMPLE_THREADS;
+        if (i < vocab && (v[u] > mine.val || mine.idx == 0x7fffffff)) { mine.val = v[u]; mine.idx = i; }
+      }
     }
     const ArgBest best = block_argbest(mine, best_scratch);
     if (tid == 0) out[row] = best.idx;
@@ -108,9 +120,18 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
   // maximum of the scaled logits
   ArgBest top = {-INFINITY, 0x7fffffff};
-  for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
-    const float v = to_f32(x[i]) / temp;
-    if (v > top.val) { top.val = v; top.idx = i; }
+  for (int i0 = tid; i0 < vocab; i0 += SAMPLE_THREADS * SAMPLE_BATCH) {
+    float v[SAMPLE_BATCH];
+#pragma unroll
+    for (int u = 0; u < SAMPLE_BATCH; ++u) {
+      const int i = i0 + u * SAMPLE_THREADS;
+      v[u] = (i < vocab) ? to_f32(x[i]) / temp : -INFINITY;
+    }
+#pragma unroll
+    for (int u = 0; u < SAMPLE_BATCH; ++u) {
+      const int i = i0 + u * SAMPLE_THREADS;
+      if (v[u] > top.val) { top.val = v[u]; top.idx = i; }
+    }
   }
   const float v_max = block_argbest(top, best_scratch).val;
 
