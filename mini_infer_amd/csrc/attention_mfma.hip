@@ -57,14 +57,15 @@ __device__ __forceinline__ float quad_sum(float v) {
 // VPF: value operands are prefetched a block ahead like the keys (more registers), or
 // loaded at the start of the block that uses them (fewer registers, so OCC waves of
 // different blocks can share a SIMD and fill each other's stalls).
-template <int D, int WAVES, int KW, int RG, bool VPF, int OCC, bool ONE_SET, int PS>
+template <int D, int WAVES, int KW, int RG, bool VPF, int OCC, int PIPE, int PS>
 __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_row_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ cu_seqlens_q, const int* __restrict__ positions, int num_requests,
     bf16_t* __restrict__ out, int64_t out_row_stride, float* __restrict__ part_acc,
     float* __restrict__ part_ml, int q_heads, int kv_heads, int page_size_arg, unsigned page_magic, float scale_log2,
-    int window, int num_splits, int heads_per_block, int tokens_per_tile, int one_tile_per_request) {
+    int window, int num_splits, int heads_per_block, int tokens_per_tile, int one_tile_per_request,
+    int pair_group) {
   constexpr int KSTEPS = D / 32;  // MFMA k-steps over the head dim for S^T
   // PS != 0: the page size is this constant (divisions become shifts, value offsets
   // immediates); PS == 0: any multiple of 16, divided by multiplying with
@@ -108,7 +109,16 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   } else {
     // Tiles are handed out last first: under the causal mask a request's later tiles
     // have more keys, and starting the long ones first keeps the GPU's tail short.
-    const int tile_index = grid_tiles - 1 - grid_tile;
+    // With two blocks resident per CU the first 2*pair_group tiles an XCD receives start at
+    // once, CU i taking the i-th and the (pair_group+i)-th: the longest pair_group tiles
+    // are followed by the SHORTEST ones in rising order, so that every CU's pair has the
+    // same sum; the rest follow longest first as CUs come free.  (pair_group 0: plain
+    // longest-first order.  Only the running time depends on this guess at the dispatcher.)
+    int tile_index = grid_tiles - 1 - grid_tile;
+    if (pair_group > 0 && grid_tiles >= 2 * pair_group) {
+      if (grid_tile >= pair_group && grid_tile < 2 * pair_group) tile_index = grid_tile - pair_group;
+      else if (grid_tile >= 2 * pair_group) tile_index = grid_tiles - 1 - (grid_tile - pair_group);
+    }
     const int search_lane = threadIdx.x % MI_WAVE;
     int tiles_before = 0;
     for (int b0 = 0; b0 < num_requests && req < 0; b0 += MI_WAVE) {
@@ -157,8 +167,9 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   const int col = lane % 16;  // this lane's row of work within a row group
   const int quad = lane / 16;  // 0..3
 
-  // a wave whose rows are all padding has nothing to do
-  if (KW == 1 && wave * 16 * RG >= n_tok * heads_per_block) return;
+  // a wave whose rows are all padding has nothing to do (unless the block's waves load
+  // the keys and values together: then it stays for the loads and the barriers)
+  if (KW == 1 && PIPE != 2 && wave * 16 * RG >= n_tok * heads_per_block) return;
 
   const int pos0 = positions[t0];  // tokens of a tile sit at consecutive positions
   int token[RG], head[RG], pos[RG], lo_row[RG];
@@ -388,7 +399,143 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   // Software pipeline: the loads of the next block are in flight while this one is
   // computed (two register sets, the loop advances two blocks a turn).
   constexpr int STEP = 32 * KW;
-  if constexpr (ONE_SET) {
+  if constexpr (PIPE == 2) {
+    // The block's waves load each 32-key tile TOGETHER (every byte leaves the cache
+    // hierarchy once per block instead of once per wave: with 4 waves a quarter of the
+    // vector-memory traffic) into LDS, two tiles deep: while a tile is computed from one
+    // buffer, the next one's global loads are in flight in a few staging registers and
+    // are written to the other buffer at the end of the turn; one barrier per turn.
+    // Key rows are padded by 16 bytes and value rows by 8 so that the operand reads of
+    // 16 lanes fall into different banks.
+    static_assert(KW == 1 && !VPF, "shared tiles are for blocks whose waves walk the same keys");
+    constexpr int THREADS = 64 * WAVES;
+    constexpr int CPR = D / 8;  // 16-byte chunks per key row
+    constexpr int KROW = D + 8;  // elements
+    constexpr int VROW = 32 + 4;
+    constexpr int K_CHUNKS = 32 * CPR, V_CHUNKS = 4 * D;
+    constexpr int K_PER = (K_CHUNKS + THREADS - 1) / THREADS, V_PER = (V_CHUNKS + THREADS - 1) / THREADS;
+    __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][32 * KROW];
+    __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][D * VROW];
+    const int tid = threadIdx.x;
+    bf16x8_t k_stage[K_PER], v_stage[V_PER];
+    auto request_tile = [&](int kb, const PageIds& ids) {
+      const bf16_t* k_base[2];
+      const bf16_t* v_base[2];
+#pragma unroll
+      for (int hlf = 0; hlf < 2; ++hlf) {
+        const int key0 = kb + 16 * hlf;
+        const int page = max(ids.page[hlf], 0);
+        const int64_t chunk_off = (int64_t)page * page_stride + head_off;
+        const int slot0 = key0 - page_index(key0) * page_size;
+        k_base[hlf] = k_pages + chunk_off + (int64_t)slot0 * D;
+        v_base[hlf] = vt_pages + chunk_off + slot0;
+      }
+#pragma unroll
+      for (int j = 0; j < K_PER; ++j) {
+        const int id = tid + j * THREADS;
+        if (K_CHUNKS % THREADS == 0 || id < K_CHUNKS) {
+          const int key = id / CPR, part = id % CPR;
+          k_stage[j] = *reinterpret_cast<const bf16x8_t*>(k_base[key / 16] + (key % 16) * D + part * 8);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < V_PER; ++j) {
+        const int id = tid + j * THREADS;
+        if (V_CHUNKS % THREADS == 0 || id < V_CHUNKS) {
+          const int hlf = id / (2 * D), dim = (id % (2 * D)) / 2, part = id % 2;
+          v_stage[j] = *reinterpret_cast<const bf16x8_t*>(v_base[hlf] + dim * page_size + part * 8);
+        }
+      }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+      for (int j = 0; j < K_PER; ++j) {
+        const int id = tid + j * THREADS;
+        if (K_CHUNKS % THREADS == 0 || id < K_CHUNKS) {
+          const int key = id / CPR, part = id % CPR;
+          *reinterpret_cast<bf16x8_t*>(&k_lds[buf][key * KROW + part * 8]) = k_stage[j];
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < V_PER; ++j) {
+        const int id = tid + j * THREADS;
+        if (V_CHUNKS % THREADS == 0 || id < V_CHUNKS) {
+          const int hlf = id / (2 * D), dim = (id % (2 * D)) / 2, part = id % 2;
+          bf16x4_t lo, hi;  // rows are 8-byte aligned only: two 8-byte stores
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            lo[i] = v_stage[j][i];
+            hi[i] = v_stage[j][4 + i];
+          }
+          bf16_t* dst = &v_lds[buf][dim * VROW + hlf * 16 + part * 8];
+          *reinterpret_cast<bf16x4_t*>(dst) = lo;
+          *reinterpret_cast<bf16x4_t*>(dst + 4) = hi;
+        }
+      }
+    };
+    auto read_operands = [&](int buf, KVBlock& blk, bf16x8_t* v) {
+#pragma unroll
+      for (int hlf = 0; hlf < 2; ++hlf)
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+          blk.k[hlf][s] = *reinterpret_cast<const bf16x8_t*>(&k_lds[buf][(16 * hlf + col) * KROW + quad * 8 + s * 32]);
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db) {
+        const bf16_t* src = &v_lds[buf][(db * 16 + col) * VROW + 4 * quad];
+        const bf16x4_t v0 = *reinterpret_cast<const bf16x4_t*>(src);
+        const bf16x4_t v1 = *reinterpret_cast<const bf16x4_t*>(src + 16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[db][i] = v0[i];
+          v[db][4 + i] = v1[i];
+        }
+      }
+    };
+    KVBlock blk;
+    int kb = (k_begin / 32) * 32;
+    if (kb < k_end) {  // the same for every wave of the block
+      const int kb_last = kb + (k_end - 1 - kb) / 32 * 32;
+      request_tile(kb, fetch_pages(kb));
+      PageIds ids_next = fetch_pages(min(kb + 32, kb_last));
+      store_tile(0);
+      __syncthreads();
+      int buf = 0;
+      bf16x8_t v_now[DBLOCKS];
+      bf16x8_t p_reg[RG];
+      float alpha[RG];
+      bool more = true;
+      while (more) {  // nested as in the one-set pipeline: the inner loop never multiplies the accumulator
+        bool moved = false;
+        while (true) {
+          request_tile(min(kb + 32, kb_last), ids_next);  // past the end: re-reads the last tile
+          ids_next = fetch_pages(min(kb + 64, kb_last));
+          read_operands(buf, blk, v_now);
+          f32x4_t s_acc[RG][2];
+          block_scores(blk, s_acc);
+          moved = block_softmax(kb, s_acc, p_reg, alpha);
+          if (moved) break;
+          block_values(v_now, p_reg);
+          store_tile(buf ^ 1);
+          __syncthreads();
+          buf ^= 1;
+          kb += 32;
+          if (kb >= k_end) {
+            more = false;
+            break;
+          }
+        }
+        if (moved) {
+          rescale(alpha);
+          block_values(v_now, p_reg);
+          store_tile(buf ^ 1);
+          __syncthreads();
+          buf ^= 1;
+          kb += 32;
+          more = kb < k_end;
+        }
+      }
+    }
+  } else if constexpr (PIPE == 1) {
     // One register set: the values of a block are requested when its turn starts and
     // used at its end; the keys of the NEXT block are requested as soon as the score
     // products have consumed this block's.  Each load has over half a turn to arrive,
@@ -537,6 +684,8 @@ static int heads_per_block_for(int group, int rows) { return group < rows ? grou
 
 // Tiling the Python side needs to size the grid: tokens per tile for a group size.
 #define MI_DECODE_KW 4  // waves that share a decode block's rows, each taking every KW-th key block
+#define MI_PREFILL_PIPE 2  // 1: each wave loads its own operands; 2: the block's waves share tiles through LDS
+#define MI_PREFILL_OCC 2
 #define MI_PREFILL_WAVES 4  // waves per block in the prefill shape
 #define MI_PREFILL_RG 2  // row groups (of 16 rows) per wave in the prefill shape
 #define MI_PREFILL_ROWS (16 * MI_PREFILL_WAVES * MI_PREFILL_RG)
@@ -602,6 +751,14 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
   MI_REQUIRE(num_splits <= 65535, "attn_mfma: too many splits");
   dim3 grid((unsigned)(num_tiles * kv_heads * head_blocks), 1, num_splits);
   const float scale_log2 = scale * LOG2E;
+  // prefill blocks run two to a CU: see the tile order in the kernel (8 XCDs share the CUs evenly)
+  int pair_group = 0;
+  if (!decode_only && MI_PREFILL_OCC == 2) {
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) == hipSuccess &&
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess)
+      pair_group = cus / 8;
+  }
   // keys reach max_blocks*page_size + 32 at most; the multiply-high division is exact below 2^32/page_size
   MI_REQUIRE(((int64_t)max_blocks * page_size + 64) * page_size < (1ll << 32),
              "attn_mfma: block table of %d pages of %d is too long for this kernel", max_blocks, page_size);
@@ -613,10 +770,10 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
       block_table, max_blocks, cu_seqlens_q, positions, num_requests, (bf16_t*)out,               \
       out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, page_magic, scale_log2,    \
       window,                                                                                     \
-      num_splits, hb, tq, one_tile_per_request)
+      num_splits, hb, tq, one_tile_per_request, pair_group)
 #define MI_LAUNCH_P(DD, PP)                                              \
-  if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, false, 2, false, PP); \
-  else MI_LAUNCH(DD, MI_PREFILL_WAVES, 1, MI_PREFILL_RG, false, 1, true, PP)
+  if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, false, 2, 0, PP); \
+  else MI_LAUNCH(DD, MI_PREFILL_WAVES, 1, MI_PREFILL_RG, false, MI_PREFILL_OCC, MI_PREFILL_PIPE, PP)
 #define MI_LAUNCH_D(DD)                 \
   if (page_size == 16) {                \
     MI_LAUNCH_P(DD, 16);                \

@@ -428,9 +428,10 @@ def paged_attention(
         num_tiles = num_requests if one_tile_per_request else sum(-(-n // tokens_per_tile) for n in q_lens)
         rows = 16 if decode_only else 128
         head_blocks = -(-group // min(group, rows))
-        # the kernel's blocks are register-heavy (one per CU at a time): about one
-        # block per CU measured best at batch 1, 8 and 64 and for short portions
-        splits = min(16, attention_splits(num_tiles * kv_heads * head_blocks, max_seq_len, target=256, min_keys=128))
+        # decode blocks are register-heavy (about one per CU at a time measured best at batch
+        # 1, 8 and 64); prefill blocks run two to a CU
+        target = 256 if decode_only else 512
+        splits = min(16, attention_splits(num_tiles * kv_heads * head_blocks, max_seq_len, target=target, min_keys=128))
         part_acc, part_ml = partials(splits)
         library.check(
             lib.mi_attn_mfma(
