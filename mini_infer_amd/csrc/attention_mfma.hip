@@ -13,16 +13,19 @@
 //     O^T[dim, row] += V^T[dim, key] . P^T[key, row]
 // whose A operand wants, per lane, consecutive keys of one dim: the cache stores
 // values transposed inside each page ([page][head][dim][slot]) to make that a
-// contiguous load.  No LDS is used; waves of a block read the same keys and meet in
-// the cache hierarchy.
+// contiguous load.
 //
-// A block is `WAVES` row groups = 16*WAVES rows = one tile of consecutive tokens of
-// one request, times `heads_per_block` heads of one key/value group.  For decode
-// (one row group) `KW` waves share the rows, each taking every KW-th block of keys,
-// and merge through LDS: more waves in flight per byte of partial results.  Keys of
-// a tile may also be cut into `num_splits` ranges across blocks; those partial
-// (max, sum, accumulator) triples are combined by attn_reduce_kernel
-// (attention_generic.hip).
+// Two shapes of block:
+//  * decode (one token per request): 16 rows = one row group; `KW` waves share the rows,
+//    each taking every KW-th block of 32 keys straight from the pages into registers
+//    (two register sets: the next block's loads are in flight while this one is
+//    computed), and merge through LDS.  Keys may also be cut into `num_splits` ranges
+//    across blocks; those partial (max, sum, accumulator) triples are combined by
+//    attn_reduce_kernel (attention_generic.hip).
+//  * prefill: `WAVES` waves x `RG` row groups = 128 rows = one tile of consecutive
+//    tokens of one request, times `heads_per_block` heads of one key/value group.  The
+//    waves load each 32-key tile of keys and values TOGETHER into LDS (SHARED), two
+//    tiles deep, and read their matrix operands from there; two blocks run per CU.
 //
 // Semantics as in the reference's oracle (cache/packed_attention.py:296-338):
 // row at absolute position p sees keys 0..p, or p-window+1..p with a window.
@@ -54,10 +57,11 @@ __device__ __forceinline__ float quad_sum(float v) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-// VPF: value operands are prefetched a block ahead like the keys (more registers), or
-// loaded at the start of the block that uses them (fewer registers, so OCC waves of
-// different blocks can share a SIMD and fill each other's stalls).
-template <int D, int WAVES, int KW, int RG, bool VPF, int OCC, int PIPE, int PS>
+// VPF (register pipeline only): value operands are prefetched a block ahead like the
+// keys (more registers), or loaded at the start of the block that uses them (fewer
+// registers, so OCC waves of different blocks can share a SIMD and fill each other's
+// stalls).  SHARED: the block's waves load key and value tiles together through LDS.
+template <int D, int WAVES, int KW, int RG, bool VPF, int OCC, bool SHARED, int PS>
 __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_row_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table, int max_blocks,
@@ -169,7 +173,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
 
   // a wave whose rows are all padding has nothing to do (unless the block's waves load
   // the keys and values together: then it stays for the loads and the barriers)
-  if (KW == 1 && PIPE != 2 && wave * 16 * RG >= n_tok * heads_per_block) return;
+  if (KW == 1 && !SHARED && wave * 16 * RG >= n_tok * heads_per_block) return;
 
   const int pos0 = positions[t0];  // tokens of a tile sit at consecutive positions
   int token[RG], head[RG], pos[RG], lo_row[RG];
@@ -399,7 +403,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   // Software pipeline: the loads of the next block are in flight while this one is
   // computed (two register sets, the loop advances two blocks a turn).
   constexpr int STEP = 32 * KW;
-  if constexpr (PIPE == 2) {
+  if constexpr (SHARED) {
     // The block's waves load each 32-key tile TOGETHER (every byte leaves the cache
     // hierarchy once per block instead of once per wave: with 4 waves a quarter of the
     // vector-memory traffic) into LDS, two tiles deep: while a tile is computed from one
@@ -535,54 +539,6 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
         }
       }
     }
-  } else if constexpr (PIPE == 1) {
-    // One register set: the values of a block are requested when its turn starts and
-    // used at its end; the keys of the NEXT block are requested as soon as the score
-    // products have consumed this block's.  Each load has over half a turn to arrive,
-    // and the registers saved keep the whole state out of the accumulation file.
-    static_assert(!VPF, "one register set loads values at the start of their block");
-    KVBlock blk;
-    int kb = (k_begin / 32) * 32 + 32 * key_wave;
-    if (kb < k_end) {
-      const int kb_last = kb + (k_end - 1 - kb) / STEP * STEP;
-      load_block(kb, fetch_pages(kb), blk);
-      PageIds ids_next = fetch_pages(min(kb + STEP, kb_last));
-      // Two loops in each other: the inner one runs while no row's reference point moves
-      // and touches the accumulator with matrix instructions only, so it stays in the
-      // accumulation registers; a block that moves a reference leaves the inner loop, has
-      // the accumulator rescaled out here, and the inner loop is entered again.
-      bf16x8_t v_now[DBLOCKS];
-      bf16x8_t p_reg[RG];
-      float alpha[RG];
-      bool more = true;
-      while (more) {
-        bool moved = false;
-        while (true) {
-          load_values(blk.v_base, v_now);
-          f32x4_t s_acc[RG][2];
-          block_scores(blk, s_acc);
-          __builtin_amdgcn_sched_barrier(0);
-          load_block(min(kb + STEP, kb_last), ids_next, blk);  // past the end: re-reads the last block
-          ids_next = fetch_pages(min(kb + 2 * STEP, kb_last));
-          __builtin_amdgcn_sched_barrier(0);
-          moved = block_softmax(kb, s_acc, p_reg, alpha);
-          if (moved) break;
-          block_values(v_now, p_reg);
-          __builtin_amdgcn_sched_barrier(0);
-          kb += STEP;
-          if (kb >= k_end) {
-            more = false;
-            break;
-          }
-        }
-        if (moved) {
-          rescale(alpha);
-          block_values(v_now, p_reg);
-          kb += STEP;
-          more = kb < k_end;
-        }
-      }
-    }
   } else {
     // The prefetch is unconditional (past the end it re-reads this wave's last block),
     // so the compiler can count outstanding loads exactly instead of draining them all.
@@ -684,8 +640,8 @@ static int heads_per_block_for(int group, int rows) { return group < rows ? grou
 
 // Tiling the Python side needs to size the grid: tokens per tile for a group size.
 #define MI_DECODE_KW 4  // waves that share a decode block's rows, each taking every KW-th key block
-#define MI_PREFILL_PIPE 2  // 1: each wave loads its own operands; 2: the block's waves share tiles through LDS
-#define MI_PREFILL_OCC 2
+// prefill blocks per CU: two where a wave's state fits 256 registers without spilling
+#define MI_PREFILL_OCC(DD) ((DD) <= 128 ? 2 : 1)
 #define MI_PREFILL_WAVES 4  // waves per block in the prefill shape
 #define MI_PREFILL_RG 2  // row groups (of 16 rows) per wave in the prefill shape
 #define MI_PREFILL_ROWS (16 * MI_PREFILL_WAVES * MI_PREFILL_RG)
@@ -753,7 +709,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
   const float scale_log2 = scale * LOG2E;
   // prefill blocks run two to a CU: see the tile order in the kernel (8 XCDs share the CUs evenly)
   int pair_group = 0;
-  if (!decode_only && MI_PREFILL_OCC == 2) {
+  if (!decode_only && MI_PREFILL_OCC(head_dim) == 2) {
     int device = 0, cus = 0;
     if (hipGetDevice(&device) == hipSuccess &&
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess)
@@ -772,8 +728,8 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
       window,                                                                                     \
       num_splits, hb, tq, one_tile_per_request, pair_group)
 #define MI_LAUNCH_P(DD, PP)                                              \
-  if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, false, 2, 0, PP); \
-  else MI_LAUNCH(DD, MI_PREFILL_WAVES, 1, MI_PREFILL_RG, false, MI_PREFILL_OCC, MI_PREFILL_PIPE, PP)
+  if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, false, 2, false, PP); \
+  else MI_LAUNCH(DD, MI_PREFILL_WAVES, 1, MI_PREFILL_RG, false, MI_PREFILL_OCC(DD), true, PP)
 #define MI_LAUNCH_D(DD)                 \
   if (page_size == 16) {                \
     MI_LAUNCH_P(DD, 16);                \

@@ -362,6 +362,20 @@ def test_paged_attention_portion_over_long_context_splits_keys(mode, dtype):
     assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
 
 
+@pytest.mark.parametrize("window", [None, 700])
+def test_paged_attention_whole_long_prompts_many_tiles(window):
+    """Whole prompts of a few thousand tokens beside a short one: dozens of tiles per head,
+    more than fit on the GPU at once, so the order in which tiles are handed out (long and
+    short ones paired) and the tile-to-request search over several requests are exercised."""
+    q_heads, kv_heads, head_dim, page_size = 8, 2, 64, 16
+    lengths = q_lens = [2210, 37, 300]
+    case = _paged_case(torch.bfloat16, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=6,
+                       v_transposed=True)
+    out = _attend(case, q_heads, kv_heads, head_dim, 0.12, window, max(lengths))
+    expected = _attention_expected(case, 0.12, window)
+    assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(torch.bfloat16, 2)
+
+
 @pytest.mark.parametrize("mode,dtype", ATTENTION_MODES)
 def test_paged_attention_finds_one_far_key_and_respects_edges(mode, dtype):
     """One key among a thousand is made to stand out; the output must be its value.
