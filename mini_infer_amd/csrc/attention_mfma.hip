@@ -69,7 +69,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     bf16_t* __restrict__ out, int64_t out_row_stride, float* __restrict__ part_acc,
     float* __restrict__ part_ml, int q_heads, int kv_heads, int page_size_arg, unsigned page_magic, float scale_log2,
     int window, int num_splits, int heads_per_block, int tokens_per_tile, int one_tile_per_request,
-    int pair_group) {
+    int pair_group, int first_token) {
   constexpr int KSTEPS = D / 32;  // MFMA k-steps over the head dim for S^T
   // PS != 0: the page size is this constant (divisions become shifts, value offsets
   // immediates); PS == 0: any multiple of 16, divided by multiplying with
@@ -97,11 +97,11 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   const int grid_tiles = (int)(gridDim.x / (unsigned)head_slots);
   int req = -1, t0 = 0, n_tok = 0;
   if (one_tile_per_request == 2) {
-    // every request brings exactly one token (a decode step): token b belongs to request b,
-    // and nothing has to be read to know it
+    // every request brings exactly one token (a decode step): request b's token is the
+    // b-th after first_token, and nothing has to be read to know it
     if (grid_tile < num_requests) {
       req = grid_tile;
-      t0 = req;
+      t0 = first_token + req;
       n_tok = 1;
     }
   } else if (one_tile_per_request) {
@@ -665,8 +665,12 @@ extern "C" int mi_attn_mfma_supported(int head_dim, int page_size) {
 // `one_tile_per_request` = 1 promises that no request has more than tokens_per_tile
 // tokens in this step, 2 that every request has exactly one (then cu_seqlens_q is not
 // read); in both cases num_tiles must be num_requests.
-// With num_splits > 1, part_acc holds num_tokens*q_heads*num_splits*head_dim floats
-// and part_ml num_tokens*q_heads*num_splits*2.
+// The requests may be a run out of a larger step: cu_seqlens_q and block_table then point
+// at the run's first request, while q, out, positions and the partial buffers stay
+// those of the whole step (cu_seqlens_q holds token numbers of the whole step);
+// `first_token` is the run's first token and `num_tokens` the run's token count.
+// With num_splits > 1, part_acc holds (first_token+num_tokens)*q_heads*num_splits*head_dim
+// floats and part_ml (first_token+num_tokens)*q_heads*num_splits*2.
 extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_pages,
                             const void* vt_pages, const int* block_table, int max_blocks,
                             const int* cu_seqlens_q, const int* positions, int num_requests,
@@ -674,7 +678,8 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
                             float* part_acc, float* part_ml, int q_heads, int kv_heads,
                             int head_dim, int page_size, int num_pages, float scale, int window,
                             int num_splits, int decode_only, int one_tile_per_request,
-                            hipStream_t stream) {
+                            int first_token, hipStream_t stream) {
+  MI_REQUIRE(first_token >= 0, "attn_mfma: first_token=%d is negative", first_token);
   MI_REQUIRE(num_tokens >= 0 && num_requests >= 0 && num_tiles >= 0,
              "attn_mfma: bad sizes tokens=%d requests=%d tiles=%d", num_tokens, num_requests, num_tiles);
   MI_REQUIRE(q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
@@ -726,7 +731,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
       block_table, max_blocks, cu_seqlens_q, positions, num_requests, (bf16_t*)out,               \
       out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, page_magic, scale_log2,    \
       window,                                                                                     \
-      num_splits, hb, tq, one_tile_per_request, pair_group)
+      num_splits, hb, tq, one_tile_per_request, pair_group, first_token)
 #define MI_LAUNCH_P(DD, PP)                                              \
   if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, false, 2, false, PP); \
   else MI_LAUNCH(DD, MI_PREFILL_WAVES, 1, MI_PREFILL_RG, false, MI_PREFILL_OCC(DD), true, PP)
@@ -748,8 +753,11 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
 #undef MI_LAUNCH_P
 #undef MI_LAUNCH
   MI_CHECK_LAUNCH("attn_mfma");
-  if (num_splits > 1)
-    return mi_attn_reduce_bf16(part_acc, part_ml, out, out_row_stride, num_tokens, q_heads,
-                               head_dim, num_splits, stream);
+  if (num_splits > 1) {
+    const int64_t first_slot = (int64_t)first_token * q_heads * num_splits;
+    return mi_attn_reduce_bf16(part_acc + first_slot * head_dim, part_ml + first_slot * 2,
+                               (bf16_t*)out + (int64_t)first_token * out_row_stride, out_row_stride,
+                               num_tokens, q_heads, head_dim, num_splits, stream);
+  }
   return MI_OK;
 }

@@ -411,37 +411,59 @@ def paged_attention(
     if v_transposed and force_plain:
         raise KernelShapeError("the plain attention kernel reads value pages that are not transposed")
 
-    def partials(splits: int) -> tuple[torch.Tensor | None, torch.Tensor | None]:
+    def partials(splits: int, rows: int = tokens) -> tuple[torch.Tensor | None, torch.Tensor | None]:
         if splits == 1:
             return None, None
         return (
-            torch.empty((tokens * q_heads * splits, head_dim), dtype=torch.float32, device=q.device),
-            torch.empty((tokens * q_heads * splits, 2), dtype=torch.float32, device=q.device),
+            torch.empty((rows * q_heads * splits, head_dim), dtype=torch.float32, device=q.device),
+            torch.empty((rows * q_heads * splits, 2), dtype=torch.float32, device=q.device),
         )
 
     if use_mfma:
         q_lens = [host_cu_seqlens_q[b + 1] - host_cu_seqlens_q[b] for b in range(num_requests)]
-        decode_only = max(q_lens) <= 1
-        tokens_per_tile = lib.mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, int(decode_only))
-        # 2: exactly one token per request (the kernel then needs no request boundaries)
-        one_tile_per_request = 2 if (decode_only and min(q_lens) == 1) else int(max(q_lens) <= tokens_per_tile)
-        num_tiles = num_requests if one_tile_per_request else sum(-(-n // tokens_per_tile) for n in q_lens)
-        rows = 16 if decode_only else 128
-        head_blocks = -(-group // min(group, rows))
-        # decode blocks are register-heavy (about one per CU at a time measured best at batch
-        # 1, 8 and 64); prefill blocks run two to a CU
-        target = 256 if decode_only else 512
-        splits = min(16, attention_splits(num_tiles * kv_heads * head_blocks, max_seq_len, target=target, min_keys=128))
-        part_acc, part_ml = partials(splits)
-        library.check(
-            lib.mi_attn_mfma(
-                _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-                block_table.shape[1], _ptr(cu_seqlens_q), _ptr(positions), num_requests, tokens,
-                num_tiles, _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads,
-                head_dim, page_size, num_pages, float(scale), int(window or 0), splits,
-                int(decode_only), int(one_tile_per_request), _stream(),
+        max_blocks = block_table.shape[1]
+
+        def run(first: int, last: int) -> None:
+            """Requests [first, last) of the step in one launch."""
+            lens = q_lens[first:last]
+            count = last - first
+            first_token = host_cu_seqlens_q[first]
+            run_tokens = host_cu_seqlens_q[last] - first_token
+            decode_only = max(lens) <= 1
+            tokens_per_tile = lib.mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, int(decode_only))
+            # 2: exactly one token per request (the kernel then needs no request boundaries)
+            one_tile_per_request = 2 if (decode_only and min(lens) == 1) else int(max(lens) <= tokens_per_tile)
+            num_tiles = count if one_tile_per_request else sum(-(-n // tokens_per_tile) for n in lens)
+            rows = 16 if decode_only else 128
+            head_blocks = -(-group // min(group, rows))
+            # decode blocks are register-heavy (about one per CU at a time measured best at
+            # batch 1, 8 and 64); prefill blocks run two to a CU
+            target = 256 if decode_only else 512
+            splits = min(16, attention_splits(num_tiles * kv_heads * head_blocks, max_seq_len, target=target, min_keys=128))
+            part_acc, part_ml = partials(splits, first_token + run_tokens)
+            library.check(
+                lib.mi_attn_mfma(
+                    _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages),
+                    _ptr(block_table) + 4 * first * max_blocks, max_blocks,
+                    _ptr(cu_seqlens_q) + 4 * first, _ptr(positions), count, run_tokens,
+                    num_tiles, _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads,
+                    head_dim, page_size, num_pages, float(scale), int(window or 0), splits,
+                    int(decode_only), int(one_tile_per_request), first_token, _stream(),
+                )
             )
-        )
+
+        # Leading requests that bring a single token (a scheduler puts its decoding requests
+        # first) run in the decode shape, where waves split the keys; inside the 128-row
+        # prefill shape each of them would walk all its keys in one block, with 3 % of the
+        # rows in use.
+        leading_single = 0
+        while leading_single < num_requests and q_lens[leading_single] == 1:
+            leading_single += 1
+        if 0 < leading_single < num_requests:
+            run(0, leading_single)
+            run(leading_single, num_requests)
+        else:
+            run(0, num_requests)
         return out
 
     splits = attention_splits(tokens * kv_heads * math.ceil(group / 4), max_seq_len)

@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -39,7 +39,7 @@ _SIGNATURES: dict[str, list] = {
     ],
     "mi_attn_mfma": [
         _P, c_int64, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, _P, c_int64, _P, _P, c_int,
-        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, _P,
+        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, _P,
     ],
     "mi_attn_mfma_tokens_per_tile": [c_int, c_int, c_int],
     "mi_attn_mfma_supported": [c_int, c_int],

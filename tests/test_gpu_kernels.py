@@ -362,6 +362,20 @@ def test_paged_attention_portion_over_long_context_splits_keys(mode, dtype):
     assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
 
 
+@pytest.mark.parametrize("mode,dtype", ATTENTION_MODES)
+def test_paged_attention_single_tokens_first_then_portions(mode, dtype):
+    """The order a scheduler produces: decoding requests (one token each, long and short
+    contexts) first, portions of prompts after them.  The matrix-core path runs the two
+    runs of requests as two launches over the same buffers."""
+    q_heads, kv_heads, head_dim, page_size = 8, 2, 64, 16
+    lengths, q_lens = [1500, 17, 640, 300, 90, 33], [1, 1, 1, 140, 90, 2]
+    case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=4,
+                       v_transposed=mode == "mfma")
+    out = _attend(case, q_heads, kv_heads, head_dim, 0.15, None, max(lengths))
+    expected = _attention_expected(case, 0.15, None)
+    assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
+
+
 @pytest.mark.parametrize("window", [None, 700])
 def test_paged_attention_whole_long_prompts_many_tiles(window):
     """Whole prompts of a few thousand tokens beside a short one: dozens of tiles per head,
