@@ -77,6 +77,26 @@ __device__ ArgBest block_argbest(ArgBest mine, ArgBest* scratch) {
   return best;
 }
 
+// Calls fn(i, x[i]) for this thread's elements i = tid, tid + THREADS, ... in rising order.
+// The elements are read in batches of independent loads: a loop with one load per turn
+// costs a memory latency per element.
+template <typename T, typename F>
+__device__ __forceinline__ void scan_row(const T* __restrict__ x, int vocab, int tid, F&& fn) {
+  for (int i0 = tid; i0 < vocab; i0 += SAMPLE_THREADS * SAMPLE_BATCH) {
+    float v[SAMPLE_BATCH];
+#pragma unroll
+    for (int u = 0; u < SAMPLE_BATCH; ++u) {
+      const int i = i0 + u * SAMPLE_THREADS;
+      v[u] = (i < vocab) ? to_f32(x[i]) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < SAMPLE_BATCH; ++u) {
+      const int i = i0 + u * SAMPLE_THREADS;
+      if (i < vocab) fn(i, v[u]);
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const T* __restrict__ logits, int64_t row_stride, int vocab,
@@ -97,22 +117,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const float temp = temperature[row];
 
   if (temp == 0.f) {
-    // a thread's elements in batches of independent loads (one load per turn would cost a
-    // memory latency per element), visited in rising index order: ties go to the first
-    ArgBest mine = {-INFINITY, 0x7fffffff};
-    for (int i0 = tid; i0 < vocab; i0 += SAMPLE_THREADS * SAMPLE_BATCH) {
-      float v[SAMPLE_BATCH];
-#pragma unroll
-      for (int u = 0; u < SAMPLE_BATCH; ++u) {
-        const int i = i0 + u * SAMPLE_THREADS;
-        v[u] = (i < vocab) ? to_f32(x[i]) : -INFINITY;
-      }
-#pragma unroll
-      for (int u = 0; u < SAMPLE_BATCH; ++u) {
-        const int i = i0 + u * SAMPLE_THREADS;
-        if (i < vocab && (v[u] > mine.val || mine.idx == 0x7fffffff)) { mine.val = v[u]; mine.idx = i; }
-      }
-    }
+    ArgBest mine = {-INFINITY, 0x7fffffff};  // rising index order: ties go to the first
+    scan_row(x, vocab, tid, [&](int i, float v) {
+      if (v > mine.val || mine.idx == 0x7fffffff) { mine.val = v; mine.idx = i; }
+    });
     const ArgBest best = block_argbest(mine, best_scratch);
     if (tid == 0) out[row] = best.idx;
     return;
@@ -120,19 +128,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
   // maximum of the scaled logits
   ArgBest top = {-INFINITY, 0x7fffffff};
-  for (int i0 = tid; i0 < vocab; i0 += SAMPLE_THREADS * SAMPLE_BATCH) {
-    float v[SAMPLE_BATCH];
-#pragma unroll
-    for (int u = 0; u < SAMPLE_BATCH; ++u) {
-      const int i = i0 + u * SAMPLE_THREADS;
-      v[u] = (i < vocab) ? to_f32(x[i]) / temp : -INFINITY;
-    }
-#pragma unroll
-    for (int u = 0; u < SAMPLE_BATCH; ++u) {
-      const int i = i0 + u * SAMPLE_THREADS;
-      if (v[u] > top.val) { top.val = v[u]; top.idx = i; }
-    }
-  }
+  scan_row(x, vocab, tid, [&](int i, float raw) {
+    const float v = raw / temp;
+    if (v > top.val) { top.val = v; top.idx = i; }
+  });
   const float v_max = block_argbest(top, best_scratch).val;
 
   uint32_t key_floor = 0;  // tokens whose key is below this are dropped
@@ -148,9 +147,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       __syncthreads();
       int run_bin = -1;
       uint32_t run_cnt = 0;
-      for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
-        const uint32_t key = order_key(to_f32(x[i]) / temp);
-        if ((key & mask) != prefix) continue;
+      scan_row(x, vocab, tid, [&](int, float raw) {
+        const uint32_t key = order_key(raw / temp);
+        if ((key & mask) != prefix) return;
         const int bin = (key >> shift) & 255;
         if (bin != run_bin) {
           if (run_cnt) atomicAdd(&cnt[run_bin], run_cnt);
@@ -158,7 +157,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
           run_cnt = 0;
         }
         ++run_cnt;
-      }
+      });
       if (run_cnt) atomicAdd(&cnt[run_bin], run_cnt);
       __syncthreads();
       if (tid == 0) {
@@ -191,10 +190,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       int run_bin = -1;
       uint32_t run_cnt = 0;
       unsigned long long run_mass = 0;
-      for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
-        const float v = to_f32(x[i]) / temp;
+      scan_row(x, vocab, tid, [&](int, float raw) {
+        const float v = raw / temp;
         const uint32_t key = order_key(v);
-        if (key < key_floor || (key & mask) != prefix) continue;
+        if (key < key_floor || (key & mask) != prefix) return;
         const int bin = (key >> shift) & 255;
         if (bin != run_bin) {
           if (run_cnt) { atomicAdd(&cnt[run_bin], run_cnt); atomicAdd(&mass[run_bin], run_mass); }
@@ -204,7 +203,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         }
         ++run_cnt;
         run_mass += (unsigned long long)(expf(v - v_max) * MASS_ONE);
-      }
+      });
       if (run_cnt) { atomicAdd(&cnt[run_bin], run_cnt); atomicAdd(&mass[run_bin], run_mass); }
       __syncthreads();
       if (tid == 0) {
@@ -239,17 +238,32 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const uint32_t k0 = seed_lo[row], k1 = seed_hi[row], draw = draw_index[row];
   ArgBest mine = {-INFINITY, 0x7fffffff};
   const int n_quads = (vocab + 3) / 4;
-  for (int quad = tid; quad < n_quads; quad += SAMPLE_THREADS) {
-    uint32_t c[4] = {(uint32_t)quad, draw, 0u, 0u};
-    philox4x32_10(c, k0, k1);
+  constexpr int QUADS = 4;  // quads whose 16 loads are issued together
+  for (int quad0 = tid; quad0 < n_quads; quad0 += SAMPLE_THREADS * QUADS) {
+    float raw[QUADS][4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int i = quad * 4 + e;
-      if (i >= vocab) break;
-      const float v = to_f32(x[i]) / temp;
-      if (order_key(v) < key_floor) continue;
-      const float score = v + gumbel_from_bits(c[e]);
-      if (score > mine.val || mine.idx == 0x7fffffff) { mine.val = score; mine.idx = i; }
+    for (int u = 0; u < QUADS; ++u) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = (quad0 + u * SAMPLE_THREADS) * 4 + e;
+        raw[u][e] = (i < vocab) ? to_f32(x[i]) : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < QUADS; ++u) {
+      const int quad = quad0 + u * SAMPLE_THREADS;
+      if (quad >= n_quads) break;
+      uint32_t c[4] = {(uint32_t)quad, draw, 0u, 0u};
+      philox4x32_10(c, k0, k1);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = quad * 4 + e;
+        if (i >= vocab) break;
+        const float v = raw[u][e] / temp;
+        if (order_key(v) < key_floor) continue;
+        const float score = v + gumbel_from_bits(c[e]);
+        if (score > mine.val || mine.idx == 0x7fffffff) { mine.val = score; mine.idx = i; }
+      }
     }
   }
   const ArgBest best = block_argbest(mine, best_scratch);
