@@ -268,6 +268,83 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   }
 }
 
+// The same for the usual layout (halves paired, every size a multiple of 4), four
+// elements per thread and step: 8- and 16-byte loads and stores instead of single
+// elements.  Arithmetic and rounding are those of the kernel above.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_vec4_kernel(
+    T* __restrict__ qkv, int64_t row_stride, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, const int* __restrict__ slot_mapping, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int q_heads, int kv_heads, int head_dim, int rotary_dim, int page_size,
+    int v_transposed) {
+  const int t = blockIdx.x;
+  const int first = blockIdx.y * blockDim.x + threadIdx.x;
+  const int stride = blockDim.x * gridDim.y;
+  const int half = rotary_dim / 2;
+  const int half4 = half / 4;
+  T* row = qkv + (int64_t)t * row_stride;
+  const float* c = cos_t + (int64_t)t * half;
+  const float* s = sin_t + (int64_t)t * half;
+
+  auto rotate4 = [&](const T* x, int j, float lo[4], float hi[4]) {
+    float x0[4], x1[4], cj[4], sj[4];
+    load4(x + j, x0);
+    load4(x + half + j, x1);
+    load4(c + j, cj);
+    load4(s + j, sj);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      lo[i] = x0[i] * cj[i] - x1[i] * sj[i];
+      hi[i] = x1[i] * cj[i] + x0[i] * sj[i];
+    }
+  };
+
+  for (int e = first; e < q_heads * half4; e += stride) {
+    const int h = e / half4, j = (e % half4) * 4;
+    T* x = row + h * head_dim;
+    float lo[4], hi[4];
+    rotate4(x, j, lo, hi);
+    store4(x + j, lo);
+    store4(x + half + j, hi);
+  }
+
+  if (kv_heads == 0 || slot_mapping == nullptr) return;
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;
+  const int page = slot / page_size, off = slot % page_size;
+  const T* k_row = row + (int64_t)q_heads * head_dim;
+  const T* v_row = k_row + (int64_t)kv_heads * head_dim;
+
+  for (int e = first; e < kv_heads * half4; e += stride) {
+    const int h = e / half4, j = (e % half4) * 4;
+    T* dst = k_pages + (((int64_t)page * kv_heads + h) * page_size + off) * head_dim;
+    float lo[4], hi[4];
+    rotate4(k_row + h * head_dim, j, lo, hi);
+    store4(dst + j, lo);
+    store4(dst + half + j, hi);
+  }
+  const int pass4 = (head_dim - rotary_dim) / 4;
+  for (int e = first; e < kv_heads * pass4; e += stride) {
+    const int h = e / pass4, d = rotary_dim + (e % pass4) * 4;
+    float x[4];
+    load4(k_row + h * head_dim + d, x);
+    store4(k_pages + (((int64_t)page * kv_heads + h) * page_size + off) * head_dim + d, x);
+  }
+  const int dim4 = head_dim / 4;
+  for (int e = first; e < kv_heads * dim4; e += stride) {
+    const int h = e / dim4, d = (e % dim4) * 4;
+    const int64_t chunk = ((int64_t)page * kv_heads + h) * page_size * head_dim;
+    if (v_transposed) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v_pages[chunk + (int64_t)(d + i) * page_size + off] = v_row[h * head_dim + d + i];
+    } else {
+      float x[4];
+      load4(v_row + h * head_dim + d, x);
+      store4(v_pages + chunk + (int64_t)off * head_dim + d, x);
+    }
+  }
+}
+
 extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const float* cos_t,
                                 const float* sin_t, const int* slot_mapping, void* k_pages,
                                 void* v_pages, int num_tokens, int q_heads, int kv_heads,
@@ -284,6 +361,26 @@ extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const 
              "rope_kv_write: pages are needed to write keys and values");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "rope_kv_write: unknown dtype %d", dtype);
   if (num_tokens == 0) return MI_OK;
+  // the usual layout, everything a multiple of 4 elements and 16-byte aligned: four elements a thread
+  const size_t elem = dtype == MI_F32 ? 4 : 2;
+  const bool aligned = ((uintptr_t)qkv | (uintptr_t)cos_t | (uintptr_t)sin_t | (uintptr_t)k_pages |
+                        (uintptr_t)v_pages | (uintptr_t)(row_stride * elem)) % 16 == 0;
+  if (!interleaved && aligned && head_dim % 4 == 0 && rotary_dim % 8 == 0) {
+    const int items = max(q_heads * (rotary_dim / 8), kv_heads * (head_dim / 4));
+    const int blocks_y = min((num_tokens >= 512) ? 2 : 16, max(1, ceil_div(items, 256)));
+    dim3 grid(num_tokens, blocks_y);
+    if (dtype == MI_F32) {
+      rope_kv_write_vec4_kernel<float><<<grid, 256, 0, stream>>>(
+          (float*)qkv, row_stride, cos_t, sin_t, slot_mapping, (float*)k_pages, (float*)v_pages,
+          q_heads, kv_heads, head_dim, rotary_dim, page_size, v_transposed);
+    } else {
+      rope_kv_write_vec4_kernel<bf16_t><<<grid, 256, 0, stream>>>(
+          (bf16_t*)qkv, row_stride, cos_t, sin_t, slot_mapping, (bf16_t*)k_pages, (bf16_t*)v_pages,
+          q_heads, kv_heads, head_dim, rotary_dim, page_size, v_transposed);
+    }
+    MI_CHECK_LAUNCH("rope_kv_write");
+    return MI_OK;
+  }
   // few tokens (decode): spread each token's heads over several blocks
   const int items = max(q_heads * (rotary_dim / 2), kv_heads * head_dim);
   const int blocks_y = min((num_tokens >= 512) ? 4 : 16, max(1, ceil_div(items, 256)));
