@@ -6,7 +6,10 @@ from mini_infer_amd.ops.kernels import (
     embed_gather,
     gemm_f32,
     gemm_skinny_bf16,
+    linear_into_residual,
     linear_swiglu,
+    normed_linear,
+    skinny_fusable,
     linear,
     mfma_attention_supported,
     paged_attention,
@@ -22,7 +25,10 @@ __all__ = [
     "embed_gather",
     "gemm_f32",
     "gemm_skinny_bf16",
+    "linear_into_residual",
     "linear_swiglu",
+    "normed_linear",
+    "skinny_fusable",
     "linear",
     "mfma_attention_supported",
     "paged_attention",
