@@ -6,10 +6,7 @@ from mini_infer_amd.ops.kernels import (
     embed_gather,
     gemm_f32,
     gemm_skinny_bf16,
-    linear_into_residual,
     linear_swiglu,
-    normed_linear,
-    skinny_fusable,
     linear,
     mfma_attention_supported,
     paged_attention,
@@ -25,10 +22,7 @@ __all__ = [
     "embed_gather",
     "gemm_f32",
     "gemm_skinny_bf16",
-    "linear_into_residual",
     "linear_swiglu",
-    "normed_linear",
-    "skinny_fusable",
     "linear",
     "mfma_attention_supported",
     "paged_attention",

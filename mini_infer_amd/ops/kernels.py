@@ -297,85 +297,6 @@ def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return torch.matmul(x, weight.t())
 
 
-STAT_ROWS = 16  # row slots per entry of a sum-of-squares table (the skinny kernel's row limit)
-_PRO_PLAIN, _PRO_NORM = 0, 1
-_EPI_STORE, _EPI_GATED, _EPI_RESIDUAL = 0, 1, 2
-
-
-def skinny_fusable(rows: int, weight: torch.Tensor) -> bool:
-    """Whether a product of `rows` bfloat16 rows with `weight` [N, K] runs on the skinny kernel,
-    and with it the variants that fold the neighbouring norm or residual add into the product."""
-    return (
-        weight.dtype == torch.bfloat16
-        and weight.dim() == 2
-        and weight.stride(1) == 1
-        and skinny_gemm_takes(rows, weight.shape[1], 8, weight.stride(0))
-    )
-
-
-def linear_into_residual(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
-    """`residual += bf16(x @ weight.T)` in one kernel (x bfloat16 [M <= 16, K], residual float32 [M, N]).
-
-    Returns the table [blocks, 16] of partial sums of squares of the new residual rows,
-    which `normed_linear` turns into the RMS norm's statistics without another pass.
-    """
-    _need_cuda(x, weight, residual)
-    m, k = x.shape
-    n = weight.shape[0]
-    if x.dtype != torch.bfloat16 or not skinny_fusable(m, weight) or x.stride(1) != 1 or x.stride(0) % 8:
-        raise KernelShapeError(f"linear_into_residual takes at most 16 bfloat16 rows; got {tuple(x.shape)} {x.dtype}")
-    if residual.dtype != torch.float32 or residual.shape != (m, n) or residual.stride(1) != 1 or weight.shape[1] != k:
-        raise KernelShapeError(f"linear_into_residual: residual must be float32 [{m}, {n}], got {tuple(residual.shape)} {residual.dtype}")
-    lib = library.load()
-    blocks = lib.mi_gemm_skinny_blocks(n, _EPI_RESIDUAL)
-    if blocks <= 0:
-        raise KernelShapeError("linear_into_residual: cannot size the table of sums of squares")
-    stats = torch.empty((blocks, STAT_ROWS), dtype=torch.float32, device=x.device)
-    library.check(
-        lib.mi_gemm_skinny_fused_bf16(
-            _PRO_PLAIN, _EPI_RESIDUAL, _ptr(x), x.stride(0), None, None, 0, 0.0, _ptr(weight), weight.stride(0),
-            _ptr(residual), residual.stride(0), _ptr(stats), m, n, k, _stream(),
-        )
-    )
-    return stats
-
-
-def normed_linear(
-    residual: torch.Tensor,
-    stats: torch.Tensor,
-    norm_weight: torch.Tensor,
-    eps: float,
-    weight: torch.Tensor,
-    gated: bool = False,
-) -> torch.Tensor:
-    """`rmsnorm(residual) @ weight.T` in one kernel, the norm's statistics taken from `stats`.
-
-    residual float32 [M <= 16, K]; `stats` as returned by `linear_into_residual` for these
-    rows; the normalized rows are rounded to bfloat16 as the stand-alone norm kernel rounds
-    them.  gated: weight is [gate; up] stacked and the result silu(gate)*up, [M, N/2].
-    """
-    _need_cuda(residual, stats, norm_weight, weight)
-    m, k = residual.shape
-    rows = weight.shape[0]
-    n = rows // 2 if gated else rows
-    if residual.dtype != torch.float32 or residual.stride(1) != 1 or residual.stride(0) % 4 or not skinny_fusable(m, weight):
-        raise KernelShapeError(f"normed_linear takes at most 16 float32 rows and a bfloat16 weight; got {tuple(residual.shape)}")
-    if weight.shape[1] != k or norm_weight.shape != (k,) or norm_weight.dtype != torch.bfloat16 or (gated and rows % 2):
-        raise KernelShapeError("normed_linear: weight, norm weight and residual widths do not fit")
-    if stats.dtype != torch.float32 or stats.dim() != 2 or stats.shape[1] != STAT_ROWS or not stats.is_contiguous():
-        raise KernelShapeError(f"normed_linear: stats must be float32 [slots, {STAT_ROWS}]")
-    out = torch.empty((m, n), dtype=torch.bfloat16, device=residual.device)
-    lib = library.load()
-    library.check(
-        lib.mi_gemm_skinny_fused_bf16(
-            _PRO_NORM, _EPI_GATED if gated else _EPI_STORE, _ptr(residual), residual.stride(0), _ptr(norm_weight),
-            _ptr(stats), stats.shape[0], float(eps), _ptr(weight), weight.stride(0), _ptr(out), out.stride(0), None,
-            m, n, k, _stream(),
-        )
-    )
-    return out
-
-
 def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
     """`silu(x @ gate.T) * (x @ up.T)` with `gate_up_weight` = [gate; up] stacked, [2I, K].
 

@@ -152,72 +152,6 @@ def test_linear_swiglu_is_the_product_followed_by_the_activation(m, inter, k):
     assert (got32.double() - exact).abs().max() < 1e-4 * float(exact.abs().max()) + 1e-6
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (8, 4096, 14336), (16, 96, 64), (7, 301, 96), (13, 4100, 160), (3, 5, 32)])
-def test_linear_into_residual_adds_the_rounded_product_and_counts_squares(m, n, k):
-    from mini_infer_amd import ops
-
-    x = _rand(m, k, dtype=torch.bfloat16, seed=20)
-    w = _rand(n, k, dtype=torch.bfloat16, seed=21, scale=0.05)
-    residual = _rand(m, n, dtype=torch.float32, seed=22)
-    expected = residual + ops.gemm_skinny_bf16(x, w).float()  # the two-kernel path: rounded product, float32 add
-    stats = ops.linear_into_residual(x, w, residual)
-    assert torch.equal(residual, expected)
-    assert stats.shape[1] == 16 and torch.all(stats[:, m:] == 0)
-    squares = stats.double().sum(0)[:m]
-    exact = (expected.double() ** 2).sum(1)
-    assert ((squares - exact).abs() / exact).max() < 1e-5
-
-
-@pytest.mark.parametrize("gated", [False, True])
-@pytest.mark.parametrize("m,n,k,slots", [(1, 6144, 4096, 256), (8, 28672, 4096, 256), (16, 96, 64, 4), (7, 302, 96, 37), (3, 6, 32, 1)])
-def test_normed_linear_is_the_norm_followed_by_the_product(gated, m, n, k, slots):
-    from mini_infer_amd import ops
-
-    eps = 1e-5
-    residual = _rand(m, k, dtype=torch.float32, seed=23, scale=2.0)
-    gain = (1 + 0.1 * _rand(k, dtype=torch.float32, seed=24)).bfloat16()
-    w = _rand(n, k, dtype=torch.bfloat16, seed=25, scale=0.05)
-    # a table of partial sums of squares as a producer would leave it: any split of the row's sum
-    squares = (residual.double() ** 2).sum(1)
-    share = torch.rand(slots, m, device=DEV, dtype=torch.float64)
-    share = share / share.sum(0)
-    stats = torch.zeros(slots, 16, device=DEV, dtype=torch.float32)
-    stats[:, :m] = (share * squares).float()
-    got = ops.normed_linear(residual, stats, gain, eps, w, gated=gated)
-    # the stand-alone kernels: norm (rounded to bfloat16), then the product (and the activation)
-    normed = ops.add_rmsnorm(None, residual.clone(), gain, eps)
-    two_step = ops.linear_swiglu(normed, w) if gated else ops.gemm_skinny_bf16(normed, w)
-    assert got.shape == two_step.shape
-    # the statistics are summed in another order, so single bfloat16 roundings may differ
-    scale = float(two_step.float().abs().max()) + 1e-6
-    assert (got.float() - two_step.float()).abs().max() < 2.0 ** -6 * scale
-    exact_norm = residual.double() * torch.rsqrt((residual.double() ** 2).mean(1, keepdim=True) + eps) * gain.double()
-    exact = exact_norm @ w.double().T
-    if gated:
-        half = n // 2
-        exact = exact[:, :half] / (1 + torch.exp(-exact[:, :half])) * exact[:, half:]
-    assert (got.double() - exact).abs().max() < 2.0 ** -5 * float(exact.abs().max()) + 1e-6
-
-
-def test_residual_product_feeds_the_normed_product():
-    """The pair as a decoder layer uses it: o-projection into the residual, then norm + gate|up."""
-    from mini_infer_amd import ops
-
-    m, hidden, inter, eps = 8, 4096, 14336, 1e-5
-    attn = _rand(m, hidden, dtype=torch.bfloat16, seed=26)
-    w_o = _rand(hidden, hidden, dtype=torch.bfloat16, seed=27, scale=0.02)
-    w_gu = _rand(2 * inter, hidden, dtype=torch.bfloat16, seed=28, scale=0.02)
-    gain = (1 + 0.1 * _rand(hidden, dtype=torch.float32, seed=29)).bfloat16()
-    residual = _rand(m, hidden, dtype=torch.float32, seed=30)
-    plain_residual = residual.clone()
-    stats = ops.linear_into_residual(attn, w_o, residual)
-    fused = ops.normed_linear(residual, stats, gain, eps, w_gu, gated=True)
-    normed = ops.add_rmsnorm(ops.gemm_skinny_bf16(attn, w_o), plain_residual, gain, eps)
-    assert torch.equal(plain_residual, residual)
-    unfused = ops.linear_swiglu(normed, w_gu)
-    assert (fused.float() - unfused.float()).abs().max() < 2.0 ** -6 * float(unfused.float().abs().max())
-
-
 def test_linear_falls_back_to_the_library_where_the_skinny_kernel_does_not_apply():
     from mini_infer_amd import ops
     from mini_infer_amd.exceptions import KernelShapeError
