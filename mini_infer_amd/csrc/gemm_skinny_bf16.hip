@@ -8,6 +8,9 @@
 // then add their partial tiles through LDS in a fixed order, so the result does not
 // depend on timing.  Activations are small and come from the cache hierarchy.
 //
+// What follows a product in a decoder layer is folded into its last step where that saves a
+// launch: the SiLU-gated product, the rotary encoding with the cache write (EPI_*).
+//
 // This stands where the reference's engine calls the vendor BLAS
 // (distributed/linear.py:167); that library's kernels reach about half of the HBM
 // rate at these shapes.
@@ -25,15 +28,38 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 // each with U*(tiles+1) loads in flight, hide the memory latency better than a deeper
 // pipeline in fewer waves.
 //
-// GATED: W holds two stacked matrices [gate; up] of n rows each and the output is
-// silu(gate . a) * (up . a): a block computes both halves of its features, so the
-// [m, 2n] intermediate is never written.  Both sums are rounded to bfloat16 before the
-// activation, exactly as when the product and the activation run as two kernels.
-template <int NT, int U, bool GATED>
+// What the last step does with the products (each folds a neighbouring launch of a
+// decoder layer into this one):
+//   EPI_STORE  c = bf16(product).
+//   EPI_GATED  W holds two stacked matrices [gate; up] of n rows each and the output is
+//              silu(gate . a) * (up . a): a block computes both halves of its features,
+//              so the [m, 2n] intermediate is never written.
+//   EPI_ROPE   W is the stacked q|k|v projection of an attention layer with half-paired
+//              rotary encoding over the whole head: a block computes dims [j, j+16) and
+//              their partners [half+j, half+j+16) of ONE head, rotates them, and writes
+//              queries to c[m, q_heads*head_dim] and keys and values straight into their
+//              cache slots.
+// In every case the sums are rounded to bfloat16 before the activation or rotation,
+// exactly as when the product and the second step run as two kernels.
+enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2 };
+
+struct RopeArgs {  // EPI_ROPE only
+  const float* cos_t;  // [m, head_dim/2]
+  const float* sin_t;
+  const int* slot_mapping;  // [m]: page * page_size + offset, negative: write nothing
+  bf16_t* k_pages;  // [pages][kv_heads][page_size][head_dim]
+  bf16_t* v_pages;  // the same, or [pages][kv_heads][head_dim][page_size] if v_transposed
+  int q_heads, kv_heads, head_dim, page_size, v_transposed;
+};
+
+template <int NT, int U, int EPI>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t ldw,
-    bf16_t* __restrict__ c, int64_t ldc, int m, int n, int k, int features_per_block) {
-  constexpr int WT = GATED ? 2 * NT : NT;  // weight tiles per block
+    bf16_t* __restrict__ c, int64_t ldc, int m, int n, int k, int features_per_block, const RopeArgs rope) {
+  constexpr bool GATED = EPI == EPI_GATED;
+  constexpr bool ROPE = EPI == EPI_ROPE;
+  static_assert(!ROPE || NT == 1, "the rotary epilogue takes one tile of dims and its partner tile");
+  constexpr int WT = (GATED || ROPE) ? 2 * NT : NT;  // weight tiles per block
   __shared__ float red[SK_WAVES][WT][256];
 
   const int wave = threadIdx.x / MI_WAVE;
@@ -42,8 +68,14 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   const int quad = lane / 16;
   // the block's features [n0, n_end): up to 16*NT, a multiple of 4 chosen by the host so
   // that the blocks spread evenly over the CUs (rows past n_end repeat the last one)
-  const int n0 = blockIdx.x * features_per_block;
-  const int n_end = min(n0 + features_per_block, n);
+  // (rotary epilogue: block = (head, 16-dim tile of the head's first half); n0 is the
+  // tile's first weight row, its partner tile lies half a head further down)
+  const int half = ROPE ? rope.head_dim / 2 : 0;
+  const int tiles_per_head = ROPE ? half / 16 : 1;
+  const int rope_head = ROPE ? blockIdx.x / tiles_per_head : 0;
+  const int rope_j0 = ROPE ? (blockIdx.x % tiles_per_head) * 16 : 0;
+  const int n0 = ROPE ? rope_head * rope.head_dim + rope_j0 : blockIdx.x * features_per_block;
+  const int n_end = ROPE ? n0 + 16 : min(n0 + features_per_block, n);
 
   const int ksteps = k / 32;
   const int per_wave = (ksteps + SK_WAVES - 1) / SK_WAVES;
@@ -55,7 +87,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   const bf16_t* wp[WT];
 #pragma unroll
   for (int t = 0; t < WT; ++t) {
-    const int row = min(n0 + (t % NT) * 16 + col, n_end - 1) + (t / NT) * n;
+    const int row = min(n0 + (t % NT) * 16 + col, n_end - 1) + (t / NT) * (ROPE ? half : n);
     wp[t] = w + (int64_t)row * ldw + quad * 8;
   }
   // activations: lane reads token `col`; lanes past M re-read the last token (the same
@@ -111,17 +143,72 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     for (int wv = 0; wv < SK_WAVES; ++wv)
 #pragma unroll
       for (int r = 0; r < 4; ++r) sum[r] += red[wv][nt][(fq * 4 + r) * 16 + token];
-    if (GATED) {
-      float up[4] = {0.f, 0.f, 0.f, 0.f};
+    float up[4] = {0.f, 0.f, 0.f, 0.f};  // the twin tile's sums: the up half (gated), the partner dims (rotary)
+    if (GATED || ROPE) {
 #pragma unroll
       for (int wv = 0; wv < SK_WAVES; ++wv)
 #pragma unroll
         for (int r = 0; r < 4; ++r) up[r] += red[wv][NT + nt][(fq * 4 + r) * 16 + token];
+    }
+    if (GATED) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float g = (float)(bf16_t)sum[r];
         sum[r] = g / (1.f + expf(-g)) * (float)(bf16_t)up[r];
       }
+    }
+    if (ROPE) {
+      // this thread: dims j..j+3 of the head's first half and their partners, one token
+      const int j = rope_j0 + fq * 4;
+      const int q_heads = rope.q_heads, kv_heads = rope.kv_heads, hd = rope.head_dim;
+      float lo[4], hi[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        lo[r] = (float)(bf16_t)sum[r];
+        hi[r] = (float)(bf16_t)up[r];
+      }
+      if (rope_head < q_heads + kv_heads) {  // queries and keys are rotated (formula: models/blocks/rope.py:411-431)
+        const f32x4_t cs = *reinterpret_cast<const f32x4_t*>(rope.cos_t + (int64_t)token * half + j);
+        const f32x4_t sn = *reinterpret_cast<const f32x4_t*>(rope.sin_t + (int64_t)token * half + j);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float x0 = lo[r], x1 = hi[r];
+          lo[r] = x0 * cs[r] - x1 * sn[r];
+          hi[r] = x1 * cs[r] + x0 * sn[r];
+        }
+      }
+      bf16x4_t lo_b, hi_b;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        lo_b[r] = (bf16_t)lo[r];
+        hi_b[r] = (bf16_t)hi[r];
+      }
+      if (rope_head < q_heads) {
+        bf16_t* dst = c + (int64_t)token * ldc + (int64_t)rope_head * hd + j;
+        *reinterpret_cast<bf16x4_t*>(dst) = lo_b;
+        *reinterpret_cast<bf16x4_t*>(dst + half) = hi_b;
+      } else {
+        const int slot = rope.slot_mapping[token];
+        if (slot >= 0) {  // padding rows of a replayed step write nothing
+          const int page = slot / rope.page_size, off = slot % rope.page_size;
+          const bool is_key = rope_head < q_heads + kv_heads;
+          const int h = rope_head - q_heads - (is_key ? 0 : kv_heads);
+          const int64_t chunk = ((int64_t)page * kv_heads + h) * rope.page_size * hd;
+          if (is_key || !rope.v_transposed) {
+            bf16_t* dst = (is_key ? rope.k_pages : rope.v_pages) + chunk + (int64_t)off * hd + j;
+            *reinterpret_cast<bf16x4_t*>(dst) = lo_b;
+            *reinterpret_cast<bf16x4_t*>(dst + half) = hi_b;
+          } else {
+            bf16_t* dst = rope.v_pages + chunk + off;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              dst[(int64_t)(j + r) * rope.page_size] = lo_b[r];
+              dst[(int64_t)(half + j + r) * rope.page_size] = hi_b[r];
+            }
+          }
+        }
+      }
+      continue;
     }
     const int feature = n0 + nt * 16 + fq * 4;
     bf16_t* dst = c + (int64_t)token * ldc + feature;
@@ -177,16 +264,17 @@ extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, in
   const bf16_t* ap = (const bf16_t*)a;
   const bf16_t* wp = (const bf16_t*)w;
   bf16_t* cp = (bf16_t*)c;
+  const RopeArgs no_rope = {};
   const int cus = compute_units();
   MI_REQUIRE(cus > 0, "gemm_skinny_bf16: cannot read the device's compute unit count");
   const int fpb = features_per_block_for(n, cus, 4);
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
   switch (ceil_div(fpb, 16)) {
-    case 1: gemm_skinny_bf16_kernel<1, 8, false><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb); break;
-    case 2: gemm_skinny_bf16_kernel<2, 8, false><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb); break;
-    case 3: gemm_skinny_bf16_kernel<3, 4, false><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb); break;
-    default: gemm_skinny_bf16_kernel<4, 2, false><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb); break;
+    case 1: gemm_skinny_bf16_kernel<1, 8, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, no_rope); break;
+    case 2: gemm_skinny_bf16_kernel<2, 8, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, no_rope); break;
+    case 3: gemm_skinny_bf16_kernel<3, 4, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, no_rope); break;
+    default: gemm_skinny_bf16_kernel<4, 2, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, no_rope); break;
   }
   MI_CHECK_LAUNCH("gemm_skinny_bf16");
   return MI_OK;
@@ -202,14 +290,56 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
   const bf16_t* ap = (const bf16_t*)a;
   const bf16_t* wp = (const bf16_t*)w;
   bf16_t* cp = (bf16_t*)out;
+  const RopeArgs no_rope = {};
   const int cus = compute_units();
   MI_REQUIRE(cus > 0, "gemm_skinny_swiglu_bf16: cannot read the device's compute unit count");
   const int fpb = features_per_block_for(n, cus, 2);  // two output tiles = four weight tiles
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
-  if (fpb <= 16) gemm_skinny_bf16_kernel<1, 4, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb);
-  else gemm_skinny_bf16_kernel<2, 2, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb);
+  if (fpb <= 16) gemm_skinny_bf16_kernel<1, 4, EPI_GATED><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, no_rope);
+  else gemm_skinny_bf16_kernel<2, 2, EPI_GATED><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, no_rope);
   MI_CHECK_LAUNCH("gemm_skinny_swiglu_bf16");
+  return MI_OK;
+}
+
+// The stacked q|k|v projection of an attention layer with the rotary encoding and the
+// cache write in its last step: q_out[m, q_heads*head_dim] gets the rotated queries, the
+// rotated keys and the values go to their slots (slot_mapping[m]; kv_heads = 0: queries only,
+// w then holds the query rows alone).  Half-paired rotation over the whole head,
+// cos/sin [m, head_dim/2] float32.  One block per (head, 16 dims of the head's first half
+// and their 16 partners).
+extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* q_out,
+                                        int64_t ldq, const float* cos_t, const float* sin_t,
+                                        const int* slot_mapping, void* k_pages, void* v_pages, int m, int k,
+                                        int q_heads, int kv_heads, int head_dim, int page_size, int num_pages,
+                                        int v_transposed, hipStream_t stream) {
+  MI_REQUIRE(q_heads >= 1 && kv_heads >= 0 && head_dim >= 32 && head_dim % 32 == 0,
+             "gemm_skinny_rope_bf16: takes head_dim a multiple of 32; got q_heads=%d kv_heads=%d head_dim=%d",
+             q_heads, kv_heads, head_dim);
+  const int n = (q_heads + 2 * kv_heads) * head_dim;
+  MI_REQUIRE(mi_gemm_skinny_bf16_supported(m, n, k, lda, ldw),
+             "gemm_skinny_rope_bf16: takes 1 <= m <= 16, k a multiple of 32, rows aligned to 16 bytes; "
+             "got m=%d n=%d k=%d lda=%lld ldw=%lld", m, n, k, (long long)lda, (long long)ldw);
+  MI_REQUIRE(lda >= k && ldw >= k && ldq >= (int64_t)q_heads * head_dim && ldq % 4 == 0,
+             "gemm_skinny_rope_bf16: a row stride is shorter than its row or not 8-byte aligned");
+  MI_REQUIRE(cos_t && sin_t, "gemm_skinny_rope_bf16: needs the rotation tables");
+  MI_REQUIRE(kv_heads == 0 || (slot_mapping && k_pages && v_pages && page_size > 0 && num_pages > 0),
+             "gemm_skinny_rope_bf16: pages and slots are needed to write keys and values");
+  RopeArgs rope;
+  rope.cos_t = cos_t;
+  rope.sin_t = sin_t;
+  rope.slot_mapping = slot_mapping;
+  rope.k_pages = (bf16_t*)k_pages;
+  rope.v_pages = (bf16_t*)v_pages;
+  rope.q_heads = q_heads;
+  rope.kv_heads = kv_heads;
+  rope.head_dim = head_dim;
+  rope.page_size = page_size;
+  rope.v_transposed = v_transposed;
+  const int blocks = (q_heads + 2 * kv_heads) * (head_dim / 32);
+  gemm_skinny_bf16_kernel<1, 8, EPI_ROPE><<<blocks, 64 * SK_WAVES, 0, stream>>>(
+      (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, 16, rope);
+  MI_CHECK_LAUNCH("gemm_skinny_rope_bf16");
   return MI_OK;
 }
 
@@ -219,8 +349,9 @@ extern "C" int mi_gemm_skinny_bf16_variant(const void* a, int64_t lda, const voi
   const bf16_t* ap = (const bf16_t*)a;
   const bf16_t* wp = (const bf16_t*)w;
   bf16_t* cp = (bf16_t*)c;
+  const RopeArgs no_rope = {};
   if (fpb <= 0 || fpb > 16 * nt || fpb % 4 != 0) return -2;
-#define V(NT_, U_) if (nt == NT_ && u == U_) { gemm_skinny_bf16_kernel<NT_, U_, false><<<ceil_div(n, fpb), 64 * SK_WAVES, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb); return 0; }
+#define V(NT_, U_) if (nt == NT_ && u == U_) { gemm_skinny_bf16_kernel<NT_, U_, EPI_STORE><<<ceil_div(n, fpb), 64 * SK_WAVES, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, no_rope); return 0; }
   V(1, 8) V(2, 8) V(3, 4) V(4, 2)
 #undef V
   return -1;

@@ -10,6 +10,8 @@ from mini_infer_amd.ops.kernels import (
     linear,
     mfma_attention_supported,
     paged_attention,
+    qkv_rope_write,
+    qkv_rope_write_takes,
     rope_kv_write,
     rope_table,
     sample,
@@ -26,6 +28,8 @@ __all__ = [
     "linear",
     "mfma_attention_supported",
     "paged_attention",
+    "qkv_rope_write",
+    "qkv_rope_write_takes",
     "rope_kv_write",
     "rope_table",
     "sample",

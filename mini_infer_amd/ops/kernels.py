@@ -297,6 +297,85 @@ def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return torch.matmul(x, weight.t())
 
 
+def qkv_rope_write_takes(x: torch.Tensor, weight: torch.Tensor, head_dim: int, rotary_dim: int, interleaved: bool) -> bool:
+    """Whether `qkv_rope_write` runs these operands: at most 16 bfloat16 rows, rotation of
+    whole heads in half pairing, head size a multiple of 32."""
+    return (
+        x.dtype == torch.bfloat16
+        and weight.dtype == torch.bfloat16
+        and x.dim() == 2
+        and x.stride(1) == 1
+        and weight.stride(1) == 1
+        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), weight.stride(0))
+        and not interleaved
+        and rotary_dim == head_dim
+        and head_dim % 32 == 0
+    )
+
+
+def qkv_rope_write(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    cos: torch.Tensor,
+    sin: torch.Tensor,
+    slot_mapping: torch.Tensor | None,
+    k_pages: torch.Tensor | None,
+    v_pages: torch.Tensor | None,
+    *,
+    q_heads: int,
+    kv_heads: int,
+    head_dim: int,
+    v_transposed: bool = False,
+) -> torch.Tensor:
+    """The stacked q|k|v projection, the rotary encoding and the cache write as ONE kernel.
+
+    x [M <= 16, K] bfloat16, weight [(q_heads + 2*kv_heads)*head_dim, K]; returns the rotated
+    queries [M, q_heads*head_dim]; rotated keys and values go to their slots.  `kv_heads=0`
+    with the query rows of the weight alone projects and rotates queries only.  The result
+    is that of `linear` followed by `rope_kv_write` (both round the product to bfloat16
+    before rotating).
+    """
+    _need_cuda(x, weight, cos, sin, slot_mapping, k_pages, v_pages)
+    for name, t in (("cos", cos), ("sin", sin), ("slot_mapping", slot_mapping), ("k_pages", k_pages), ("v_pages", v_pages)):
+        _need_contiguous(name, t)
+    _need_int32("slot_mapping", slot_mapping)
+    if not qkv_rope_write_takes(x, weight, head_dim, head_dim, False):
+        raise KernelShapeError(
+            f"qkv_rope_write takes at most 16 bfloat16 rows and head sizes in steps of 32; got "
+            f"x {tuple(x.shape)} {x.dtype}, head_dim={head_dim}"
+        )
+    m, k = x.shape
+    if weight.shape != ((q_heads + 2 * kv_heads) * head_dim, k):
+        raise KernelShapeError(f"qkv_rope_write: weight {tuple(weight.shape)} does not fit (q+2kv)*head_dim x {k}")
+    if cos.shape != (m, head_dim // 2) or sin.shape != cos.shape or cos.dtype != torch.float32 or sin.dtype != torch.float32:
+        raise KernelShapeError(f"cos/sin must be float32 [{m}, {head_dim // 2}], got {tuple(cos.shape)} {cos.dtype}")
+    page_size = num_pages = 0
+    if kv_heads > 0:
+        if slot_mapping is None or k_pages is None or v_pages is None:
+            raise KernelShapeError("writing keys and values needs slot_mapping, k_pages and v_pages")
+        if k_pages.dtype != torch.bfloat16 or v_pages.dtype != torch.bfloat16:
+            raise KernelShapeError("qkv_rope_write writes bfloat16 pages")
+        if k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != head_dim:
+            raise KernelShapeError(
+                f"k_pages must be [num_pages, {kv_heads}, page_size, {head_dim}], got {tuple(k_pages.shape)}"
+            )
+        _check_v_pages(k_pages, v_pages, v_transposed)
+        if slot_mapping.numel() != m:
+            raise KernelShapeError("slot_mapping needs one entry per row")
+        num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
+    q_out = torch.empty((m, q_heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    lib = library.load()
+    library.check(
+        lib.mi_gemm_skinny_rope_bf16(
+            _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(q_out), q_out.stride(0), _ptr(cos), _ptr(sin),
+            _ptr(slot_mapping) if kv_heads > 0 else None, _ptr(k_pages) if kv_heads > 0 else None,
+            _ptr(v_pages) if kv_heads > 0 else None, m, k, q_heads, kv_heads, head_dim, page_size, num_pages,
+            int(v_transposed), _stream(),
+        )
+    )
+    return q_out
+
+
 def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
     """`silu(x @ gate.T) * (x @ up.T)` with `gate_up_weight` = [gate; up] stacked, [2I, K].
 

@@ -76,6 +76,20 @@ class GQAttention(Mixer):
     ) -> torch.Tensor:
         assert cache.group is not None and cache.k_pages is not None and cache.v_pages is not None
         q_width = self.num_heads * self.head_dim
+        assert self.qkv.weight is not None
+        if self.position is not None and ops.qkv_rope_write_takes(
+            x, self.qkv.weight, self.head_dim, self.position.rotary_dim, self.position.interleaved
+        ):
+            # few rows (decode): projection, rotation and cache write are one kernel
+            cos, sin = self.position.tables(ctx)
+            kv_heads = self.num_kv_heads if writes_cache else 0
+            queries = ops.qkv_rope_write(
+                x, self.qkv.weight if writes_cache else self.qkv.weight[:q_width], cos, sin,
+                ctx.slot_mapping[cache.group] if writes_cache else None, cache.k_pages, cache.v_pages,
+                q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
+                v_transposed=cache.v_transposed,
+            )
+            return self.out.forward(self._attend(queries, ctx, cache))
         if writes_cache:
             qkv = self.qkv.forward(x)
             kv_heads, slots = self.num_kv_heads, ctx.slot_mapping[cache.group]
@@ -99,13 +113,16 @@ class GQAttention(Mixer):
                 q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
                 rotary_dim=0, interleaved=False, v_transposed=cache.v_transposed,
             )
-        attended = ops.paged_attention(
-            qkv, cache.k_pages, cache.v_pages, ctx.block_tables[cache.group], ctx.token_request,
+        return self.out.forward(self._attend(qkv, ctx, cache))
+
+    def _attend(self, queries: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        """Attention of the rotated queries (the first columns of `queries`) over the cache pages."""
+        return ops.paged_attention(
+            queries, cache.k_pages, cache.v_pages, ctx.block_tables[cache.group], ctx.token_request,
             ctx.positions, ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
             max_seq_len=ctx.max_seq_len, v_transposed=cache.v_transposed,
         )
-        return self.out.forward(attended)
 
 
 @register_mixer("gqa_attention")

@@ -152,6 +152,53 @@ def test_linear_swiglu_is_the_product_followed_by_the_activation(m, inter, k):
     assert (got32.double() - exact).abs().max() < 1e-4 * float(exact.abs().max()) + 1e-6
 
 
+@pytest.mark.parametrize("v_transposed", [False, True])
+@pytest.mark.parametrize(
+    "m,hidden,q_heads,kv_heads,head_dim,page_size",
+    [(8, 4096, 32, 8, 128, 16), (1, 4096, 32, 8, 128, 16), (16, 96, 3, 1, 32, 16), (5, 160, 6, 2, 64, 32), (9, 64, 4, 4, 96, 48)],
+)
+def test_qkv_rope_write_is_the_product_followed_by_rotation_and_cache_write(
+    v_transposed, m, hidden, q_heads, kv_heads, head_dim, page_size
+):
+    from mini_infer_amd import ops
+
+    num_pages = 7
+    width = (q_heads + 2 * kv_heads) * head_dim
+    x = _rand(m, hidden, dtype=torch.bfloat16, seed=31)
+    w = _rand(width, hidden, dtype=torch.bfloat16, seed=32, scale=0.1)
+    positions = torch.tensor([0, 1, 700, 5, 131071, 17, 18, 19, 3000, 2, 4, 6, 8, 10, 12, 14][:m], dtype=torch.int32, device=DEV)
+    inv_freq = torch.from_numpy(pl.inv_freq_default(head_dim, 500000.0)).to(DEV)
+    cos, sin = ops.rope_table(positions, inv_freq)
+    slots = torch.tensor([40, 3, 17, 16, 0, 43, -1, 9, 22, 5, 6, 7, 30, 31, 32, 33][:m], dtype=torch.int32, device=DEV)
+    slots = torch.where(slots >= 0, slots % (num_pages * page_size), slots)
+
+    def pages():
+        k = torch.full((num_pages, kv_heads, page_size, head_dim), 7.0, dtype=torch.bfloat16, device=DEV)
+        v_shape = (num_pages, kv_heads, head_dim, page_size) if v_transposed else k.shape
+        return k, torch.full(v_shape, 7.0, dtype=torch.bfloat16, device=DEV)
+
+    k_two, v_two = pages()
+    qkv = ops.gemm_skinny_bf16(x, w)
+    ops.rope_kv_write(qkv, cos, sin, slots, k_two, v_two, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+                      rotary_dim=head_dim, interleaved=False, v_transposed=v_transposed)
+    k_one, v_one = pages()
+    queries = ops.qkv_rope_write(x, w, cos, sin, slots, k_one, v_one, q_heads=q_heads, kv_heads=kv_heads,
+                                 head_dim=head_dim, v_transposed=v_transposed)
+    assert queries.shape == (m, q_heads * head_dim)
+    # the same products rounded the same way, the same rotation formula: equal up to how the
+    # compiler contracts a multiply-add before the final rounding
+    tol = 2.0 ** -7 * float(qkv.float().abs().max())
+    assert (queries.float() - qkv[:, : q_heads * head_dim].float()).abs().max() <= tol
+    assert (k_one.float() - k_two.float()).abs().max() <= tol
+    assert torch.equal(v_one, v_two)  # values are copied, not rotated
+    # queries only (a layer that reads another layer's keys and values): pages stay untouched
+    k_none, v_none = pages()
+    only_q = ops.qkv_rope_write(x, w[: q_heads * head_dim], cos, sin, None, k_none, v_none, q_heads=q_heads,
+                                kv_heads=0, head_dim=head_dim, v_transposed=v_transposed)
+    assert torch.equal(only_q, queries)
+    assert torch.all(k_none == 7.0) and torch.all(v_none == 7.0)
+
+
 def test_linear_falls_back_to_the_library_where_the_skinny_kernel_does_not_apply():
     from mini_infer_amd import ops
     from mini_infer_amd.exceptions import KernelShapeError
