@@ -35,10 +35,10 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 //              silu(gate . a) * (up . a): a block computes both halves of its features,
 //              so the [m, 2n] intermediate is never written.
 //   EPI_ROPE   W is the stacked q|k|v projection of an attention layer with half-paired
-//              rotary encoding over the whole head: a block computes dims [j, j+16) and
-//              their partners [half+j, half+j+16) of ONE head, rotates them, and writes
-//              queries to c[m, q_heads*head_dim] and keys and values straight into their
-//              cache slots.
+//              rotary encoding over the whole head: a block computes some dims of a
+//              head's first half and their partners, rotates them, and writes queries
+//              to c[m, q_heads*head_dim] and keys and values straight into their cache
+//              slots.
 // In every case the sums are rounded to bfloat16 before the activation or rotation,
 // exactly as when the product and the second step run as two kernels.
 enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2 };
@@ -68,14 +68,16 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   const int quad = lane / 16;
   // the block's features [n0, n_end): up to 16*NT, a multiple of 4 chosen by the host so
   // that the blocks spread evenly over the CUs (rows past n_end repeat the last one)
-  // (rotary epilogue: block = (head, 16-dim tile of the head's first half); n0 is the
-  // tile's first weight row, its partner tile lies half a head further down)
+  // Rotary epilogue: the unit of work is a PAIR (a dim of a head's first half and its
+  // partner half a head further on); pairs are numbered through all heads and a block
+  // takes `features_per_block` (a multiple of 4, at most 16) consecutive ones, which may
+  // lie in two heads: tile 0 holds the pairs' first dims, tile 1 their partners.
   const int half = ROPE ? rope.head_dim / 2 : 0;
-  const int tiles_per_head = ROPE ? half / 16 : 1;
-  const int rope_head = ROPE ? blockIdx.x / tiles_per_head : 0;
-  const int rope_j0 = ROPE ? (blockIdx.x % tiles_per_head) * 16 : 0;
-  const int n0 = ROPE ? rope_head * rope.head_dim + rope_j0 : blockIdx.x * features_per_block;
-  const int n_end = ROPE ? n0 + 16 : min(n0 + features_per_block, n);
+  const int total_pairs = ROPE ? (rope.q_heads + 2 * rope.kv_heads) * half : 0;
+  const int pair0 = ROPE ? blockIdx.x * features_per_block : 0;
+  const int pair_end = ROPE ? min(pair0 + features_per_block, total_pairs) : 0;
+  const int n0 = blockIdx.x * features_per_block;
+  const int n_end = min(n0 + features_per_block, n);
 
   const int ksteps = k / 32;
   const int per_wave = (ksteps + SK_WAVES - 1) / SK_WAVES;
@@ -87,7 +89,13 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   const bf16_t* wp[WT];
 #pragma unroll
   for (int t = 0; t < WT; ++t) {
-    const int row = min(n0 + (t % NT) * 16 + col, n_end - 1) + (t / NT) * (ROPE ? half : n);
+    int row;
+    if (ROPE) {
+      const int pair = min(pair0 + col, pair_end - 1);
+      row = (pair / half) * rope.head_dim + pair % half + t * half;
+    } else {
+      row = min(n0 + (t % NT) * 16 + col, n_end - 1) + (t / NT) * n;
+    }
     wp[t] = w + (int64_t)row * ldw + quad * 8;
   }
   // activations: lane reads token `col`; lanes past M re-read the last token (the same
@@ -158,8 +166,10 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
       }
     }
     if (ROPE) {
-      // this thread: dims j..j+3 of the head's first half and their partners, one token
-      const int j = rope_j0 + fq * 4;
+      // this thread: four consecutive pairs (never across a head: half is a multiple of 4), one token
+      const int pair = pair0 + fq * 4;
+      if (pair >= pair_end) continue;
+      const int rope_head = pair / half, j = pair % half;
       const int q_heads = rope.q_heads, kv_heads = rope.kv_heads, hd = rope.head_dim;
       float lo[4], hi[4];
 #pragma unroll
@@ -306,8 +316,7 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
 // cache write in its last step: q_out[m, q_heads*head_dim] gets the rotated queries, the
 // rotated keys and the values go to their slots (slot_mapping[m]; kv_heads = 0: queries only,
 // w then holds the query rows alone).  Half-paired rotation over the whole head,
-// cos/sin [m, head_dim/2] float32.  One block per (head, 16 dims of the head's first half
-// and their 16 partners).
+// cos/sin [m, head_dim/2] float32.
 extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* q_out,
                                         int64_t ldq, const float* cos_t, const float* sin_t,
                                         const int* slot_mapping, void* k_pages, void* v_pages, int m, int k,
@@ -336,9 +345,16 @@ extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* 
   rope.head_dim = head_dim;
   rope.page_size = page_size;
   rope.v_transposed = v_transposed;
-  const int blocks = (q_heads + 2 * kv_heads) * (head_dim / 32);
+  // pairs per block: an even share over the CUs in whole rounds, as for the plain product
+  const int cus = compute_units();
+  MI_REQUIRE(cus > 0, "gemm_skinny_rope_bf16: cannot read the device's compute unit count");
+  const int total_pairs = n / 2;
+  const int rounds = ceil_div(total_pairs, cus * 16);
+  int pairs_per_block = ceil_div(ceil_div(total_pairs, cus * rounds), 4) * 4;
+  if (pairs_per_block > 16) pairs_per_block = 16;
+  const int blocks = ceil_div(total_pairs, pairs_per_block);
   gemm_skinny_bf16_kernel<1, 8, EPI_ROPE><<<blocks, 64 * SK_WAVES, 0, stream>>>(
-      (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, 16, rope);
+      (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, pairs_per_block, rope);
   MI_CHECK_LAUNCH("gemm_skinny_rope_bf16");
   return MI_OK;
 }
