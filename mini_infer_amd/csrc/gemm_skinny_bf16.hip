@@ -358,17 +358,3 @@ extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* 
   MI_CHECK_LAUNCH("gemm_skinny_rope_bf16");
   return MI_OK;
 }
-
-// Tuning hook: the plain product with the block shape chosen by the caller.
-extern "C" int mi_gemm_skinny_bf16_variant(const void* a, int64_t lda, const void* w, int64_t ldw, void* c,
-                                           int64_t ldc, int m, int n, int k, int nt, int u, int fpb, hipStream_t stream) {
-  const bf16_t* ap = (const bf16_t*)a;
-  const bf16_t* wp = (const bf16_t*)w;
-  bf16_t* cp = (bf16_t*)c;
-  const RopeArgs no_rope = {};
-  if (fpb <= 0 || fpb > 16 * nt || fpb % 4 != 0) return -2;
-#define V(NT_, U_) if (nt == NT_ && u == U_) { gemm_skinny_bf16_kernel<NT_, U_, EPI_STORE><<<ceil_div(n, fpb), 64 * SK_WAVES, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, no_rope); return 0; }
-  V(1, 8) V(2, 8) V(3, 4) V(4, 2)
-#undef V
-  return -1;
-}
