@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--serving]
 
 Default workload: the layer sizes of Llama 3.1 8B with random bfloat16 weights
 made on the device, a batch of 8 requests with 2,048-token uniform-random prompts,
@@ -41,6 +41,28 @@ LLAMA_31_8B = {
     "tie_word_embeddings": False,
     "max_position_embeddings": 131072,
 }
+# the serving workload's model (--serving): Llama 3.2 3B layer sizes
+LLAMA_32_3B = {
+    "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 28,
+    "hidden_size": 3072,
+    "num_attention_heads": 24,
+    "num_key_value_heads": 8,
+    "head_dim": 128,
+    "intermediate_size": 8192,
+    "vocab_size": 128256,
+    "rope_theta": 500000.0,
+    "rope_scaling": {
+        "rope_type": "llama3",
+        "factor": 32.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 4.0,
+        "original_max_position_embeddings": 8192,
+    },
+    "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": True,
+    "max_position_embeddings": 131072,
+}
 FULL_LAYERS = LLAMA_31_8B["num_hidden_layers"]
 PROMPT_LEN = 2048
 BLOCK_SIZE = 16
@@ -71,6 +93,55 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
     return linear + attention + head
 
 
+def measure_serving(dtype: str) -> dict:
+    """Continuous batching through the scheduler: 32 concurrent requests, prompt lengths
+    uniform in [128, 4096] of uniform-random ids, 256 greedy tokens each, a 2,048-token
+    budget per step, at Llama-3.2-3B layer sizes with random weights."""
+    import numpy as np
+    import torch
+
+    from mini_infer_amd import ContinuousScheduler, ModelRunner, Request, SamplingParams
+
+    requests_n, new_tokens, longest = 32, 256, 4096
+    pages = requests_n * (-(-(longest + new_tokens) // BLOCK_SIZE)) + 64
+    runner = ModelRunner.from_random(
+        LLAMA_32_3B, seed=0, dtype=dtype, num_blocks=pages, block_size=BLOCK_SIZE, max_concurrent=requests_n
+    )
+    scheduler = ContinuousScheduler(
+        runner, max_concurrent=requests_n, chunk_size=2048, max_num_batched_tokens=2048
+    )
+    rng = np.random.default_rng(3)
+
+    def workload() -> list:
+        lengths = rng.integers(128, longest + 1, size=requests_n)
+        return [
+            Request(rng.integers(0, LLAMA_32_3B["vocab_size"], size=int(n)).tolist(), SamplingParams(ignore_eos=True), new_tokens)
+            for n in lengths
+        ]
+
+    scheduler.run_all(workload()[:4])  # warm-up: kernels built, graphs of the first buckets recorded
+    batch = workload()
+    prompt_tokens = sum(len(r.prompt) for r in batch)
+    steps_before = scheduler.stats["steps"]
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    results = scheduler.run_all(batch)
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - started
+    generated = sum(len(r.tokens) for r in results)
+    return {
+        "model": "Llama-3.2-3B layer sizes",
+        "requests": requests_n,
+        "prompt_tokens": prompt_tokens,
+        "generated_tokens": generated,
+        "seconds": round(seconds, 3),
+        "steps": scheduler.stats["steps"] - steps_before,
+        "generated_tok_s": round(generated / seconds, 1),
+        "total_tok_s": round((prompt_tokens + generated) / seconds, 1),
+        "preemptions": scheduler.stats["preemptions"],
+    }
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -82,6 +153,10 @@ def main() -> int:
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument(
+        "--serving", action="store_true",
+        help="also run 32 concurrent requests through the scheduler at Llama-3.2-3B sizes (adds a 'serving' entry)",
+    )
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -217,6 +292,10 @@ def main() -> int:
     points = {f"decode_b{b}": round(b / per_batch[b][0], 2) for b in batches if b != args.batch}
     if points:
         line["points"] = points
+    if args.serving:
+        del runner
+        torch.cuda.empty_cache()
+        line["serving"] = measure_serving(args.dtype)
     print(json.dumps(line), flush=True)
     return 0
 
