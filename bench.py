@@ -63,7 +63,10 @@ LLAMA_32_3B = {
     "tie_word_embeddings": True,
     "max_position_embeddings": 131072,
 }
-FULL_LAYERS = LLAMA_31_8B["num_hidden_layers"]
+LLAMA_31_70B = dict(
+    LLAMA_31_8B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64, intermediate_size=28672
+)
+SIZES = {"8b": ("Llama-3.1-8B", LLAMA_31_8B), "3b": ("Llama-3.2-3B", LLAMA_32_3B), "70b": ("Llama-3.1-70B", LLAMA_31_70B)}
 PROMPT_LEN = 2048
 BLOCK_SIZE = 16
 
@@ -149,8 +152,9 @@ def main() -> int:
     parser.add_argument("--steps", type=int, default=PROMPT_LEN - 8)
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
-    parser.add_argument("--layers", type=int, default=FULL_LAYERS)
+    parser.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (both numbers are reported)")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
+    parser.add_argument("--sizes", choices=sorted(SIZES), default="8b", help="layer sizes of the model (default: Llama 3.1 8B)")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument(
@@ -171,8 +175,10 @@ def main() -> int:
     from mini_infer_amd.engine import ModelRunner, StepEntry
     from mini_infer_amd.sampling import SamplingParams, sample_tokens
 
-    cfg = dict(LLAMA_31_8B)
-    cfg["num_hidden_layers"] = args.layers
+    model_name, sizes = SIZES[args.sizes]
+    full_layers = sizes["num_hidden_layers"]
+    cfg = dict(sizes)
+    cfg["num_hidden_layers"] = args.layers if args.layers is not None else full_layers
     elem = 2 if args.dtype == "bfloat16" else 4
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     context_end = PROMPT_LEN + args.warmup + args.steps
@@ -250,7 +256,7 @@ def main() -> int:
     step_bytes = weight_bytes(cfg, elem) + args.batch * mean_context * kv_bytes_per_token(cfg, elem)
     achieved = step_bytes / seconds / 1e9
     line = {
-        "metric": "decode tok/s at batch 8, Llama-3.1-8B layer sizes, 2048-token prompts",
+        "metric": f"decode tok/s at batch {args.batch}, {model_name} layer sizes, 2048-token prompts",
         "value": round(args.batch / seconds, 2),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -263,9 +269,9 @@ def main() -> int:
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: uniform-random token ids, random-init weights N(0, 0.02)",
         "config": {
-            "model": "Llama-3.1-8B layer sizes",
-            "layers": args.layers,
-            "layers_full_model": FULL_LAYERS,
+            "model": f"{model_name} layer sizes",
+            "layers": cfg["num_hidden_layers"],
+            "layers_full_model": full_layers,
             "hidden_size": cfg["hidden_size"],
             "num_attention_heads": cfg["num_attention_heads"],
             "num_key_value_heads": cfg["num_key_value_heads"],
