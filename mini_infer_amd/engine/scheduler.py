@@ -27,9 +27,10 @@ emitted, `max_tokens` ends with "length", the last emitted token is never fed
 from __future__ import annotations
 
 import collections
+import dataclasses
 import threading
 import time
-from typing import Any, Callable, Iterable, Sequence
+from typing import Any, Callable, Iterable, Iterator, Sequence
 
 from mini_infer_amd.engine.batch import StepEntry
 from mini_infer_amd.engine.request import (
@@ -50,6 +51,18 @@ def _device_sampler(logits, params, seeds, draws) -> list[int]:
     from mini_infer_amd.sampling.sampler import sample_batch
 
     return sample_batch(logits, params, seeds, draws)
+
+
+@dataclasses.dataclass(frozen=True)
+class SchedulerLoad:
+    """Queue lengths and cache use at one moment (the reference's `load_stats`,
+    scheduler/continuous_scheduler.py:280-300)."""
+
+    num_waiting: int
+    num_running: int
+    kv_cache_usage: float
+    block_size: int
+    num_blocks: int
 
 
 class RequestHandle:
@@ -83,6 +96,28 @@ class RequestHandle:
 
     def steps(self) -> list[GenerationStep]:
         return list(self._running.steps)
+
+    def stream(self, poll_seconds: float = 0.002) -> Iterator[GenerationStep]:
+        """The request's steps as the engine produces them, the terminal one (with its
+        `finish_reason`) last; as the reference's `RequestHandle.steps()`
+        (scheduler/continuous_scheduler.py:195-204).  Without an engine thread the caller
+        drives the engine while it waits."""
+        sent = 0
+        while True:
+            produced = self._running.steps
+            while sent < len(produced):
+                step = produced[sent]
+                sent += 1
+                yield step
+                if step.finish_reason is not None:
+                    return
+            if self._scheduler._thread is None:
+                if not self._scheduler.step() and not self._scheduler.has_work() and sent >= len(self._running.steps):
+                    raise EngineNotRunningError("the request was never finished and the engine has no work left")
+            else:
+                if not self._scheduler.engine_alive and sent >= len(self._running.steps):
+                    raise EngineNotRunningError("the engine stopped before the request finished")
+                time.sleep(poll_seconds)
 
 
 class ContinuousScheduler:
@@ -158,6 +193,27 @@ class ContinuousScheduler:
 
     def run(self, request: Request) -> GenerationResult:
         return self.submit(request).wait()
+
+    def stream(self, request: Request) -> Iterator[GenerationStep]:
+        """Submit and yield each generation step as the engine produces it."""
+        yield from self.submit(request).stream()
+
+    def load_stats(self) -> SchedulerLoad:
+        """Queue lengths and cache use now; callable from any thread (a value may be one step old)."""
+        running = sum(1 for r in list(self._running) if r.state != RequestState.DONE)
+        num_blocks = self.runner.num_blocks
+        return SchedulerLoad(
+            num_waiting=len(self._waiting),
+            num_running=running,
+            kv_cache_usage=1.0 - self._free_pages() / num_blocks if num_blocks else 0.0,
+            block_size=self.runner.block_size,
+            num_blocks=num_blocks,
+        )
+
+    @property
+    def is_running(self) -> bool:
+        """Whether the engine thread is alive (False before `start`, after `stop`, after a crash)."""
+        return self.engine_alive
 
     def run_all(self, requests: Iterable[Request]) -> list[GenerationResult]:
         """Submit all, drive the engine until all are done; results in submission order."""

@@ -246,3 +246,44 @@ def test_out_of_memory_with_nothing_to_preempt_is_raised():
     handle = sched.submit(Request(prompt(4, 0), SamplingParams(), max_tokens=2))
     sched.step()  # preempting the only request cancels it
     assert handle.wait().finish_reason == "cancelled"
+
+
+def test_stream_yields_each_token_then_the_terminal_step():
+    # driven by the caller (no engine thread)
+    sched = make(FakeRunner())
+    steps = list(sched.stream(Request(prompt(7, 5), SamplingParams(), max_tokens=4)))
+    assert [s.tokens for s in steps[:-1]] == [(t,) for t in expected_tokens(prompt(7, 5), 4)]
+    assert steps[-1].finish_reason == "length" and all(s.finish_reason is None for s in steps[:-1])
+    # and with the engine thread, two streams at once
+    sched = make(FakeRunner())
+    sched.start()
+    try:
+        first = sched.submit(Request(prompt(5, 6), SamplingParams(), max_tokens=3))
+        second = sched.submit(Request(prompt(11, 7), SamplingParams(), max_tokens=6))
+        got_second = [s for s in second.stream()]
+        got_first = [s for s in first.stream()]
+        assert sched.is_running
+    finally:
+        sched.stop()
+    assert not sched.is_running
+    assert [t for s in got_first for t in s.tokens] == expected_tokens(prompt(5, 6), 3)
+    assert [t for s in got_second for t in s.tokens] == expected_tokens(prompt(11, 7), 6)
+    assert got_first[-1].finish_reason == "length" and got_second[-1].finish_reason == "length"
+
+
+def test_load_stats_counts_queues_and_pages():
+    runner = FakeRunner(num_blocks=16, block_size=4, max_concurrent=2)
+    sched = make(runner, max_concurrent=2, decode_headroom_blocks=0)
+    load = sched.load_stats()
+    assert (load.num_waiting, load.num_running, load.kv_cache_usage) == (0, 0, 0.0)
+    assert (load.block_size, load.num_blocks) == (4, 16)
+    handles = [sched.submit(Request(prompt(8, s), SamplingParams(), max_tokens=50)) for s in range(3)]
+    assert sched.load_stats().num_waiting == 3
+    sched.step()  # two seats: two admitted and prefilled, one waits
+    load = sched.load_stats()
+    assert (load.num_waiting, load.num_running) == (1, 2)
+    assert load.kv_cache_usage == pytest.approx(4 / 16)  # 2 requests x 8 tokens = 4 pages of 4
+    for handle in handles:
+        handle.cancel()
+    sched.step()
+    assert sched.load_stats().kv_cache_usage == 0.0
