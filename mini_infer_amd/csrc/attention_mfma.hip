@@ -326,12 +326,14 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     bool moved = false;
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) {
+      // raw scores; the scale (positive) is applied to their maximum once and to each
+      // score inside the exponential's argument, as one multiply-add
       float sc[8];
       float mx = -INFINITY;
       if (interior) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          sc[i] = s_acc[rg][i / 4][i % 4] * scale_log2;
+          sc[i] = s_acc[rg][i / 4][i % 4];
           mx = fmaxf(mx, sc[i]);
         }
       } else {
@@ -341,13 +343,13 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
           for (int r = 0; r < 4; ++r) {
             const int key = kb + 16 * hlf + 4 * quad + r;
             const bool visible = key >= lo_row[rg] && key <= pos[rg] && key >= k_begin && key < k_end;
-            const float v = visible ? s_acc[rg][hlf][r] * scale_log2 : -INFINITY;
+            const float v = visible ? s_acc[rg][hlf][r] : -INFINITY;
             sc[hlf * 4 + r] = v;
             mx = fmaxf(mx, v);
           }
         }
       }
-      mx = quad_max(mx);
+      mx = quad_max(mx) * scale_log2;
       // The reference point of the exponentials follows the running maximum lazily: it
       // moves only when the maximum grows by more than RESCALE_SLACK (in log2 units), so
       // probabilities stay below 2^RESCALE_SLACK and the accumulator is rarely rescaled.
@@ -360,7 +362,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
       float sum = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const float p = __builtin_amdgcn_exp2f(sc[i] - m_safe);
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], scale_log2, -m_safe));
         sum += p;
         p_reg[rg][i] = (bf16_t)p;
       }
@@ -690,6 +692,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
   MI_REQUIRE(num_pages > 0 && max_blocks > 0, "attn_mfma: bad page counts num_pages=%d max_blocks=%d",
              num_pages, max_blocks);
   MI_REQUIRE(window >= 0, "attn_mfma: window=%d must be 0 (none) or positive", window);
+  MI_REQUIRE(scale > 0.f, "attn_mfma: the score scale must be positive, got %g", (double)scale);
   MI_REQUIRE(num_splits >= 1 && num_splits <= 64, "attn_mfma: num_splits=%d must be 1..64", num_splits);
   MI_REQUIRE(num_splits == 1 || (part_acc && part_ml), "attn_mfma: split keys need partial buffers");
   MI_REQUIRE(q_row_stride >= (int64_t)q_heads * head_dim && out_row_stride >= (int64_t)q_heads * head_dim,
