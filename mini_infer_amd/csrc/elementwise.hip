@@ -93,6 +93,36 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
   T* o = out + (int64_t)b * hidden;
   const bool store_sum = (rows == nullptr) && (delta != nullptr);
 
+  if (VEC == 4 && hidden <= (int)blockDim.x * 4) {
+    // the whole row is one vector per thread: it stays in registers between the two
+    // passes (no second trip to memory), and the weight is requested before the
+    // reduction instead of after it
+    const int i = threadIdx.x * 4;
+    const bool mine = i < hidden;
+    float s[4] = {0.f, 0.f, 0.f, 0.f}, w[4] = {0.f, 0.f, 0.f, 0.f};
+    if (mine) {
+      load4(res + i, s);
+      load4(weight + i, w);
+      if (dl) {
+        float d[4];
+        load4(dl + i, d);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) s[k] += d[k];
+        if (store_sum) store4(res + i, s);
+      }
+    }
+    float squares = 0.f;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) squares += s[k] * s[k];
+    const float inv_one = rsqrtf(block_sum(squares, scratch) / (float)hidden + eps);
+    if (mine) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) s[k] = w[k] * (s[k] * inv_one);
+      store4(o + i, s);
+    }
+    return;
+  }
+
   float sumsq = 0.f;
   if (VEC == 4) {
     for (int i = threadIdx.x * 4; i < hidden; i += blockDim.x * 4) {
