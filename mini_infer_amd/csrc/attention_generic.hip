@@ -164,6 +164,23 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
   const int t = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x;
   const int64_t base = ((int64_t)t * q_heads + h) * num_splits;
+  constexpr int BATCH = 8;
+  // Few splits of a head of at most 128 dims (the usual decode step): every partial value
+  // this lane needs is requested up front, together with the (max, sum) pairs, so the
+  // kernel waits for memory once.
+  const bool small = num_splits <= BATCH && head_dim <= 2 * MI_WAVE;
+  float early[2][BATCH];
+  if (small) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int d = half * MI_WAVE + lane;
+#pragma unroll
+      for (int i = 0; i < BATCH; ++i) {
+        const int sp = min(i, num_splits - 1);  // past the end: re-read the last split, weight 0 below
+        early[half][i] = (d < head_dim) ? part_acc[(base + sp) * head_dim + d] : 0.f;
+      }
+    }
+  }
   // num_splits <= 64: lane s holds split s
   const float m_s = (lane < num_splits) ? part_ml[(base + lane) * 2] : -INFINITY;
   const float l_s = (lane < num_splits) ? part_ml[(base + lane) * 2 + 1] : 0.f;
@@ -175,7 +192,20 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
   // The partial accumulators are read in batches of independent loads (a load per split
   // issued one after the other's use would cost a memory latency per split) and added in
   // split order.
-  constexpr int BATCH = 8;
+  if (small) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int d = half * MI_WAVE + lane;
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < BATCH; ++i) {
+        const float w = __shfl(w_s, i, MI_WAVE);
+        if (i < num_splits) o += early[half][i] * w;
+      }
+      if (d < head_dim) out[(int64_t)t * out_row_stride + (int64_t)h * head_dim + d] = from_f32<T>(o * inv);
+    }
+    return;
+  }
   for (int d0 = 0; d0 < head_dim; d0 += MI_WAVE) {  // all lanes stay in the loop for the shuffles
     const int d = d0 + lane;
     const bool active = d < head_dim;
