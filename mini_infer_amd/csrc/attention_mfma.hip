@@ -57,11 +57,10 @@ __device__ __forceinline__ float quad_sum(float v) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-// VPF (register pipeline only): value operands are prefetched a block ahead like the
-// keys (more registers), or loaded at the start of the block that uses them (fewer
-// registers, so OCC waves of different blocks can share a SIMD and fill each other's
-// stalls).  SHARED: the block's waves load key and value tiles together through LDS.
-template <int D, int WAVES, int KW, int RG, bool VPF, int OCC, bool SHARED, int PS>
+// OCC: waves per SIMD the registers are budgeted for.  SHARED: the block's waves load key
+// and value tiles together through LDS (prefill); else every wave loads its own operands
+// through two register sets (decode), the values at the start of the block that uses them.
+template <int D, int WAVES, int KW, int RG, int OCC, bool SHARED, int PS>
 __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_row_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table, int max_blocks,
@@ -235,13 +234,12 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     l_run[rg] = 0.f;
   }
 
-  // One 32-key block: the K operands of its two 16-key halves and the V^T operands of
-  // all dim blocks.  A half never straddles a page; K rows of a (page, head) chunk are
+  // One 32-key block: the K operands of its two 16-key halves and where its V^T operands
+  // start.  A half never straddles a page; K rows of a (page, head) chunk are
   // [slot][D], V^T rows are [D][slot].  Released or unallocated pages read page 0:
   // every key of them is masked in the compute step.
   struct KVBlock {
     bf16x8_t k[2][KSTEPS];
-    bf16x8_t v[VPF ? DBLOCKS : 1];
     const bf16_t* v_base[2];
   };
   // Addresses are a wave-uniform base (page, head, first slot: scalar registers) plus a
@@ -296,7 +294,6 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
       for (int s = 0; s < KSTEPS; ++s)
         blk.k[hlf][s] = *reinterpret_cast<const bf16x8_t*>(k_base[hlf] + (k_lane_off + s * 32));
     }
-    if (VPF) load_values(blk.v_base, blk.v);
   };
 
   // The three phases run over all row groups of the wave in turn (scores for every
@@ -391,15 +388,15 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
         o_acc[rg][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op[db], p_reg[rg], o_acc[rg][db], 0, 0, 0);
   };
   auto compute_block = [&](int kb, KVBlock& blk) {
-    bf16x8_t v_late[VPF ? 1 : DBLOCKS];
-    if (!VPF) load_values(blk.v_base, v_late);  // in flight during the scores and the softmax
+    bf16x8_t v_late[DBLOCKS];
+    load_values(blk.v_base, v_late);  // in flight during the scores and the softmax
     f32x4_t s_acc[RG][2];
     block_scores(blk, s_acc);
     bf16x8_t p_reg[RG];
     float alpha[RG];
     // (one branch around the whole rescale, so that it is not turned into selects)
     if (block_softmax(kb, s_acc, p_reg, alpha)) rescale(alpha);
-    block_values(VPF ? blk.v : v_late, p_reg);
+    block_values(v_late, p_reg);
   };
 
   // Software pipeline: the loads of the next block are in flight while this one is
@@ -413,7 +410,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     // are written to the other buffer at the end of the turn; one barrier per turn.
     // Key rows are padded by 16 bytes and value rows by 8 so that the operand reads of
     // 16 lanes fall into different banks.
-    static_assert(KW == 1 && !VPF, "shared tiles are for blocks whose waves walk the same keys");
+    static_assert(KW == 1, "shared tiles are for blocks whose waves walk the same keys");
     constexpr int THREADS = 64 * WAVES;
     constexpr int CPR = D / 8;  // 16-byte chunks per key row
     constexpr int KROW = D + 8;  // elements
@@ -510,7 +507,11 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
       bf16x8_t p_reg[RG];
       float alpha[RG];
       bool more = true;
-      while (more) {  // nested as in the one-set pipeline: the inner loop never multiplies the accumulator
+      // Two loops in each other: the inner one runs while no row's reference point moves and
+      // touches the accumulator with matrix instructions only, so the compiler keeps it in
+      // place; a block that moves a reference leaves the inner loop, has the accumulator
+      // rescaled out here, and the inner loop is entered again.
+      while (more) {
         bool moved = false;
         while (true) {
           request_tile(min(kb + 32, kb_last), ids_next);  // past the end: re-reads the last tile
@@ -728,16 +729,16 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
              "attn_mfma: block table of %d pages of %d is too long for this kernel", max_blocks, page_size);
   const unsigned page_magic = (unsigned)((1ull << 32) / (unsigned)page_size) + 1u;
 
-#define MI_LAUNCH(DD, WW, KK, RR, VV, OO, SS, PP)                                                 \
-  attn_mfma_kernel<DD, WW, KK, RR, VV, OO, SS, PP><<<grid, 64 * WW * KK, 0, stream>>>(                    \
+#define MI_LAUNCH(DD, WW, KK, RR, OO, SS, PP)                                                 \
+  attn_mfma_kernel<DD, WW, KK, RR, OO, SS, PP><<<grid, 64 * WW * KK, 0, stream>>>(                    \
       (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages, (const bf16_t*)vt_pages,            \
       block_table, max_blocks, cu_seqlens_q, positions, num_requests, (bf16_t*)out,               \
       out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, page_magic, scale_log2,    \
       window,                                                                                     \
       num_splits, hb, tq, one_tile_per_request, pair_group, first_token)
 #define MI_LAUNCH_P(DD, PP)                                              \
-  if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, false, 2, false, PP); \
-  else MI_LAUNCH(DD, MI_PREFILL_WAVES, 1, MI_PREFILL_RG, false, MI_PREFILL_OCC(DD), true, PP)
+  if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, 2, false, PP); \
+  else MI_LAUNCH(DD, MI_PREFILL_WAVES, 1, MI_PREFILL_RG, MI_PREFILL_OCC(DD), true, PP)
 #define MI_LAUNCH_D(DD)                 \
   if (page_size == 16) {                \
     MI_LAUNCH_P(DD, 16);                \
