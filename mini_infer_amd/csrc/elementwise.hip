@@ -75,6 +75,32 @@ extern "C" int mi_embed_gather(int dtype, const void* table, const int* ids, flo
 }
 
 // ---------------------------------------------------------------------------
+// Token ids that are still on the device: ids[i] = source[from_rows[i]] where
+// from_rows[i] >= 0 (the token a previous step sampled, not yet read by the host), else
+// ids[i] stays what the host sent.  Values are clamped into the vocabulary.
+// ---------------------------------------------------------------------------
+
+__global__ void take_device_tokens_kernel(int* __restrict__ ids, const int* __restrict__ from_rows,
+                                          const int* __restrict__ source, int n, int source_len, int vocab) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int row = from_rows[i];
+  if (row < 0) return;
+  const int token = source[min(row, source_len - 1)];
+  ids[i] = min(max(token, 0), vocab - 1);
+}
+
+extern "C" int mi_take_device_tokens(int* ids, const int* from_rows, const int* source, int n, int source_len,
+                                     int vocab, hipStream_t stream) {
+  MI_REQUIRE(n >= 0 && source_len >= 1 && vocab >= 1, "take_device_tokens: bad sizes n=%d source=%d vocab=%d", n,
+             source_len, vocab);
+  if (n == 0) return MI_OK;
+  take_device_tokens_kernel<<<ceil_div(n, 256), 256, 0, stream>>>(ids, from_rows, source, n, source_len, vocab);
+  MI_CHECK_LAUNCH("take_device_tokens");
+  return MI_OK;
+}
+
+// ---------------------------------------------------------------------------
 // residual add + RMSNorm
 //   s = residual[r] + delta[r]           (float32; stored back unless `rows` is given)
 //   out[b] = weight * s * rsqrt(mean(s^2) + eps)

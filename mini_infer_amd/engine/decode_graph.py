@@ -17,6 +17,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
+from mini_infer_amd import ops
 from mini_infer_amd.parts.base import StepContext
 
 MIN_WIDTH = 16
@@ -32,20 +33,23 @@ def bucket_of(value: int, minimum: int = 1) -> int:
 class DecodeGraph:
     """One captured decode step for `batch` rows and block tables `width` pages wide."""
 
-    def __init__(self, runner, batch: int, width: int) -> None:
+    def __init__(self, runner, batch: int, width: int, max_device_tokens: int = 64) -> None:
         self.runner = runner
         self.batch = batch
         self.width = width
         self.num_groups = len(runner.cache.groups)
         # layout of the staging buffer (all int32): see `fill`
         b = batch
-        self.sizes = [b, b, b, b + 1, b, b, b] + [n for _ in range(self.num_groups) for n in (b, b * width)]
+        self.sizes = [b, b, b, b + 1, b, b, b] + [n for _ in range(self.num_groups) for n in (b, b * width)] + [b]
         self.total = sum(self.sizes)
         self.host = torch.empty(self.total, dtype=torch.int32, pin_memory=True)
         self.device = torch.zeros(self.total, dtype=torch.int32, device=runner.device)
         views = list(torch.split(self.device, self.sizes))
         slot_mapping = [views[7 + 2 * g] for g in range(self.num_groups)]
         block_tables = [views[8 + 2 * g].view(batch, width) for g in range(self.num_groups)]
+        # rows whose token is still on the device take it from `device_tokens` (first node of the graph)
+        self.from_rows = views[-1]
+        self.device_tokens = torch.zeros(max_device_tokens, dtype=torch.int32, device=runner.device)
         cu = list(range(batch + 1))
         self.ctx = StepContext(
             num_tokens=batch,
@@ -70,7 +74,7 @@ class DecodeGraph:
         self.logits: torch.Tensor | None = None
         self._copied: torch.cuda.Event | None = None  # set once the staging buffer may be rewritten
 
-    def fill(self, token_ids: np.ndarray, index) -> None:
+    def fill(self, token_ids: np.ndarray, index, from_rows: np.ndarray | None = None) -> None:
         """Write this step's integers (padded to the bucket) into the pinned staging buffer."""
         b, real = self.batch, len(index.request_ids)
         if self._copied is not None:
@@ -99,6 +103,7 @@ class DecodeGraph:
             wide[:real, : table.shape[1]] = table
             wide[:real, table.shape[1] :] = -1
             at += b * self.width
+        put(from_rows if from_rows is not None else np.empty(0, dtype=np.int32), b, pad=-1)
         assert at == self.total
 
     def capture(self) -> None:
@@ -114,13 +119,22 @@ class DecodeGraph:
         self.ctx.shared.clear()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
+            ops.take_device_tokens(self.ctx.token_ids, self.from_rows, self.device_tokens, self.runner.vocab_size)
             self.logits = model.forward(self.ctx, caches)
         self.graph = graph
 
-    def run(self, token_ids: np.ndarray, index) -> torch.Tensor:
+    def run(
+        self,
+        token_ids: np.ndarray,
+        index,
+        from_rows: np.ndarray | None = None,
+        device_tokens: torch.Tensor | None = None,
+    ) -> torch.Tensor:
         """Logits [real rows, vocab] of this step; they live until the next replay."""
-        self.fill(token_ids, index)
+        self.fill(token_ids, index, from_rows)
         self.device.copy_(self.host, non_blocking=True)
+        if from_rows is not None and device_tokens is not None:
+            self.device_tokens[: device_tokens.numel()].copy_(device_tokens, non_blocking=True)
         if self._copied is None:
             self._copied = torch.cuda.Event()
         self._copied.record()
@@ -139,21 +153,28 @@ class DecodeGraphs:
         self.graphs: dict[tuple[int, int], DecodeGraph] = {}
         self.replays = 0
 
-    def takes(self, index, rows: np.ndarray) -> bool:
+    def takes(self, index, rows: np.ndarray, device_tokens: torch.Tensor | None = None) -> bool:
         real = len(index.request_ids)
         return (
             index.max_q_len == 1
             and real <= self.max_batch
             and len(rows) == real
             and bool((rows == np.arange(real)).all())
+            and (device_tokens is None or device_tokens.numel() <= self.max_batch)
         )
 
-    def run(self, token_ids: np.ndarray, index) -> torch.Tensor:
+    def run(
+        self,
+        token_ids: np.ndarray,
+        index,
+        from_rows: np.ndarray | None = None,
+        device_tokens: torch.Tensor | None = None,
+    ) -> torch.Tensor:
         batch = bucket_of(len(index.request_ids))
         width = bucket_of(max([t.shape[1] for t in index.block_tables] + [1]), MIN_WIDTH)
         key = (batch, width)
         graph = self.graphs.get(key)
         if graph is None:
-            graph = self.graphs[key] = DecodeGraph(self.runner, batch, width)
+            graph = self.graphs[key] = DecodeGraph(self.runner, batch, width, self.max_batch)
         self.replays += 1
-        return graph.run(token_ids, index)
+        return graph.run(token_ids, index, from_rows, device_tokens)

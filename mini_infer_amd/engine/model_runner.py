@@ -16,6 +16,7 @@ from typing import Any, Hashable, Sequence
 import numpy as np
 import torch
 
+from mini_infer_amd import ops
 from mini_infer_amd.cache.manager import CacheManager
 from mini_infer_amd.config import DEFAULT_BLOCK_SIZE, DEFAULT_NUM_BLOCKS, read_config_json
 from mini_infer_amd.engine.batch import StepEntry
@@ -144,13 +145,19 @@ class ModelRunner:
 
     # -- the step ---------------------------------------------------------------
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], device_tokens: torch.Tensor | None = None) -> torch.Tensor:
         """Run the given tokens as one batch from the cache; logits [wanted, vocab] float32.
 
         Rows come in the order of `entries` and, within an entry, of its `want`.
         The tensor may be reused by the next step: read or copy it before calling
         `step` again.  Requests seen for the first time are admitted.  Raises `OutOfMemoryError`
         before anything changes if the pages for this step are not there.
+
+        `device_tokens` (int32, on the device) holds token ids the host has not read yet,
+        e.g. what `sample_tokens` returned for the last step; an entry with `device_row`
+        takes its token from there, so the next step can be launched before the ids of the
+        last one have come back (the reference's asynchronous sampling,
+        scheduler/continuous_scheduler.py:529-646).
         """
         entries = [e for e in entries if len(e.tokens) > 0]
         if not entries:
@@ -168,6 +175,21 @@ class ModelRunner:
         token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
         if token_ids.min() < 0 or token_ids.max() >= self.vocab_size:
             raise ValueError(f"token ids must lie in 0..{self.vocab_size - 1}")
+        from_rows: np.ndarray | None = None
+        if any(e.device_row is not None for e in entries):
+            if device_tokens is None or device_tokens.dtype != torch.int32 or device_tokens.dim() != 1:
+                raise ValueError("entries with device_row need device_tokens, a 1-d int32 tensor on the device")
+            from_rows = np.full(token_ids.size, -1, dtype=np.int32)
+            at = 0
+            for entry in entries:
+                if entry.device_row is not None:
+                    if len(entry.tokens) != 1 or not 0 <= entry.device_row < device_tokens.numel():
+                        raise ValueError(
+                            f"request {entry.request_id!r}: device_row goes with exactly one placeholder token "
+                            f"and must index the {device_tokens.numel()} device tokens"
+                        )
+                    from_rows[at] = entry.device_row
+                at += len(entry.tokens)
 
         admitted: list[Hashable] = []
         try:
@@ -188,15 +210,21 @@ class ModelRunner:
             dtype=np.int32,
         )
         token_ids = token_ids.astype(np.int32)
-        if self.decode_graphs is not None and self.decode_graphs.takes(index, rows):
-            logits = self.decode_graphs.run(token_ids, index)
+        if self.decode_graphs is not None and self.decode_graphs.takes(index, rows, device_tokens):
+            logits = self.decode_graphs.run(token_ids, index, from_rows, device_tokens)
         else:
-            logits = self.model.forward(self._to_device(token_ids, rows, index), self._layer_caches)
+            ctx, from_rows_device = self._to_device(token_ids, rows, index, from_rows)
+            if from_rows_device is not None:
+                ops.take_device_tokens(ctx.token_ids, from_rows_device, device_tokens, self.vocab_size)
+            logits = self.model.forward(ctx, self._layer_caches)
         self.cache.commit(extents)
         return logits
 
-    def _to_device(self, token_ids: np.ndarray, rows: np.ndarray, index) -> StepContext:
-        """All of a step's integers in one pinned buffer and one copy to the device."""
+    def _to_device(
+        self, token_ids: np.ndarray, rows: np.ndarray, index, from_rows: np.ndarray | None = None
+    ) -> tuple[StepContext, torch.Tensor | None]:
+        """All of a step's integers in one pinned buffer and one copy to the device
+        (the step's context, and `from_rows` on the device if it was given)."""
         pieces = [
             token_ids,
             index.positions,
@@ -209,6 +237,8 @@ class ModelRunner:
         for mapping, table in zip(index.slot_mapping, index.block_tables):
             pieces.append(mapping)
             pieces.append(table.reshape(-1))
+        if from_rows is not None:
+            pieces.append(from_rows)
         sizes = [int(p.size) for p in pieces]
         staging = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=True)
         host = staging.numpy()
@@ -223,7 +253,7 @@ class ModelRunner:
         for g, table in enumerate(index.block_tables):
             slot_mapping.append(views[7 + 2 * g])
             block_tables.append(views[8 + 2 * g].view(table.shape))
-        return StepContext(
+        ctx = StepContext(
             num_tokens=int(token_ids.size),
             num_requests=len(index.request_ids),
             page_size=self.block_size,
@@ -242,3 +272,4 @@ class ModelRunner:
             host_seq_lens=index.seq_lens.tolist(),
             host_state_slots=index.state_slots.tolist(),
         )
+        return ctx, (views[-1] if from_rows is not None else None)

@@ -16,6 +16,7 @@ from mini_infer_amd.ops.kernels import (
     rope_table,
     sample,
     silu_mul,
+    take_device_tokens,
 )
 
 __all__ = [
@@ -34,4 +35,5 @@ __all__ = [
     "rope_table",
     "sample",
     "silu_mul",
+    "take_device_tokens",
 ]

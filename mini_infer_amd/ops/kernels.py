@@ -93,6 +93,20 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def take_device_tokens(ids: torch.Tensor, from_rows: torch.Tensor, source: torch.Tensor, vocab: int) -> None:
+    """In place: `ids[i] = source[from_rows[i]]` where `from_rows[i] >= 0` (all int32, on the device)."""
+    _need_cuda(ids, from_rows, source)
+    for name, t in (("ids", ids), ("from_rows", from_rows), ("source", source)):
+        _need_contiguous(name, t)
+        _need_int32(name, t)
+    if ids.dim() != 1 or from_rows.shape != ids.shape or source.dim() != 1 or source.numel() == 0:
+        raise KernelShapeError("take_device_tokens: ids and from_rows are [n], source is [rows >= 1]")
+    lib = library.load()
+    library.check(
+        lib.mi_take_device_tokens(_ptr(ids), _ptr(from_rows), _ptr(source), ids.numel(), source.numel(), int(vocab), _stream())
+    )
+
+
 def add_rmsnorm(
     delta: torch.Tensor | None,
     residual: torch.Tensor,

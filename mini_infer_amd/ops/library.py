@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -22,6 +22,7 @@ _lib_path: Path | None = None
 _P = c_void_p
 _SIGNATURES: dict[str, list] = {
     "mi_embed_gather": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
+    "mi_take_device_tokens": [_P, _P, _P, c_int, c_int, c_int, _P],
     "mi_add_rmsnorm": [c_int, _P, _P, _P, _P, _P, c_int, c_int, c_float, _P],
     "mi_rope_table": [_P, _P, _P, _P, c_int, c_int, _P],
     "mi_rope_kv_write": [

@@ -322,6 +322,46 @@ def test_graph_replays_equal_eager_steps_with_eager_work_between(tmp_path, dtype
         runner.cache.check()
 
 
+@pytest.mark.parametrize("cuda_graph", [True, False])
+def test_tokens_left_on_the_device_give_the_steps_of_tokens_from_the_host(tmp_path, cuda_graph):
+    """A decode step whose tokens are still on the device (`device_row`) equals the step fed
+    from the host; in changing row order, with rows left out, beside a prompt portion."""
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.sampling import SamplingParams, sample_tokens
+
+    cfg, block, weights, folder = _folder(tmp_path, "B", 61)
+    runners = [ModelRunner.from_pretrained(folder, dtype="float32", num_blocks=64, block_size=block, cuda_graph=cuda_graph)
+               for _ in range(2)]
+    by_device, by_host = runners
+    ids = ["p", "q", "r"]
+    greedy = [SamplingParams()] * 3
+    for n, rid in enumerate(ids):
+        prompt = tiny.random_tokens(cfg, 9 + 5 * n, seed=n)
+        for runner in runners:
+            runner.step([StepEntry(rid, prompt, [])])
+    first = [3, 5, 7]
+    device_logits = by_device.step([StepEntry(r, [t], [0]) for r, t in zip(ids, first)])
+    host_logits = by_host.step([StepEntry(r, [t], [0]) for r, t in zip(ids, first)])
+    for step in range(6):
+        sampled = sample_tokens(device_logits, greedy, [0] * 3, [step] * 3)  # stays on the device
+        on_host = sample_tokens(host_logits, greedy, [0] * 3, [step] * 3).tolist()
+        order = [(step + i) % 3 for i in range(3)]  # the rows change places from step to step
+        entries_d = [StepEntry(ids[j], [0], [0], device_row=j) for j in order]
+        entries_h = [StepEntry(ids[j], [on_host[j]], [0]) for j in order]
+        if step == 3:  # a new request's prompt beside the decode tokens: not a pure decode step
+            extra = StepEntry("new", tiny.random_tokens(cfg, 6, seed=9), [5])
+            entries_d.append(extra), entries_h.append(extra)
+        device_logits = by_device.step(entries_d, device_tokens=sampled)
+        host_logits = by_host.step(entries_h)
+        assert torch.equal(device_logits, host_logits), f"step {step}"
+        inverse = [order.index(j) for j in range(3)]  # back to the order of `ids` for the next sample
+        device_logits, host_logits = device_logits[inverse], host_logits[inverse]
+    with pytest.raises(ValueError, match="device_row"):
+        by_device.step([StepEntry("p", [0], [0], device_row=0)])
+    with pytest.raises(ValueError, match="device_row"):
+        by_device.step([StepEntry("p", [0, 1], [0], device_row=0)], device_tokens=sampled)
+
+
 def test_model_with_a_host_looping_part_is_not_graphed(tmp_path):
     from mini_infer_amd.parts import Mixer
 
