@@ -5,7 +5,8 @@
 Default workload: the layer sizes of Llama 3.1 8B with random bfloat16 weights
 made on the device, a batch of 8 requests with 2,048-token uniform-random prompts,
 decoded greedily from position 2,048 on; one "step" is one decode step of the whole
-batch (step function + greedy choice on the device + ids back to the host).  The
+batch (step function + greedy choice on the device + ids back to the host, which reads
+them one step late: the next step takes its tokens from the device).  The
 line it prints also holds the prefill rate of one 2,048-token prompt, the decode
 rates at batch 1 and 64, and the decode step's share of the HBM roofline.
 """
@@ -210,18 +211,45 @@ def main() -> int:
             logits = prefill(rid, prompt)
             last.append(int(sample_tokens(logits, [greedy], [0], [0]).tolist()[0]))
         params, seeds = [greedy] * batch, [0] * batch
+        host_ids = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        copied = [torch.cuda.Event(), torch.cuda.Event()]
 
-        def one_step(tokens: list[int], draw: int) -> list[int]:
-            logits = runner.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
-            return sample_tokens(logits, params, seeds, [draw] * batch).tolist()
+        # A step: the step function, the greedy choice on the device, the ids on their way to
+        # the host.  The next step takes its tokens from the device (`device_row`), so it is
+        # launched before the last one's ids have arrived; the host reads them one step late.
+        def one_step(ids_on_device: torch.Tensor | None, tokens: list[int], draw: int) -> torch.Tensor:
+            if ids_on_device is None:
+                entries = [StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)]
+            else:
+                entries = [StepEntry(rid, [0], [0], device_row=row) for row, rid in enumerate(ids)]
+            logits = runner.step(entries, device_tokens=ids_on_device)
+            sampled = sample_tokens(logits, params, seeds, [draw] * batch)
+            host_ids[draw % 2].copy_(sampled, non_blocking=True)
+            copied[draw % 2].record()
+            return sampled
 
+        def read_ids(draw: int) -> list[int]:
+            copied[draw % 2].synchronize()
+            return host_ids[draw % 2].tolist()
+
+        on_device = None
         for w in range(args.warmup):
-            last = one_step(last, w)
+            on_device = one_step(on_device, last, w)
+            if w > 0:
+                read_ids(w - 1)
+        if args.warmup > 0:
+            last = read_ids(args.warmup - 1)
         sync()
         started = time.perf_counter()
+        generated = 0
         for k in range(args.steps):
-            last = one_step(last, args.warmup + k)
+            draw = args.warmup + k
+            on_device = one_step(on_device, last, draw)
+            if k > 0:
+                generated += len(read_ids(draw - 1))
+        generated += len(read_ids(args.warmup + args.steps - 1))
         sync()
+        assert generated == batch * args.steps
         seconds = (time.perf_counter() - started) / args.steps
         for rid in ids:
             runner.free_request(rid)
