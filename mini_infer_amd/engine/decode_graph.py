@@ -14,6 +14,8 @@ the host over `ctx.host_*` lists cannot be replayed with other lengths.
 
 from __future__ import annotations
 
+import gc
+
 import numpy as np
 import torch
 
@@ -118,9 +120,19 @@ class DecodeGraph:
         torch.cuda.synchronize()
         self.ctx.shared.clear()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            ops.take_device_tokens(self.ctx.token_ids, self.from_rows, self.device_tokens, self.runner.vocab_size)
-            self.logits = model.forward(self.ctx, caches)
+        # No garbage collection while the stream records: a collector run frees whatever cyclic
+        # garbage earlier work left (pinned buffers, events, other graphs), their destructors make
+        # runtime calls that a recording stream forbids, and an error inside a destructor aborts.
+        collecting = gc.isenabled()
+        gc.collect()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                ops.take_device_tokens(self.ctx.token_ids, self.from_rows, self.device_tokens, self.runner.vocab_size)
+                self.logits = model.forward(self.ctx, caches)
+        finally:
+            if collecting:
+                gc.enable()
         self.graph = graph
 
     def run(

@@ -35,6 +35,7 @@ class LLM:
         chunk_size: int = DEFAULT_CHUNK_SIZE,
         decode_headroom_blocks: int = DEFAULT_DECODE_HEADROOM_BLOCKS,
         seed: int = 0,
+        async_sampling: bool | None = None,
     ) -> None:
         self.runner = ModelRunner.from_pretrained(
             model,
@@ -55,6 +56,7 @@ class LLM:
             eos_token_id=raw.get("eos_token_id"),
             tokenizer=self.tokenizer,
             base_seed=seed,
+            async_sampling=async_sampling,
         )
 
     def generate(

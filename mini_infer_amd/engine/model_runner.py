@@ -129,6 +129,8 @@ class ModelRunner:
         return cls(model, config, num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent,
                    cuda_graph=cuda_graph)
 
+    supports_device_tokens = True  # `step(entries, device_tokens=)`, `StepEntry.device_row`
+
     # -- requests ---------------------------------------------------------------
 
     def add_request(self, request_id: Hashable) -> None:

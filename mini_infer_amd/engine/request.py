@@ -66,6 +66,9 @@ class RunningRequest:
     preemptions: int = 0
     steps: list[GenerationStep] = dataclasses.field(default_factory=list)
     done_event: threading.Event = dataclasses.field(default_factory=threading.Event)
+    # asynchronous sampling: the request's newest token has been sampled but not read by the
+    # host yet; it is this row of the scheduler's pending sample
+    pending_row: int | None = None
 
     @property
     def feed(self) -> list[int]:

@@ -22,6 +22,13 @@ emitted, `max_tokens` ends with "length", the last emitted token is never fed
     greedy and seeded outputs are unchanged.  The reference cancels the youngest
     request instead (:388-416).  A request that cannot fit even alone is
     finished as "cancelled".
+
+Asynchronous sampling (the reference's `async_sampling`, :529-646): tokens are sampled on
+the device and the NEXT step is launched from them while they are still there; the host
+reads a step's ids one step late, so its work (bookkeeping, building the next batch)
+overlaps the device's.  End-of-sequence is therefore seen one step late: the request has
+been fed once more by then, and that step's result for it is dropped.  Outputs are the
+same as without it.
 """
 
 from __future__ import annotations
@@ -63,6 +70,16 @@ class SchedulerLoad:
     kv_cache_usage: float
     block_size: int
     num_blocks: int
+
+
+@dataclasses.dataclass
+class _PendingSample:
+    """Ids sampled by the last step that the host has not read yet."""
+
+    requests: list[RunningRequest]  # row i belongs to requests[i]
+    on_device: Any  # int32 tensor [rows]
+    on_host: Any  # pinned int32 tensor [rows], valid once `copied` has happened
+    copied: Any  # event
 
 
 class RequestHandle:
@@ -133,6 +150,7 @@ class ContinuousScheduler:
         tokenizer: Any = None,
         base_seed: int = 0,
         sampler: Callable[..., list[int]] | None = None,
+        async_sampling: bool | None = None,
     ) -> None:
         if max_concurrent <= 0 or chunk_size <= 0 or max_num_batched_tokens <= 0:
             raise ValueError("max_concurrent, chunk_size and max_num_batched_tokens must be positive")
@@ -153,6 +171,14 @@ class ContinuousScheduler:
         self.tokenizer = tokenizer
         self.base_seed = base_seed
         self._sample = sampler or _device_sampler
+        # None: on where it can be (the runner takes tokens from the device and the sampler is the device's own)
+        can_async = sampler is None and bool(getattr(runner, "supports_device_tokens", False))
+        if async_sampling and not can_async:
+            raise ValueError("async_sampling needs a runner that takes device tokens and the built-in sampler")
+        self.async_sampling = can_async if async_sampling is None else bool(async_sampling)
+        self._pending: _PendingSample | None = None
+        self._ids_on_host = None  # pinned int32 [max_concurrent], made at the first asynchronous sample
+        self._ids_copied = None  # event after the copy into it
         self._waiting: collections.deque[RunningRequest] = collections.deque()
         self._running: list[RunningRequest] = []
         self._next_id = 0
@@ -248,6 +274,7 @@ class ContinuousScheduler:
             self._finish(running, "cancelled")
         self._running.clear()
         self._waiting.clear()
+        self._pending = None
 
     def _engine_loop(self) -> None:
         try:
@@ -263,22 +290,29 @@ class ContinuousScheduler:
     # -- one step -------------------------------------------------------------------
 
     def has_work(self) -> bool:
-        return bool(self._waiting or self._running)
+        return bool(self._waiting or self._running or self._pending is not None)
 
     def step(self) -> bool:
         """Admit, build one batch, run it, sample, finish.  False when there was nothing to do."""
         self._cancel_pending()
         self._admit_waiting()
         if not self._running:
-            return False
+            return self._resolve_pending()
         while True:
             entries, owners = self._build_batch()
             if not entries:
-                return False
+                return self._resolve_pending()
             try:
-                logits = self.runner.step(entries)
+                device_tokens = self._pending.on_device if any(e.device_row is not None for e in entries) else None
+                if device_tokens is not None:
+                    logits = self.runner.step(entries, device_tokens=device_tokens)
+                else:
+                    logits = self.runner.step(entries)
                 break
             except OutOfMemoryError:
+                # what is still on the device is read first, so that a preempted request
+                # keeps every token it has been given
+                self._resolve_pending()
                 if not self._preempt_youngest():
                     raise
         self.stats["steps"] += 1
@@ -286,19 +320,64 @@ class ContinuousScheduler:
         sampled_for: list[RunningRequest] = []
         for entry, running in zip(entries, owners):
             running.tokens_fed += len(entry.tokens)
-            running.state = (
-                RequestState.DECODING if running.prefill_remaining == 0 else RequestState.CHUNKED_PREFILLING
-            )
             if entry.want:
                 sampled_for.append(running)
+        # the ids of the step before this one have had this step's launch to arrive
+        self._resolve_pending()
+        for running in owners:
+            if running.state != RequestState.DONE:
+                running.state = (
+                    RequestState.DECODING if running.prefill_remaining == 0 else RequestState.CHUNKED_PREFILLING
+                )
         if sampled_for:
-            token_ids = self._sample(
-                logits,
-                [r.request.sampling_params for r in sampled_for],
-                [r.seed for r in sampled_for],
-                [len(r.tokens_generated) for r in sampled_for],
-            )
-            for running, token in zip(sampled_for, token_ids):
+            # (rows of requests that the late ids have just finished are sampled too and dropped)
+            params = [r.request.sampling_params for r in sampled_for]
+            seeds = [r.seed for r in sampled_for]
+            draws = [len(r.tokens_generated) for r in sampled_for]
+            if self.async_sampling:
+                self._sample_later(logits, sampled_for, params, seeds, draws)
+            else:
+                token_ids = self._sample(logits, params, seeds, draws)
+                for running, token in zip(sampled_for, token_ids):
+                    if running.state != RequestState.DONE:
+                        self._accept_token(running, int(token))
+        self._reap_done()
+        return True
+
+    # -- asynchronous sampling ---------------------------------------------------------------
+
+    def _sample_later(self, logits, sampled_for, params, seeds, draws) -> None:
+        """Sample on the device, start the copy of the ids to the host, read nothing yet."""
+        import torch
+
+        from mini_infer_amd.sampling.sampler import sample_tokens
+
+        on_device = sample_tokens(logits, params, seeds, draws)
+        # One pinned buffer and one event for the scheduler's life: the ids of a step are read
+        # (`_resolve_pending`) before the next step's ids are copied into the same place.
+        if self._ids_on_host is None or self._ids_on_host.numel() < on_device.numel():
+            self._ids_on_host = torch.empty(max(self.max_concurrent, on_device.numel()), dtype=torch.int32, pin_memory=True)
+            self._ids_copied = torch.cuda.Event()
+        on_host = self._ids_on_host[: on_device.numel()]
+        on_host.copy_(on_device, non_blocking=True)
+        copied = self._ids_copied
+        copied.record()
+        for row, running in enumerate(sampled_for):
+            if running.state != RequestState.DONE:
+                running.pending_row = row
+        self._pending = _PendingSample(list(sampled_for), on_device, on_host, copied)
+
+    def _resolve_pending(self) -> bool:
+        """Read the ids still on their way and give each request its token.  False if there were none."""
+        pending, self._pending = self._pending, None
+        if pending is None:
+            return False
+        pending.copied.synchronize()
+        for running, token in zip(pending.requests, pending.on_host.tolist()):
+            if running.pending_row is None:
+                continue  # finished or cancelled since
+            running.pending_row = None
+            if running.state != RequestState.DONE:
                 self._accept_token(running, int(token))
         self._reap_done()
         return True
@@ -376,8 +455,19 @@ class ContinuousScheduler:
         budget = self.max_num_batched_tokens
         entries: list[StepEntry] = []
         owners: list[RunningRequest] = []
-        decoders = [r for r in self._running if r.prefill_remaining == 1 and r.tokens_fed > 0]
-        prefillers = [r for r in self._running if r not in decoders]
+        # a request whose newest token is still on the device decodes from there, unless that
+        # token is its last (then it ends when the token is read and is fed nothing more)
+        on_device = [r for r in self._running if r.pending_row is not None]
+        decoders = [r for r in self._running if r.pending_row is None and r.prefill_remaining == 1 and r.tokens_fed > 0]
+        prefillers = [r for r in self._running if r.pending_row is None and r not in decoders]
+        for running in on_device:
+            if budget <= 0:
+                break
+            if len(running.tokens_generated) + 1 >= running.request.max_tokens:
+                continue
+            entries.append(StepEntry(running.request_id, [0], [0], device_row=running.pending_row))
+            owners.append(running)
+            budget -= 1
         for running in decoders:
             if budget <= 0:
                 break
@@ -436,6 +526,7 @@ class ContinuousScheduler:
         if running.state == RequestState.DONE:
             return
         running.finish_reason = reason  # type: ignore[assignment]
+        running.pending_row = None
         in_cache = running in self._running and not already_freed
         running.state = RequestState.DONE
         if in_cache and self.cache.has_request(running.request_id):

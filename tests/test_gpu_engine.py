@@ -197,6 +197,54 @@ def test_preemption_on_the_real_engine_keeps_outputs(tmp_path):
     assert llm.runner.num_free_blocks() == 14
 
 
+def test_asynchronous_sampling_gives_the_tokens_of_synchronous_sampling(tmp_path):
+    """Ids read one step late: the same tokens and finish reasons as reading them at once, with
+    requests that end by end-of-sequence (seen a step late), by length (1 and more tokens),
+    sampled and greedy ones, so few pages that requests are preempted, and a cancelled one."""
+    from mini_infer_amd import ContinuousScheduler, ModelRunner, Request, SamplingParams
+
+    cfg, block, weights, folder = _folder(tmp_path, "B", 62)
+    prompts = [tiny.random_tokens(cfg, n, seed=20 + n) for n in (3, 40, 17, 64, 9, 31)]
+    # an end-of-sequence id that greedy decoding of the first prompts runs into after a few tokens
+    greedy = _plain_greedy(cfg, weights, prompts[1], 10)
+    eos = greedy[4]
+    limits = [9, 30, 1, 12, 2, 25]
+    params = [SamplingParams(), SamplingParams(), SamplingParams(temperature=0.9, seed=3),
+              SamplingParams(temperature=0.7, seed=4, top_k=40), SamplingParams(), SamplingParams(ignore_eos=True)]
+
+    def run(async_sampling, num_blocks):
+        runner = ModelRunner.from_pretrained(folder, dtype="float32", num_blocks=num_blocks, block_size=block)
+        scheduler = ContinuousScheduler(runner, max_concurrent=4, chunk_size=16, max_num_batched_tokens=24,
+                                        decode_headroom_blocks=0, eos_token_id=eos, async_sampling=async_sampling)
+        assert scheduler.async_sampling is async_sampling
+        results = scheduler.run_all([Request(p, sp, n) for p, sp, n in zip(prompts, params, limits)])
+        assert runner.num_free_blocks() == num_blocks and not scheduler.has_work()
+        runner.cache.check()
+        return [(r.tokens, r.finish_reason) for r in results], scheduler.stats
+
+    for num_blocks in (64, 9):  # plenty of pages; so few that requests are preempted and recomputed
+        late, late_stats = run(True, num_blocks)
+        at_once, _ = run(False, num_blocks)
+        assert late == at_once, f"{num_blocks} pages"
+        if num_blocks == 9:
+            assert late_stats["preemptions"] >= 1
+    assert at_once[1] == (greedy[:4], "stop")  # the end-of-sequence id is not emitted
+    assert at_once[2][1] == "length" and len(at_once[2][0]) == 1
+    assert len(at_once[5][0]) == 25  # ignore_eos runs to its length
+    # streaming and cancelling while ids are in flight
+    runner = ModelRunner.from_pretrained(folder, dtype="float32", num_blocks=64, block_size=block)
+    scheduler = ContinuousScheduler(runner, async_sampling=True)
+    keep = scheduler.submit(Request(prompts[0], SamplingParams(ignore_eos=True), 8))
+    drop = scheduler.submit(Request(prompts[2], SamplingParams(ignore_eos=True), 50))
+    streamed = []
+    for step in keep.stream():
+        streamed += list(step.tokens)
+        if len(streamed) == 3:
+            drop.cancel()
+    assert streamed == keep.wait().tokens and len(streamed) == 8
+    assert drop.wait().finish_reason == "cancelled" and runner.num_free_blocks() == 64
+
+
 def test_command_line_generates(tmp_path):
     cfg, block, weights, folder = _folder(tmp_path, "A", 54)
     prompt = tiny.random_tokens(cfg, 6, seed=1)
