@@ -30,6 +30,7 @@ def _add_engine_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--max-num-batched-tokens", type=int, default=2048)
     parser.add_argument("--chunk-size", type=int, default=256)
     parser.add_argument("--decode-headroom-blocks", type=int, default=8)
+    parser.add_argument("--trace-out", default=None, help="write a Chrome trace of the steps to this file")
 
 
 def _generate(args: argparse.Namespace) -> int:
@@ -54,6 +55,7 @@ def _generate(args: argparse.Namespace) -> int:
         chunk_size=args.chunk_size,
         decode_headroom_blocks=args.decode_headroom_blocks,
         seed=args.seed,
+        trace_out=args.trace_out,
     )
     params = SamplingParams(
         temperature=args.temperature,

@@ -36,6 +36,7 @@ class LLM:
         decode_headroom_blocks: int = DEFAULT_DECODE_HEADROOM_BLOCKS,
         seed: int = 0,
         async_sampling: bool | None = None,
+        trace_out: str | None = None,
     ) -> None:
         self.runner = ModelRunner.from_pretrained(
             model,
@@ -57,6 +58,7 @@ class LLM:
             tokenizer=self.tokenizer,
             base_seed=seed,
             async_sampling=async_sampling,
+            trace_out=trace_out,
         )
 
     def generate(
@@ -73,4 +75,6 @@ class LLM:
         if len(sampling_params) != len(prompts):
             raise ValueError("one SamplingParams per prompt (or one for all)")
         requests = [Request(p, sp, max_tokens) for p, sp in zip(prompts, sampling_params)]
-        return self.scheduler.run_all(requests)
+        results = self.scheduler.run_all(requests)
+        self.scheduler.write_trace()
+        return results

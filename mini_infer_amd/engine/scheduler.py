@@ -35,6 +35,7 @@ from __future__ import annotations
 
 import collections
 import dataclasses
+import json
 import threading
 import time
 from typing import Any, Callable, Iterable, Iterator, Sequence
@@ -151,6 +152,7 @@ class ContinuousScheduler:
         base_seed: int = 0,
         sampler: Callable[..., list[int]] | None = None,
         async_sampling: bool | None = None,
+        trace_out: str | None = None,
     ) -> None:
         if max_concurrent <= 0 or chunk_size <= 0 or max_num_batched_tokens <= 0:
             raise ValueError("max_concurrent, chunk_size and max_num_batched_tokens must be positive")
@@ -188,6 +190,12 @@ class ContinuousScheduler:
         self._stop = threading.Event()
         self._crashed: BaseException | None = None
         self.stats = {"steps": 0, "preemptions": 0, "tokens_run": 0, "rejected": 0}
+        # A timeline of the steps in the Chrome trace-event format, as the reference records
+        # it (scheduler/continuous_scheduler.py:223-229, :502-527): one duration event per
+        # step that ran the model, written by `stop()` or `write_trace()`.
+        self.trace_out = trace_out
+        self._trace_events: list[dict[str, Any]] | None = [] if trace_out is not None else None
+        self._trace_start: float | None = None
 
     # -- submitting -----------------------------------------------------------
 
@@ -266,6 +274,7 @@ class ContinuousScheduler:
     def stop(self) -> None:
         thread = self._thread
         if thread is None:
+            self.write_trace()
             return
         self._stop.set()
         thread.join()
@@ -275,6 +284,35 @@ class ContinuousScheduler:
         self._running.clear()
         self._waiting.clear()
         self._pending = None
+        self.write_trace()
+
+    def write_trace(self) -> None:
+        """Write the steps recorded so far to `trace_out` (nothing without it)."""
+        if self._trace_events is not None and self.trace_out is not None:
+            with open(self.trace_out, "w") as f:
+                json.dump({"traceEvents": self._trace_events}, f)
+
+    def _record_step(self, started: float, entries: list[StepEntry]) -> None:
+        """One "X" event: host time from building the batch to the end of the step's
+        bookkeeping, with the number of requests, the tokens run and the kind of step
+        (`prefill`: portions of prompts only, `decode`: single tokens only, else `mixed`)."""
+        if self._trace_events is None:
+            return
+        if self._trace_start is None:
+            self._trace_start = started
+        single = sum(1 for e in entries if len(e.tokens) == 1 and e.want)
+        phase = "decode" if single == len(entries) else ("prefill" if single == 0 else "mixed")
+        self._trace_events.append(
+            {
+                "name": "step",
+                "ph": "X",
+                "ts": (started - self._trace_start) * 1e6,
+                "dur": (time.perf_counter() - started) * 1e6,
+                "pid": 0,
+                "tid": 0,
+                "args": {"B": len(entries), "phase": phase, "total_q": sum(len(e.tokens) for e in entries)},
+            }
+        )
 
     def _engine_loop(self) -> None:
         try:
@@ -294,6 +332,7 @@ class ContinuousScheduler:
 
     def step(self) -> bool:
         """Admit, build one batch, run it, sample, finish.  False when there was nothing to do."""
+        started = time.perf_counter()
         self._cancel_pending()
         self._admit_waiting()
         if not self._running:
@@ -342,6 +381,7 @@ class ContinuousScheduler:
                     if running.state != RequestState.DONE:
                         self._accept_token(running, int(token))
         self._reap_done()
+        self._record_step(started, entries)
         return True
 
     # -- asynchronous sampling ---------------------------------------------------------------

@@ -287,3 +287,29 @@ def test_load_stats_counts_queues_and_pages():
         handle.cancel()
     sched.step()
     assert sched.load_stats().kv_cache_usage == 0.0
+
+
+def test_trace_out_holds_one_event_per_step_with_its_kind_and_sizes(tmp_path):
+    # one duration event per step that ran the model, as the reference records them
+    # (scheduler/continuous_scheduler.py:502-527): B, phase, total_q
+    path = tmp_path / "steps.json"
+    runner = FakeRunner()
+    sched = make(runner, chunk_size=4, max_num_batched_tokens=6, trace_out=str(path))
+    handles = [sched.submit(Request(prompt(n, n), SamplingParams(), max_tokens=3)) for n in (3, 7)]
+    while sched.step():
+        pass
+    for handle in handles:
+        handle.wait()
+    sched.stop()  # no thread was started: only writes the trace
+    import json
+
+    events = json.loads(path.read_text())["traceEvents"]
+    assert len(events) == len(runner.steps) == sched.stats["steps"]
+    assert [e["args"]["B"] for e in events] == [len(s) for s in runner.steps]
+    assert [e["args"]["total_q"] for e in events] == [sum(n for _, n, _ in s) for s in runner.steps]
+    # step 0: both prompts' first portions (3 whole + 3 of 7); step 1: a decoded token beside a portion
+    assert events[0]["args"]["phase"] == "prefill"
+    assert events[1]["args"]["phase"] == "mixed"
+    assert events[-1]["args"]["phase"] == "decode"
+    assert all(e["ph"] == "X" and e["name"] == "step" and e["dur"] >= 0 for e in events)
+    assert events[0]["ts"] == 0 and all(a["ts"] <= b["ts"] for a, b in zip(events, events[1:]))
