@@ -466,6 +466,28 @@ def test_paged_attention_finds_one_far_key_and_respects_edges(mode, dtype):
         assert np.abs(out.double().cpu().numpy() - expected)[rows].max() < _tol(dtype, 2)
 
 
+def test_paged_attention_long_context_in_many_key_ranges():
+    """One token over 9,000 keys of one head: the matrix-core kernel cuts them into more
+    ranges than for short contexts; a planted key in the first, a middle and the last
+    range is found, and an unplanted case matches the plain model."""
+    from mini_infer_amd import ops
+
+    head_dim, page_size, length = 128, 16, 9000
+    assert min(32, ops.attention_splits(1, length, target=256, min_keys=128)) == 32
+    for spot in (3, 4500, 8999):
+        case = _paged_case(torch.bfloat16, 4, 1, head_dim, page_size, [length], [1], seed=spot, v_transposed=True)
+        q = case["qs"][0][0, 2].float()  # the third of the four heads that share the keys
+        page = case["block_table"][0, spot // page_size].item()
+        case["k_pages"][page, 0, spot % page_size] = (q * 2.0).bfloat16().to(DEV)
+        out = _attend(case, 4, 1, head_dim, 1.0, None, length)
+        value = case["vs"][0][spot, 0].float()
+        assert (out[0, 2 * head_dim : 3 * head_dim].float().cpu() - value).abs().max() < 2e-2, spot
+    case = _paged_case(torch.bfloat16, 4, 1, head_dim, page_size, [length], [1], seed=11, v_transposed=True)
+    out = _attend(case, 4, 1, head_dim, 0.05, None, length)
+    expected = _attention_expected(case, 0.05, None)
+    assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(torch.bfloat16, 2)
+
+
 def test_kernels_refuse_what_they_do_not_take():
     from mini_infer_amd import ops
     from mini_infer_amd.exceptions import KernelShapeError
