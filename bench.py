@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--serving]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--serving] [--reference-workload]
 
 Default workload: the layer sizes of Llama 3.1 8B with random bfloat16 weights
 made on the device, a batch of 8 requests with 2,048-token uniform-random prompts,
@@ -146,6 +146,68 @@ def measure_serving(dtype: str) -> dict:
     }
 
 
+def measure_reference_workload(dtype: str) -> dict:
+    """The workload the reference publishes numbers for (docs/benchmarks/
+    2026-11-05-model-metrics.md:19-41; scripts/bench/modal_model_metrics.py:58-62, :239-252):
+    1,024-token prompts, 128 greedy tokens, 2,048 pages of 16, 16 seats.  Time to the first
+    token and decode speed of one request at a time (median of 5), then 16 requests that
+    start together.  Here: Llama-3.1-8B layer sizes with random weights, prompts of random
+    ids (no request stops early), and up to 4,096 tokens a step, which is what a step of the
+    reference can carry in this setting (16 requests x its chunk of 256 each; it has no
+    budget over all requests)."""
+    import statistics
+
+    import numpy as np
+    import torch
+
+    from mini_infer_amd import ContinuousScheduler, ModelRunner, Request, SamplingParams
+
+    prompt_len, new_tokens, concurrency = 1024, 128, 16
+    runner = ModelRunner.from_random(
+        LLAMA_31_8B, seed=0, dtype=dtype, num_blocks=2048, block_size=BLOCK_SIZE, max_concurrent=concurrency
+    )
+    scheduler = ContinuousScheduler(runner, max_concurrent=concurrency, chunk_size=4096, max_num_batched_tokens=4096)
+    rng = np.random.default_rng(5)
+
+    def request() -> Request:
+        ids = rng.integers(0, LLAMA_31_8B["vocab_size"], size=prompt_len).tolist()
+        return Request(ids, SamplingParams(ignore_eos=True), new_tokens)
+
+    def timed(requests: list) -> list[dict]:
+        """Drive the engine from here; per request: submit, first token and last token times, tokens."""
+        handles, marks = [], []
+        for r in requests:
+            marks.append({"submit": time.perf_counter(), "first": None, "last": None, "tokens": 0})
+            handles.append(scheduler.submit(r))
+        while not all(h.done() for h in handles):
+            scheduler.step()
+            now = time.perf_counter()
+            for h, mark in zip(handles, marks):
+                tokens = sum(1 for step in h.steps() if step.finish_reason is None)
+                if tokens > mark["tokens"]:
+                    mark["tokens"], mark["last"] = tokens, now
+                    if mark["first"] is None:
+                        mark["first"] = now
+        return marks
+
+    timed([request() for _ in range(2)])  # warm-up: graphs of the buckets recorded
+    timed([request() for _ in range(concurrency)])
+    single = [timed([request()])[0] for _ in range(5)]
+    torch.cuda.synchronize()
+    batch = timed([request() for _ in range(concurrency)])
+    torch.cuda.synchronize()
+    seconds = max(m["last"] for m in batch) - min(m["submit"] for m in batch)
+    return {
+        "prompt_tokens": prompt_len,
+        "new_tokens": new_tokens,
+        "tokens_per_step": 4096,
+        "ttft_ms": round(statistics.median((m["first"] - m["submit"]) * 1e3 for m in single), 2),
+        "decode_tok_s": round(statistics.median((m["tokens"] - 1) / (m["last"] - m["first"]) for m in single), 1),
+        "throughput_tok_s_16": round(sum(m["tokens"] for m in batch) / seconds, 1),
+        "ttft_at_16_ms": round(statistics.median((m["first"] - m["submit"]) * 1e3 for m in batch), 1),
+    }
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -161,6 +223,11 @@ def main() -> int:
     parser.add_argument(
         "--serving", action="store_true",
         help="also run 32 concurrent requests through the scheduler at Llama-3.2-3B sizes (adds a 'serving' entry)",
+    )
+    parser.add_argument(
+        "--reference-workload", action="store_true",
+        help="also run the workload the reference publishes numbers for (1,024-token prompts, 128 tokens, "
+        "1 request and 16 at once; adds a 'reference_workload' entry)",
     )
     args = parser.parse_args()
     if args.gpus != 1:
@@ -330,6 +397,10 @@ def main() -> int:
         del runner
         torch.cuda.empty_cache()
         line["serving"] = measure_serving(args.dtype)
+    if args.reference_workload:
+        runner = None
+        torch.cuda.empty_cache()
+        line["reference_workload"] = measure_reference_workload(args.dtype)
     print(json.dumps(line), flush=True)
     return 0
 
