@@ -70,6 +70,34 @@ def test_norm_part(dtype):
     assert np.abs(out.float().cpu().numpy() - expected).max() < (1e-5 if dtype == "float32" else 4e-2)
 
 
+def test_position_part():
+    """The rotary part alone, built through the registry: the llama3 rescale of the table and
+    the angles in float32 as the plain model makes them, at positions up to the model's reach;
+    one table per step, shared by every layer that asks."""
+    from mini_infer_amd.registry import POSITION_ENCODINGS
+
+    llama3 = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}
+    for desc, table in (
+        ({"kind": "rotary", "head_dim": 128, "theta": 500000.0, "llama3": llama3},
+         pl.inv_freq_llama3(pl.inv_freq_default(128, 500000.0), 8.0, 1.0, 4.0, 8192)),
+        ({"kind": "rotary", "head_dim": 48, "theta": 100.0}, pl.inv_freq_default(48, 100.0)),
+        ({"kind": "rotary", "head_dim": 48, "theta": 100.0, "rotary_dim": 16}, pl.inv_freq_default(16, 100.0)),
+    ):
+        part = POSITION_ENCODINGS.lookup("rotary")(desc, torch.bfloat16, DEV)
+        assert part.param_specs("x.") == {}
+        ours = part.inv_freq.cpu().numpy()
+        assert ours.dtype == np.float32 and np.allclose(ours, table, rtol=5e-7, atol=0)  # an ulp or two of the power
+        positions = [0, 1, 2, 8191, 8192, 131071, 5, 70000]
+        ctx = _context(positions, [0, len(positions)], [131072])
+        cos, sin = part.tables(ctx)
+        assert cos.dtype == torch.float32 and cos.shape == (len(positions), len(table))
+        want_cos, want_sin = pl.rope_tables(np.array(positions), ours)
+        # the angle is one float32 product, here as there; cos and sin of it within float32 rounding
+        assert np.abs(cos.cpu().numpy() - want_cos[:, : len(table)]).max() < 2e-6
+        assert np.abs(sin.cpu().numpy() - want_sin[:, : len(table)]).max() < 2e-6
+        assert part.tables(ctx)[0] is cos  # made once a step
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_feed_forward_part(dtype):
     from mini_infer_amd.registry import FEED_FORWARDS
