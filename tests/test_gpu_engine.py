@@ -152,6 +152,57 @@ def test_attention_part_in_two_portions(dtype, window):
     assert np.abs(got - expected).max() < (2e-5 if dtype == "float32" else 4e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_block_part_arranges_norms_mixer_and_feed_forward_around_the_residual(dtype):
+    """The pre-norm block alone, built through the registry: what comes in still to be added
+    is added by its first norm, the mixer's output by its second, and its own feed-forward
+    output goes out unadded (models/blocks/transformer_block.py:95-120)."""
+    from mini_infer_amd.parts import LayerCache
+    from mini_infer_amd.registry import BLOCKS
+
+    hidden, heads, kv_heads, head_dim, inter, page, eps, n = 40, 6, 2, 16, 56, 4, 3e-6, 9
+    desc = {
+        "kind": "pre_norm",
+        "norm": {"kind": "rms_norm", "hidden_size": hidden, "eps": eps},
+        "mixer": {"kind": "gqa_attention", "hidden_size": hidden, "num_heads": heads, "num_kv_heads": kv_heads,
+                  "head_dim": head_dim, "window": None,
+                  "position": {"kind": "rotary", "head_dim": head_dim, "theta": 100.0}},
+        "feed_forward": {"kind": "swiglu", "hidden_size": hidden, "intermediate_size": inter},
+        "names": {"mixer_norm": "n1.", "mixer": "att.", "ffn_norm": "n2.", "feed_forward": "ff."},
+    }
+    block = BLOCKS.lookup("pre_norm")(desc, TORCH[dtype], DEV, {})
+    rng = np.random.default_rng(4)
+    shapes = {"n1.weight": (hidden,), "n2.weight": (hidden,), "att.q_proj.weight": (heads * head_dim, hidden),
+              "att.k_proj.weight": (kv_heads * head_dim, hidden), "att.v_proj.weight": (kv_heads * head_dim, hidden),
+              "att.o_proj.weight": (hidden, heads * head_dim), "ff.gate_proj.weight": (inter, hidden),
+              "ff.up_proj.weight": (inter, hidden), "ff.down_proj.weight": (hidden, inter)}
+    assert set(block.param_specs("L.")) == {"L." + name for name in shapes}
+    w = {name: tiny.bf16_round(1 + rng.standard_normal(s) / 10 if len(s) == 1 else rng.standard_normal(s) / 6)
+         for name, s in shapes.items()}
+    block.load_params("L.", lambda name: torch.from_numpy(w[name[2:]]).to(TORCH[dtype]).to(DEV))
+    x = tiny.bf16_round(rng.standard_normal((n, hidden)))
+    incoming = tiny.bf16_round(rng.standard_normal((n, hidden)))
+    # plain: the residual takes the incoming piece, then the mixer's; the feed-forward's stays apart
+    cos, sin = pl.rope_tables(np.arange(n), pl.inv_freq_default(head_dim, 100.0))
+    stream = x + incoming
+    mixed, _ = pl.attention_layer(pl.rms_norm(stream, w["n1.weight"], eps), w["att.q_proj.weight"],
+                                  w["att.k_proj.weight"], w["att.v_proj.weight"], w["att.o_proj.weight"], cos, sin,
+                                  heads, kv_heads, head_dim, None)
+    stream = stream + mixed
+    out = pl.swiglu(pl.rms_norm(stream, w["n2.weight"], eps), w["ff.gate_proj.weight"], w["ff.up_proj.weight"],
+                    w["ff.down_proj.weight"])
+    cache = LayerCache(group=0, k_pages=torch.zeros((4, kv_heads, page, head_dim), dtype=TORCH[dtype], device=DEV),
+                       v_pages=torch.zeros((4, kv_heads, page, head_dim), dtype=TORCH[dtype], device=DEV))
+    table = [[2, 0, 3]]
+    slots = [table[0][p // page] * page + p % page for p in range(n)]
+    residual = torch.from_numpy(x).float().to(DEV)
+    delta = torch.from_numpy(incoming).to(TORCH[dtype]).to(DEV)
+    got = block.forward(delta, residual, _context(list(range(n)), [0, n], [n], slots, table), cache)
+    tol = 3e-5 if dtype == "float32" else 6e-2
+    assert np.abs(residual.cpu().numpy() - stream).max() < tol
+    assert np.abs(got.float().cpu().numpy() - out).max() < tol
+
+
 # -- generation through the entry points ---------------------------------------------
 
 
