@@ -694,3 +694,106 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path, dtype):
     finally:
         ARCHITECTURES.unregister("ToyStateTestLM")
         MIXERS.unregister("decaying_sum")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_routed_feed_forward_registers_builds_and_steps(tmp_path, dtype):
+    """A feed-forward defined here that routes each token to one of two small experts (router
+    logits and their softmax in float32) takes the place of layer 0's SwiGLU: registered,
+    built from a layer description, loaded by name, stepped in mixed batches.  The layer
+    beside it keeps its dense feed-forward: one model, two kinds."""
+    import copy
+    import dataclasses
+
+    from mini_infer_amd.engine import ModelRunner
+    from mini_infer_amd.models.spec import LayerSpec
+    from mini_infer_amd.parts import FeedForward, ParamSpec
+    from mini_infer_amd.registry import ARCHITECTURES, FEED_FORWARDS
+
+    hidden, inner = tiny.TINY_A["hidden_size"], 24
+
+    class OneOfTwo(FeedForward):
+        def param_specs(self, prefix):
+            specs = {prefix + "router.weight": ParamSpec((2, hidden))}
+            for e in range(2):
+                specs[prefix + f"experts.{e}.up.weight"] = ParamSpec((inner, hidden))
+                specs[prefix + f"experts.{e}.down.weight"] = ParamSpec((hidden, inner))
+            return specs
+
+        def load_params(self, prefix, get):
+            self.router = get(prefix + "router.weight").float()
+            self.up = [get(prefix + f"experts.{e}.up.weight") for e in range(2)]
+            self.down = [get(prefix + f"experts.{e}.down.weight") for e in range(2)]
+
+        def forward(self, x, ctx):
+            share = torch.softmax(x.float() @ self.router.T, dim=-1)
+            choice = share.argmax(dim=-1)
+            out = torch.zeros_like(x)
+            for e in range(2):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    inside = torch.nn.functional.silu((x[rows].float() @ self.up[e].float().T)).to(x.dtype)
+                    result = (inside.float() @ self.down[e].float().T) * share[rows, e : e + 1]
+                    out[rows] = result.to(x.dtype)
+            return out
+
+    FEED_FORWARDS.register("one_of_two", lambda desc, dtype_, device, shared=None: OneOfTwo(dtype_, device))
+
+    def with_toy(spec):
+        layers = list(spec.layers)
+        block = copy.deepcopy(layers[0].block)
+        block["feed_forward"] = {"kind": "one_of_two"}
+        layers[0] = LayerSpec(layers[0].prefix, block)
+        return dataclasses.replace(spec, layers=layers)
+
+    _register_variant("ToyRoutedTestLM", with_toy)
+    try:
+        cfg = dict(tiny.TINY_A, architectures=["ToyRoutedTestLM"])
+        weights = tiny.make_weights(cfg, 63)
+        for n in ("gate", "up", "down"):
+            del weights[f"model.layers.0.mlp.{n}_proj.weight"]
+        rng = np.random.default_rng(6)
+        p = "model.layers.0.mlp."
+        weights[p + "router.weight"] = tiny.bf16_round(rng.standard_normal((2, hidden)) * 2)  # clear choices
+        for e in range(2):
+            weights[p + f"experts.{e}.up.weight"] = tiny.bf16_round(rng.standard_normal((inner, hidden)) / 6)
+            weights[p + f"experts.{e}.down.weight"] = tiny.bf16_round(rng.standard_normal((hidden, inner)) / 6)
+        folder = tiny.write_model_dir(tmp_path / "routed", cfg, weights)
+        experts_used = set()
+
+        def plain(tokens):
+            eps = cfg["rms_norm_eps"]
+            r = pl.embedding(weights["model.embed_tokens.weight"], np.array(tokens))
+            cos, sin = pl.rope_tables(np.arange(len(tokens)), pl.config_inv_freq(cfg))
+            for layer in range(2):
+                q = f"model.layers.{layer}."
+                a, _ = pl.attention_layer(
+                    pl.rms_norm(r, weights[q + "input_layernorm.weight"], eps),
+                    *(weights[q + f"self_attn.{n}_proj.weight"] for n in "qkvo"), cos, sin, 4, 2, 16)
+                r = r + a
+                h = pl.rms_norm(r, weights[q + "post_attention_layernorm.weight"], eps)
+                if layer == 1:
+                    r = r + pl.swiglu(h, *(weights[q + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+                    continue
+                share = [pl.softmax(row) for row in h @ weights[p + "router.weight"].astype(np.float64).T]
+                rows = []
+                for row, s in zip(h, share):
+                    e = int(np.argmax(s))
+                    experts_used.add(e)
+                    inside = pl.silu(weights[p + f"experts.{e}.up.weight"].astype(np.float64) @ row)
+                    rows.append(weights[p + f"experts.{e}.down.weight"].astype(np.float64) @ inside * s[e])
+                r = r + np.array(rows)
+            return pl.rms_norm(r, weights["model.norm.weight"], eps) @ weights["model.embed_tokens.weight"].astype(np.float64).T
+
+        requests = {f"r{i}": tiny.random_tokens(cfg, n, seed=10 + i) for i, n in enumerate((18, 7, 13, 22))}
+        expected = {rid: plain(t) for rid, t in requests.items()}
+        assert experts_used == {0, 1}
+        runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=24, block_size=4, max_concurrent=4)
+        assert not runner.model.graph_safe  # the toy part does not say it is: its steps are not recorded
+        got = ru.run_schedule(runner, requests, ru.schedule_mixed(requests, seed=5, tail=4))
+        for rid in requests:
+            ru.assert_close(got[rid], expected[rid], dtype, f"routed {rid}")
+        runner.cache.check()
+    finally:
+        ARCHITECTURES.unregister("ToyRoutedTestLM")
+        FEED_FORWARDS.unregister("one_of_two")
