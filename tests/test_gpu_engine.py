@@ -797,3 +797,75 @@ def test_toy_routed_feed_forward_registers_builds_and_steps(tmp_path, dtype):
     finally:
         ARCHITECTURES.unregister("ToyRoutedTestLM")
         FEED_FORWARDS.unregister("one_of_two")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_position_encoding_registers_builds_and_steps(tmp_path, dtype):
+    """Another position encoding defined here (rotation angles of positions squeezed by a
+    factor, with tables it makes itself in torch) is named in the mixer's description of
+    layer 1 and used by the framework's attention part as it is."""
+    import copy
+    import dataclasses
+
+    from mini_infer_amd.engine import ModelRunner
+    from mini_infer_amd.models.spec import LayerSpec
+    from mini_infer_amd.parts import PositionEncoding
+    from mini_infer_amd.registry import ARCHITECTURES, POSITION_ENCODINGS
+
+    squeeze = 4.0
+
+    class SqueezedRotary(PositionEncoding):
+        interleaved = False
+
+        def __init__(self, desc, dtype_, device):
+            super().__init__(dtype_, device)
+            self.rotary_dim = int(desc["head_dim"])
+            table = pl.inv_freq_default(self.rotary_dim, float(desc["theta"]))
+            self.inv_freq = torch.from_numpy(table).to(device)
+
+        def tables(self, ctx):
+            angle = (ctx.positions.float() / squeeze)[:, None] * self.inv_freq[None, :]
+            return torch.cos(angle).contiguous(), torch.sin(angle).contiguous()
+
+    POSITION_ENCODINGS.register("squeezed_rotary", lambda desc, dtype_, device, shared=None: SqueezedRotary(desc, dtype_, device))
+
+    def with_toy(spec):
+        layers = list(spec.layers)
+        block = copy.deepcopy(layers[1].block)
+        block["mixer"]["position"] = dict(block["mixer"]["position"], kind="squeezed_rotary")
+        layers[1] = LayerSpec(layers[1].prefix, block)
+        return dataclasses.replace(spec, layers=layers)
+
+    _register_variant("ToyPositionTestLM", with_toy)
+    try:
+        cfg = dict(tiny.TINY_A, architectures=["ToyPositionTestLM"])
+        weights = tiny.make_weights(cfg, 64)
+        folder = tiny.write_model_dir(tmp_path / "squeezed", cfg, weights)
+
+        def plain(tokens):
+            eps = cfg["rms_norm_eps"]
+            r = pl.embedding(weights["model.embed_tokens.weight"], np.array(tokens))
+            for layer in range(2):
+                positions = np.arange(len(tokens)) / (squeeze if layer == 1 else 1.0)
+                cos, sin = pl.rope_tables(positions, pl.config_inv_freq(cfg))
+                q = f"model.layers.{layer}."
+                a, _ = pl.attention_layer(
+                    pl.rms_norm(r, weights[q + "input_layernorm.weight"], eps),
+                    *(weights[q + f"self_attn.{n}_proj.weight"] for n in "qkvo"), cos, sin, 4, 2, 16)
+                r = r + a
+                r = r + pl.swiglu(pl.rms_norm(r, weights[q + "post_attention_layernorm.weight"], eps),
+                                  *(weights[q + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            return pl.rms_norm(r, weights["model.norm.weight"], eps) @ weights["model.embed_tokens.weight"].astype(np.float64).T
+
+        requests = {f"s{i}": tiny.random_tokens(cfg, n, seed=20 + i) for i, n in enumerate((25, 6, 15))}
+        expected = {rid: plain(t) for rid, t in requests.items()}
+        # the squeeze matters: with plain positions in layer 1 the logits are others
+        assert np.abs(expected["s0"] - pl.llama_logits(cfg, weights, np.array(requests["s0"]))).max() > 1e-2
+        runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=24, block_size=4, max_concurrent=3)
+        got = ru.run_schedule(runner, requests, ru.schedule_mixed(requests, seed=6, tail=5))
+        for rid in requests:
+            ru.assert_close(got[rid], expected[rid], dtype, f"squeezed {rid}")
+        runner.cache.check()
+    finally:
+        ARCHITECTURES.unregister("ToyPositionTestLM")
+        POSITION_ENCODINGS.unregister("squeezed_rotary")
