@@ -869,3 +869,48 @@ def test_toy_position_encoding_registers_builds_and_steps(tmp_path, dtype):
     finally:
         ARCHITECTURES.unregister("ToyPositionTestLM")
         POSITION_ENCODINGS.unregister("squeezed_rotary")
+
+
+_LONG = {}
+
+
+def _long_case():
+    """8,300 tokens of tiny B and their plain logits at the places the test looks at (made once: the
+    plain model takes half a minute at this length)."""
+    if not _LONG:
+        cfg = dict(tiny.TINY_B, max_position_embeddings=16384)
+        weights = tiny.make_weights(cfg, 57)
+        tokens = tiny.random_tokens(cfg, 8300, seed=12)
+        _LONG.update(cfg=cfg, weights=weights, tokens=tokens, expected=pl.llama_logits(cfg, weights, np.array(tokens)))
+    return _LONG
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_context_past_eight_thousand_keys(tmp_path, dtype):
+    """8,288 tokens in portions of 2,048, then 12 tokens one by one, where single tokens'
+    keys are cut into the many ranges of long contexts.  (In float32 a page read from the
+    wrong place anywhere in the 8,000 moves the logits by far more than the tolerance; for
+    bfloat16 the kernel tests plant single far keys.)"""
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+
+    case = _long_case()
+    tokens, expected = case["tokens"], case["expected"]
+    folder = tiny.write_model_dir(tmp_path / "long", case["cfg"], case["weights"])
+    runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=len(tokens) // 16 + 2, block_size=16)
+    got, fed, whole = [], 0, len(tokens) - 12
+    while fed < whole:
+        count = min(2048, whole - fed)
+        want = list(range(count - 5, count))  # the last five places of each portion
+        got.append((fed + count - 5, runner.step([StepEntry("r", tokens[fed : fed + count], want)]).cpu().numpy()))
+        fed += count
+    for _ in range(12):
+        got.append((fed, runner.step([StepEntry("r", tokens[fed : fed + 1], [0])]).cpu().numpy()))
+        fed += 1
+    # as everywhere, the bfloat16 bound is relative to the largest logit of the whole sequence:
+    # the engine's rows take their places in a copy of the plain model's
+    seen = expected.copy()
+    for start, rows in got:
+        seen[start : start + len(rows)] = rows
+    ru.assert_close(seen, expected, dtype, "long context")
+    runner.free_request("r")
+    runner.cache.check()
