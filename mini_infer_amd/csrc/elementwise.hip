@@ -105,19 +105,51 @@ extern "C" int mi_take_device_tokens(int* ids, const int* from_rows, const int* 
 //   s = residual[r] + delta[r]           (float32; stored back unless `rows` is given)
 //   out[b] = weight * s * rsqrt(mean(s^2) + eps)
 // One block per output row; with `rows`, output row b reads input row rows[b].
+// The delta may come in pieces: `partials` [num_partials][all rows][hidden] float32, the
+// sums of a product over ranges of K (gemm_mid_bf16.hip); they are added in order and
+// rounded to T, which gives the delta the product would have written itself.
 // ---------------------------------------------------------------------------
 
 template <typename T, int VEC>
 __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
     const T* __restrict__ delta, float* __restrict__ residual, const T* __restrict__ weight,
-    T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps) {
+    T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps,
+    const float* __restrict__ partials, int num_partials, int64_t partial_stride) {
   __shared__ float scratch[16];
   const int b = blockIdx.x;
   const int64_t r = rows ? rows[b] : b;
   float* res = residual + r * hidden;
   const T* dl = delta ? delta + r * hidden : nullptr;
+  const float* pt = partials ? partials + r * hidden : nullptr;
   T* o = out + (int64_t)b * hidden;
-  const bool store_sum = (rows == nullptr) && (delta != nullptr);
+  const bool has_delta = dl != nullptr || pt != nullptr;
+  const bool store_sum = (rows == nullptr) && has_delta;
+  // 4 consecutive values of the delta at i (VEC == 4 paths)
+  auto delta4 = [&](int i, float* d) {
+    if (pt) {
+      float sum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+      for (int p = 0; p < num_partials; ++p) {  // the loads do not wait for one another
+        float piece[4];
+        load4(pt + (int64_t)p * partial_stride + i, piece);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) sum[k] += piece[k];
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) d[k] = to_f32(from_f32<T>(sum[k]));
+    } else {
+      load4(dl + i, d);
+    }
+  };
+  auto delta1 = [&](int i) -> float {
+    if (pt) {
+      float sum = 0.f;
+#pragma unroll 8
+      for (int p = 0; p < num_partials; ++p) sum += pt[(int64_t)p * partial_stride + i];
+      return to_f32(from_f32<T>(sum));
+    }
+    return to_f32(dl[i]);
+  };
 
   if (VEC == 4 && hidden <= (int)blockDim.x * 4) {
     // the whole row is one vector per thread: it stays in registers between the two
@@ -129,9 +161,9 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
     if (mine) {
       load4(res + i, s);
       load4(weight + i, w);
-      if (dl) {
+      if (has_delta) {
         float d[4];
-        load4(dl + i, d);
+        delta4(i, d);
 #pragma unroll
         for (int k = 0; k < 4; ++k) s[k] += d[k];
         if (store_sum) store4(res + i, s);
@@ -154,9 +186,9 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
     for (int i = threadIdx.x * 4; i < hidden; i += blockDim.x * 4) {
       float s[4];
       load4(res + i, s);
-      if (dl) {
+      if (has_delta) {
         float d[4];
-        load4(dl + i, d);
+        delta4(i, d);
 #pragma unroll
         for (int k = 0; k < 4; ++k) s[k] += d[k];
         if (store_sum) store4(res + i, s);
@@ -167,8 +199,8 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
   } else {
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
       float s = res[i];
-      if (dl) {
-        s += to_f32(dl[i]);
+      if (has_delta) {
+        s += delta1(i);
         if (store_sum) res[i] = s;
       }
       sumsq += s * s;
@@ -176,7 +208,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
   }
   const float total = block_sum(sumsq, scratch);
   const float inv = rsqrtf(total / (float)hidden + eps);
-  const bool re_add = (dl != nullptr) && !store_sum;
+  const bool re_add = has_delta && !store_sum;
 
   if (VEC == 4) {
     for (int i = threadIdx.x * 4; i < hidden; i += blockDim.x * 4) {
@@ -184,7 +216,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
       load4(res + i, s);
       if (re_add) {
         float d[4];
-        load4(dl + i, d);
+        delta4(i, d);
 #pragma unroll
         for (int k = 0; k < 4; ++k) s[k] += d[k];
       }
@@ -196,7 +228,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
   } else {
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
       float s = res[i];
-      if (re_add) s += to_f32(dl[i]);
+      if (re_add) s += delta1(i);
       o[i] = from_f32<T>(to_f32(weight[i]) * (s * inv));
     }
   }
@@ -205,31 +237,42 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
 template <typename T>
 static int add_rmsnorm_launch(const void* delta, float* residual, const void* weight, void* out,
                               const int* rows, int num_out_rows, int hidden, float eps,
+                              const float* partials, int num_partials, int64_t partial_stride,
                               hipStream_t stream) {
   if (num_out_rows == 0) return MI_OK;
   if (hidden % 4 == 0) {
     // one vector of 4 per thread and pass where the row allows: fewer dependent steps
     const int threads = min(1024, max(256, ceil_div(hidden / 4, 64) * 64));
     add_rmsnorm_kernel<T, 4><<<num_out_rows, threads, 0, stream>>>(
-        (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps);
+        (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps, partials, num_partials,
+        partial_stride);
   } else {
     add_rmsnorm_kernel<T, 1><<<num_out_rows, 256, 0, stream>>>(
-        (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps);
+        (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps, partials, num_partials,
+        partial_stride);
   }
   MI_CHECK_LAUNCH("add_rmsnorm");
   return MI_OK;
 }
 
+// `delta` (element type) or `partials` (float32 [num_partials][all rows][hidden],
+// `partial_stride` = all rows * hidden) or neither; never both.
 extern "C" int mi_add_rmsnorm(int dtype, const void* delta, float* residual, const void* weight,
                               void* out, const int* rows, int num_out_rows, int hidden, float eps,
+                              const float* partials, int num_partials, int64_t partial_stride,
                               hipStream_t stream) {
   MI_REQUIRE(num_out_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d hidden=%d",
              num_out_rows, hidden);
+  MI_REQUIRE(!(delta && partials), "add_rmsnorm: a delta or its partial sums, not both");
+  MI_REQUIRE(!partials || (num_partials >= 1 && num_partials <= 16 && partial_stride >= hidden),
+             "add_rmsnorm: bad partial sums count=%d stride=%lld", num_partials, (long long)partial_stride);
   MI_REQUIRE(eps > 0.f, "add_rmsnorm: eps must be positive, got %g", (double)eps);
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "add_rmsnorm: unknown dtype %d", dtype);
   if (dtype == MI_F32)
-    return add_rmsnorm_launch<float>(delta, residual, weight, out, rows, num_out_rows, hidden, eps, stream);
-  return add_rmsnorm_launch<bf16_t>(delta, residual, weight, out, rows, num_out_rows, hidden, eps, stream);
+    return add_rmsnorm_launch<float>(delta, residual, weight, out, rows, num_out_rows, hidden, eps, partials,
+                                     num_partials, partial_stride, stream);
+  return add_rmsnorm_launch<bf16_t>(delta, residual, weight, out, rows, num_out_rows, hidden, eps, partials,
+                                    num_partials, partial_stride, stream);
 }
 
 // ---------------------------------------------------------------------------

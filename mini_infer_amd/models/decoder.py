@@ -45,6 +45,10 @@ class DecoderModel:
             device,
             tied_to=self.embedding if spec.tie_word_embeddings else None,
         )
+        # a product whose output only ever meets norms that can add up its pieces may leave them apart
+        if self.final_norm.takes_partial_sums and all(block.takes_partial_sums for block in self.blocks):
+            for block in self.blocks:
+                block.enable_partial_sums()
 
     @property
     def graph_safe(self) -> bool:

@@ -7,6 +7,7 @@ refuses a size.  There is no CPU path: a CPU tensor is an error.
 
 from __future__ import annotations
 
+import dataclasses
 import math
 
 import torch
@@ -107,8 +108,25 @@ def take_device_tokens(ids: torch.Tensor, from_rows: torch.Tensor, source: torch
     )
 
 
+@dataclasses.dataclass
+class PartialSums:
+    """A product that has not been added up yet: `pieces` [S, T, N] float32 holds its sums
+    over S ranges of K (`linear(..., partial_ok=True)`).  Their sum in order, rounded to
+    `dtype`, is what `linear` returns otherwise; `add_rmsnorm` takes the pieces as they are
+    and adds them on its way, anything else calls `finish()`."""
+
+    pieces: torch.Tensor
+    dtype: torch.dtype
+
+    def finish(self) -> torch.Tensor:
+        total = self.pieces[0]
+        for piece in self.pieces[1:]:
+            total = total + piece
+        return total.to(self.dtype)
+
+
 def add_rmsnorm(
-    delta: torch.Tensor | None,
+    delta: torch.Tensor | PartialSums | None,
     residual: torch.Tensor,
     weight: torch.Tensor,
     eps: float,
@@ -118,6 +136,19 @@ def add_rmsnorm(
 
     Returns [T, H] (or [len(rows), H]) in the dtype of `weight`.
     """
+    pieces = None
+    if isinstance(delta, PartialSums):
+        if delta.dtype != weight.dtype:
+            raise KernelShapeError(f"partial sums for {delta.dtype} meet a norm weight of {weight.dtype}")
+        pieces, delta = delta.pieces, None
+        _need_cuda(pieces)
+        _need_contiguous("partial sums", pieces)
+        if pieces.dtype != torch.float32 or pieces.dim() != 3 or tuple(pieces.shape[1:]) != tuple(residual.shape):
+            raise KernelShapeError(
+                f"partial sums {tuple(pieces.shape)} {pieces.dtype} do not fit residual {tuple(residual.shape)}"
+            )
+        if not 1 <= pieces.shape[0] <= 16:
+            raise KernelShapeError(f"1 to 16 partial sums are taken, got {pieces.shape[0]}")
     _need_cuda(delta, residual, weight, rows)
     _need_contiguous("residual", residual)
     _need_contiguous("delta", delta)
@@ -140,7 +171,8 @@ def add_rmsnorm(
     library.check(
         lib.mi_add_rmsnorm(
             _dtype_code(weight), _ptr(delta), _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows),
-            n_out, hidden, float(eps), _stream(),
+            n_out, hidden, float(eps), _ptr(pieces), 0 if pieces is None else pieces.shape[0],
+            tokens * hidden, _stream(),
         )
     )
     return out
@@ -289,17 +321,76 @@ def skinny_gemm_takes(m: int, k: int, lda: int, ldw: int) -> bool:
     return 1 <= m <= SKINNY_MAX_ROWS and k >= 32 and k % 32 == 0 and lda % 8 == 0 and ldw % 8 == 0
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+PARTIAL_SUMS_MAX_ROWS = 64
+
+
+def partial_sums_pay(m: int, n: int, k: int) -> bool:
+    """Whether a product of these sizes is left as sums over ranges of K when its caller
+    takes them (`linear(..., partial_ok=True)`).  Measured on MI355X: with a long K
+    (4096 x 14336: 24.5 us at any number of rows up to 16, against 27 / 31 / 37 us whole at
+    1 / 8 / 16 rows, and 25 / 29 us at 32 / 64 rows against the vendor library's 34 / 41),
+    and for a 4096 x 4096 product from 12 rows on (10.3 against 11.5 us at 16 rows; 10.7 /
+    12.7 against 13 / 15 us at 32 / 64).  Wide products (many features) fill the GPU without
+    cutting K and gain nothing; with a single row the whole step ran 0.5 % slower this way
+    (270 -> 269 tok/s at Llama-3.1-8B sizes, though the product alone timed faster), at batch
+    8 / 16 / 64 it ran 1.6 / 5 / 2.8 % faster."""
+    if not 1 <= m <= PARTIAL_SUMS_MAX_ROWS or n > 8192:
+        return False
+    return (k >= 8192 and m >= 5) or (k >= 4096 and m >= 12)
+
+
+def linear_partial_sums(x: torch.Tensor, weight: torch.Tensor) -> PartialSums:
+    """`x @ weight.T` for up to 64 bfloat16 rows as float32 sums over ranges of K."""
+    _need_cuda(x, weight)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or x.dim() != 2 or weight.dim() != 2:
+        raise KernelShapeError("linear_partial_sums takes 2-D bfloat16 tensors")
+    m, k = x.shape
+    n = weight.shape[0]
+    lib = library.load()
+    if (
+        weight.shape[1] != k
+        or x.stride(1) != 1
+        or weight.stride(1) != 1
+        or not lib.mi_gemm_mid_bf16_supported(m, n, k, x.stride(0), weight.stride(0))
+    ):
+        raise KernelShapeError(
+            f"linear_partial_sums takes 1 to 64 rows, K a multiple of 32, rows aligned to 16 bytes; "
+            f"got x {tuple(x.shape)} strides {x.stride()}, weight {tuple(weight.shape)} strides {weight.stride()}"
+        )
+    ranges = lib.mi_gemm_mid_bf16_ranges(n, k)
+    if ranges < 1:
+        raise KernelShapeError("linear_partial_sums: cannot read the device's compute unit count")
+    pieces = torch.empty((ranges, m, n), dtype=torch.float32, device=x.device)
+    library.check(
+        lib.mi_gemm_mid_partial_bf16(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(pieces), m, n, k, _stream())
+    )
+    return PartialSums(pieces, torch.bfloat16)
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, partial_ok: bool = False) -> torch.Tensor | PartialSums:
     """`x @ weight.T` without bias.
 
     float32 runs the hand-written true-float32 kernel.  bfloat16 with at most 16
     rows (decode) runs the hand-written weight-streaming kernel; more rows go to
     the vendor GEMM library through torch, as the reference's engine does
     (distributed/linear.py:167, `F.linear` -> the vendor BLAS).
+    With `partial_ok` the result may come as `PartialSums` where that pays
+    (`partial_sums_pay`: up to 64 rows, few features, a long K).
     """
     if x.dtype == torch.float32:
         return gemm_f32(x, weight)
     _need_cuda(x, weight)
+    plain = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2 and weight.dim() == 2
+    plain = plain and x.stride(1) == 1 and weight.stride(1) == 1 and weight.shape[1] == x.shape[1]
+    if (
+        partial_ok
+        and plain
+        and partial_sums_pay(x.shape[0], weight.shape[0], x.shape[1])
+        and x.shape[1] % 32 == 0
+        and x.stride(0) % 8 == 0
+        and weight.stride(0) % 8 == 0
+    ):
+        return linear_partial_sums(x, weight)
     if (
         x.dtype == torch.bfloat16
         and x.dim() == 2

@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -23,7 +23,7 @@ _P = c_void_p
 _SIGNATURES: dict[str, list] = {
     "mi_embed_gather": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
     "mi_take_device_tokens": [_P, _P, _P, c_int, c_int, c_int, _P],
-    "mi_add_rmsnorm": [c_int, _P, _P, _P, _P, _P, c_int, c_int, c_float, _P],
+    "mi_add_rmsnorm": [c_int, _P, _P, _P, _P, _P, c_int, c_int, c_float, _P, c_int, c_int64, _P],
     "mi_rope_table": [_P, _P, _P, _P, c_int, c_int, _P],
     "mi_rope_kv_write": [
         c_int, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -32,6 +32,9 @@ _SIGNATURES: dict[str, list] = {
     "mi_silu_mul": [c_int, _P, _P, c_int, c_int, _P],
     "mi_gemm_f32": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_gemm_skinny_bf16": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
+    "mi_gemm_mid_partial_bf16": [_P, c_int64, _P, c_int64, _P, c_int, c_int, c_int, _P],
+    "mi_gemm_mid_bf16_ranges": [c_int, c_int],
+    "mi_gemm_mid_bf16_supported": [c_int, c_int, c_int, c_int64, c_int64],
     "mi_gemm_skinny_swiglu_bf16": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_gemm_skinny_rope_bf16": [
         _P, c_int64, _P, c_int64, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,

@@ -89,7 +89,7 @@ class GQAttention(Mixer):
                 q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
                 v_transposed=cache.v_transposed,
             )
-            return self.out.forward(self._attend(queries, ctx, cache))
+            return self.out.forward(self._attend(queries, ctx, cache), partial_ok=self.emit_partial_sums)
         if writes_cache:
             qkv = self.qkv.forward(x)
             kv_heads, slots = self.num_kv_heads, ctx.slot_mapping[cache.group]
@@ -113,7 +113,7 @@ class GQAttention(Mixer):
                 q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
                 rotary_dim=0, interleaved=False, v_transposed=cache.v_transposed,
             )
-        return self.out.forward(self._attend(qkv, ctx, cache))
+        return self.out.forward(self._attend(qkv, ctx, cache), partial_ok=self.emit_partial_sums)
 
     def _attend(self, queries: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
         """Attention of the rotated queries (the first columns of `queries`) over the cache pages."""

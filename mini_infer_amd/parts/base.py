@@ -148,7 +148,13 @@ class Norm(Part):
     Adds `delta` (or nothing) into the float32 residual stream in place and
     returns the normalized sum in the compute dtype.  With `rows`, only those
     rows are normalized and returned, and the residual is left as it was.
+
+    `takes_partial_sums`: `delta` may also be an `ops.PartialSums` (a product whose sums
+    over ranges of K are still apart); a model lets its mixers and feed-forwards emit
+    those only if every one of its norms says it takes them.
     """
+
+    takes_partial_sums = False
 
     def forward(
         self,
@@ -164,7 +170,12 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    """Mixes tokens of one request: attention here, anything with a cache or a state."""
+    """Mixes tokens of one request: attention here, anything with a cache or a state.
+
+    `emit_partial_sums` is set by the model, never by the part: when true, `forward` may
+    return an `ops.PartialSums` instead of a tensor (parts that ignore it are fine)."""
+
+    emit_partial_sums = False
 
     def cache_needs(self) -> CacheNeeds:
         return CacheNeeds()
@@ -176,7 +187,9 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """Acts on each token alone: dense or routed experts."""
+    """Acts on each token alone: dense or routed experts.  `emit_partial_sums`: as for `Mixer`."""
+
+    emit_partial_sums = False
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
@@ -191,6 +204,14 @@ class Block(Part):
     """
 
     mixer: Mixer
+
+    # Whether every norm of the block takes `ops.PartialSums` as its delta; only if all
+    # blocks of a model and its final norm do, the model calls `enable_partial_sums()`,
+    # which lets the block's mixer and feed-forward emit them.
+    takes_partial_sums = False
+
+    def enable_partial_sums(self) -> None:
+        pass
 
     def forward(
         self,

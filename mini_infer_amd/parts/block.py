@@ -45,6 +45,14 @@ class PreNormBlock(Block):
     def graph_safe(self) -> bool:  # type: ignore[override]
         return all(part.graph_safe for _, part in self._children())
 
+    @property
+    def takes_partial_sums(self) -> bool:  # type: ignore[override]
+        return self.mixer_norm.takes_partial_sums and self.ffn_norm.takes_partial_sums
+
+    def enable_partial_sums(self) -> None:
+        self.mixer.emit_partial_sums = True
+        self.feed_forward.emit_partial_sums = True
+
     def _children(self):
         return (
             (self.names["mixer_norm"], self.mixer_norm),

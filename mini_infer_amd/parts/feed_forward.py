@@ -38,7 +38,7 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         assert self.gate_up.weight is not None, "SwiGLU used before its weights were loaded"
-        return self.down.forward(ops.linear_swiglu(x, self.gate_up.weight))
+        return self.down.forward(ops.linear_swiglu(x, self.gate_up.weight), partial_ok=self.emit_partial_sums)
 
 
 @register_feed_forward("swiglu")

@@ -45,6 +45,7 @@ class Linear(Part):
         blocks = [get(prefix + name + ".weight") for name in self.names]
         self.weight = (blocks[0] if len(blocks) == 1 else torch.cat(blocks, dim=0)).contiguous()
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, partial_ok: bool = False):
+        """`x @ weight.T`; with `partial_ok` possibly as `ops.PartialSums` for a norm to add up."""
         assert self.weight is not None, "Linear used before its weight was loaded"
-        return ops.linear(x, self.weight)
+        return ops.linear(x, self.weight, partial_ok=partial_ok)

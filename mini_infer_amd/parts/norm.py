@@ -17,6 +17,7 @@ from mini_infer_amd.registry import register_norm
 
 class RMSNorm(Norm):
     graph_safe = True
+    takes_partial_sums = True
 
     def __init__(self, hidden_size: int, eps: float, dtype: torch.dtype, device) -> None:
         super().__init__(dtype, device)

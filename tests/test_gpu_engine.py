@@ -914,3 +914,30 @@ def test_context_past_eight_thousand_keys(tmp_path, dtype):
     ru.assert_close(seen, expected, dtype, "long context")
     runner.free_request("r")
     runner.cache.check()
+
+
+def test_products_left_in_partial_sums_through_the_engine(tmp_path, monkeypatch):
+    """The tiny models never meet the sizes at which a product is left as sums over ranges of
+    K for the next norm; here the rule is made to say yes always, so that every o and down
+    product of a replay (portions, single tokens, mixed batches up to 64 rows) takes that way."""
+    from mini_infer_amd.engine import ModelRunner
+    from mini_infer_amd.ops import kernels
+
+    taken = []
+
+    def always(m, n, k):
+        taken.append((m, n, k))
+        return m <= kernels.PARTIAL_SUMS_MAX_ROWS
+
+    monkeypatch.setattr(kernels, "partial_sums_pay", always)
+    cfg, block, weights, folder = _folder(tmp_path, "B", 58)
+    requests = {f"p{i}": tiny.random_tokens(cfg, n, seed=30 + i) for i, n in enumerate((70, 33, 90, 41, 57))}
+    expected = {rid: pl.llama_logits(cfg, weights, np.array(t)) for rid, t in requests.items()}
+    runner = ModelRunner.from_pretrained(folder, dtype="bfloat16", num_blocks=20, block_size=block, max_concurrent=4)
+    for schedule in (ru.schedule_prefill_then_decode(requests, tail=8), ru.schedule_mixed(requests, seed=7, tail=6)):
+        got = ru.run_schedule(runner, requests, schedule)
+        for rid in requests:
+            ru.assert_close(got[rid], expected[rid], "bfloat16", f"partial sums {rid}")
+    rows = {m for m, _, _ in taken}
+    assert 1 in rows and any(m > 16 for m in rows) and len({(n, k) for _, n, k in taken}) == 2  # o and down
+    runner.cache.check()

@@ -126,6 +126,57 @@ def test_gemm_skinny_bf16(m, n, k):
 
 
 @pytest.mark.parametrize(
+    "m,n,k",
+    [(1, 4096, 14336), (8, 1000, 8192 + 32), (16, 4096, 4096), (17, 1003, 4096), (33, 136, 608), (64, 4096, 14336),
+     (47, 5, 32), (64, 260, 8192 - 224)],
+)
+def test_linear_in_partial_sums_then_norm_is_linear_then_norm(m, n, k):
+    """A product left as sums over ranges of K, added up by the norm that follows it: the
+    same residual and output, bit for bit, as with the pieces added first (`finish`), and the
+    product itself within float32 accumulation of the exact one; a row's pieces do not
+    depend on the other rows."""
+    from mini_infer_amd import ops
+
+    a, w = _rand(m, k, dtype=torch.bfloat16, seed=31), _rand(n, k, dtype=torch.bfloat16, seed=32, scale=0.05)
+    partial = ops.linear_partial_sums(a, w)
+    assert partial.pieces.dtype == torch.float32 and partial.pieces.shape[1:] == (m, n)
+    delta = partial.finish()
+    expected = a.double() @ w.double().T
+    assert (delta.double() - expected).abs().max() < 2.0 ** -8 * float(expected.abs().max()) + 1e-6
+    alone = ops.linear_partial_sums(a[m // 2 : m // 2 + 1].contiguous(), w)
+    assert torch.equal(alone.pieces[:, 0], partial.pieces[:, m // 2])
+    # strided activations: a slice of a wider buffer
+    wide = _rand(m, k + 8, dtype=torch.bfloat16, seed=35)
+    assert torch.equal(ops.linear_partial_sums(wide[:, :k], w).pieces, ops.linear_partial_sums(wide[:, :k].contiguous(), w).pieces)
+    weight = _rand(n, dtype=torch.bfloat16, seed=33).abs() + 0.5
+    for rows in (None, torch.tensor([m - 1, 0], dtype=torch.int32, device=DEV)):
+        res_a, res_b = _rand(m, n, seed=34), _rand(m, n, seed=34)
+        out_a = ops.add_rmsnorm(partial, res_a, weight, 1e-5, rows)
+        out_b = ops.add_rmsnorm(delta, res_b, weight, 1e-5, rows)
+        assert torch.equal(out_a, out_b) and torch.equal(res_a, res_b)
+
+
+def test_linear_leaves_partial_sums_only_where_asked_and_where_it_pays():
+    from mini_infer_amd import ops
+    from mini_infer_amd.exceptions import KernelShapeError
+
+    a, w = _rand(8, 8192, dtype=torch.bfloat16, seed=36), _rand(64, 8192, dtype=torch.bfloat16, seed=37, scale=0.05)
+    assert ops.partial_sums_pay(8, 64, 8192) and isinstance(ops.linear(a, w, partial_ok=True), ops.PartialSums)
+    assert isinstance(ops.linear(a, w), torch.Tensor)
+    assert not ops.partial_sums_pay(8, 64, 4096) and ops.partial_sums_pay(12, 64, 4096)
+    assert not ops.partial_sums_pay(4, 64, 8192)
+    assert not ops.partial_sums_pay(65, 64, 8192) and not ops.partial_sums_pay(8, 28672, 8192)
+    assert isinstance(ops.linear(a[:, :4096].contiguous(), w[:, :4096].contiguous(), partial_ok=True), torch.Tensor)
+    assert isinstance(ops.linear(a.float(), w.float(), partial_ok=True), torch.Tensor)
+    partial = ops.linear(a, w, partial_ok=True)
+    with pytest.raises(KernelShapeError, match="partial sums"):
+        ops.add_rmsnorm(ops.PartialSums(partial.pieces[:, :1].contiguous(), torch.bfloat16), _rand(8, 64),
+                        _rand(64, dtype=torch.bfloat16), 1e-5)
+    with pytest.raises(KernelShapeError, match="1 to 64 rows"):
+        ops.linear_partial_sums(_rand(65, 64, dtype=torch.bfloat16), _rand(16, 64, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize(
     "m,inter,k",
     [(1, 14336, 4096), (8, 14336, 4096), (16, 160, 64), (7, 301, 96), (13, 4100, 160), (3, 5, 32), (9, 8192, 3072)],
 )
