@@ -110,7 +110,7 @@ extern "C" int mi_take_device_tokens(int* ids, const int* from_rows, const int* 
 // rounded to T, which gives the delta the product would have written itself.
 // ---------------------------------------------------------------------------
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool PIECES>
 __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
     const T* __restrict__ delta, float* __restrict__ residual, const T* __restrict__ weight,
     T* __restrict__ out, const int* __restrict__ rows, int hidden, float eps,
@@ -120,13 +120,13 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
   const int64_t r = rows ? rows[b] : b;
   float* res = residual + r * hidden;
   const T* dl = delta ? delta + r * hidden : nullptr;
-  const float* pt = partials ? partials + r * hidden : nullptr;
+  const float* pt = PIECES ? partials + r * hidden : nullptr;
   T* o = out + (int64_t)b * hidden;
-  const bool has_delta = dl != nullptr || pt != nullptr;
+  const bool has_delta = PIECES || dl != nullptr;
   const bool store_sum = (rows == nullptr) && has_delta;
   // 4 consecutive values of the delta at i (VEC == 4 paths)
   auto delta4 = [&](int i, float* d) {
-    if (pt) {
+    if constexpr (PIECES) {
       float sum[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll 8
       for (int p = 0; p < num_partials; ++p) {  // the loads do not wait for one another
@@ -142,13 +142,14 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(
     }
   };
   auto delta1 = [&](int i) -> float {
-    if (pt) {
+    if constexpr (PIECES) {
       float sum = 0.f;
 #pragma unroll 8
       for (int p = 0; p < num_partials; ++p) sum += pt[(int64_t)p * partial_stride + i];
       return to_f32(from_f32<T>(sum));
+    } else {
+      return to_f32(dl[i]);
     }
-    return to_f32(dl[i]);
   };
 
   if (VEC == 4 && hidden <= (int)blockDim.x * 4) {
@@ -243,13 +244,21 @@ static int add_rmsnorm_launch(const void* delta, float* residual, const void* we
   if (hidden % 4 == 0) {
     // one vector of 4 per thread and pass where the row allows: fewer dependent steps
     const int threads = min(1024, max(256, ceil_div(hidden / 4, 64) * 64));
-    add_rmsnorm_kernel<T, 4><<<num_out_rows, threads, 0, stream>>>(
-        (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps, partials, num_partials,
-        partial_stride);
+    if (partials)
+      add_rmsnorm_kernel<T, 4, true><<<num_out_rows, threads, 0, stream>>>(
+          (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps, partials, num_partials,
+          partial_stride);
+    else
+      add_rmsnorm_kernel<T, 4, false><<<num_out_rows, threads, 0, stream>>>(
+          (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps, nullptr, 0, 0);
   } else {
-    add_rmsnorm_kernel<T, 1><<<num_out_rows, 256, 0, stream>>>(
-        (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps, partials, num_partials,
-        partial_stride);
+    if (partials)
+      add_rmsnorm_kernel<T, 1, true><<<num_out_rows, 256, 0, stream>>>(
+          (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps, partials, num_partials,
+          partial_stride);
+    else
+      add_rmsnorm_kernel<T, 1, false><<<num_out_rows, 256, 0, stream>>>(
+          (const T*)delta, residual, (const T*)weight, (T*)out, rows, hidden, eps, nullptr, 0, 0);
   }
   MI_CHECK_LAUNCH("add_rmsnorm");
   return MI_OK;

@@ -326,17 +326,25 @@ PARTIAL_SUMS_MAX_ROWS = 64
 
 def partial_sums_pay(m: int, n: int, k: int) -> bool:
     """Whether a product of these sizes is left as sums over ranges of K when its caller
-    takes them (`linear(..., partial_ok=True)`).  Measured on MI355X: with a long K
-    (4096 x 14336: 24.5 us at any number of rows up to 16, against 27 / 31 / 37 us whole at
-    1 / 8 / 16 rows, and 25 / 29 us at 32 / 64 rows against the vendor library's 34 / 41),
-    and for a 4096 x 4096 product from 12 rows on (10.3 against 11.5 us at 16 rows; 10.7 /
-    12.7 against 13 / 15 us at 32 / 64).  Wide products (many features) fill the GPU without
-    cutting K and gain nothing; with a single row the whole step ran 0.5 % slower this way
-    (270 -> 269 tok/s at Llama-3.1-8B sizes, though the product alone timed faster), at batch
-    8 / 16 / 64 it ran 1.6 / 5 / 2.8 % faster."""
-    if not 1 <= m <= PARTIAL_SUMS_MAX_ROWS or n > 8192:
+    takes them (`linear(..., partial_ok=True)`).  Measured on MI355X, the product alone,
+    microseconds whole / in pieces at 8, 16, 32, 64 rows (whole = `gemm_skinny_bf16` up to
+    16 rows, the vendor library above):
+
+        4096 x 14336 (8B down)    30 / 24   37 / 25   34 / 25    39 / 28
+        8192 x 28672 (70B down)  101 / 86  120 / 86  101 / 89   144 / 100
+        3072 x 8192  (3B down)    15 / 18   18 / 18   17 / 20    23 / 22
+        4096 x 4096  (8B o)       10 / 10   11 / 10   13 / 11    15 / 13
+        3072 x 3072  (3B o)        8 / 8     9 / 8    11 / 9     16 / 11
+        8192 x 8192  (70B o)      29 / 36   33 / 36   31 / 38    34 / 40
+
+    so: a long K from 5 rows on (with fewer rows the step as a whole ran 0.5 % slower this
+    way at 8B sizes), a small square-ish product from 12 rows on, nothing else.  Whole
+    steps at 8B sizes: batch 8 / 16 / 64 run 1.6 / 5 / 2.8 % faster."""
+    if not 5 <= m <= PARTIAL_SUMS_MAX_ROWS or n > 8192:
         return False
-    return (k >= 8192 and m >= 5) or (k >= 4096 and m >= 12)
+    if k >= 12288:
+        return True
+    return m >= 12 and n <= 4096 and 2048 <= k <= 4096
 
 
 def linear_partial_sums(x: torch.Tensor, weight: torch.Tensor) -> PartialSums:
