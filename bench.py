@@ -111,8 +111,10 @@ def measure_serving(dtype: str) -> dict:
     runner = ModelRunner.from_random(
         LLAMA_32_3B, seed=0, dtype=dtype, num_blocks=pages, block_size=BLOCK_SIZE, max_concurrent=requests_n
     )
+    import os
+
     scheduler = ContinuousScheduler(
-        runner, max_concurrent=requests_n, chunk_size=2048, max_num_batched_tokens=2048
+        runner, max_concurrent=requests_n, chunk_size=2048, max_num_batched_tokens=2048, trace_out=os.devnull
     )
     rng = np.random.default_rng(3)
 
@@ -127,13 +129,25 @@ def measure_serving(dtype: str) -> dict:
     batch = workload()
     prompt_tokens = sum(len(r.prompt) for r in batch)
     steps_before = scheduler.stats["steps"]
+    events_before = len(scheduler.trace_events())
     torch.cuda.synchronize()
     started = time.perf_counter()
     results = scheduler.run_all(batch)
     torch.cuda.synchronize()
     seconds = time.perf_counter() - started
     generated = sum(len(r.tokens) for r in results)
+    # host time from one step to the next, by kind of step (with asynchronous sampling a
+    # step's time shows in the step after it, so the kinds blur at their borders)
+    step_ms: dict[str, list[float]] = {}
+    for event in scheduler.trace_events()[events_before:]:
+        step_ms.setdefault(event["args"]["phase"], []).append(event["dur"] / 1e3)
+    histogram = {
+        kind: {"steps": len(v), "p50_ms": round(float(np.percentile(v, 50)), 2), "p90_ms": round(float(np.percentile(v, 90)), 2),
+               "max_ms": round(max(v), 2)}
+        for kind, v in step_ms.items()
+    }
     return {
+        "step_ms": histogram,
         "model": "Llama-3.2-3B layer sizes",
         "requests": requests_n,
         "prompt_tokens": prompt_tokens,

@@ -286,6 +286,10 @@ class ContinuousScheduler:
         self._pending = None
         self.write_trace()
 
+    def trace_events(self) -> list[dict[str, Any]]:
+        """The step events recorded so far (empty without `trace_out`)."""
+        return list(self._trace_events or [])
+
     def write_trace(self) -> None:
         """Write the steps recorded so far to `trace_out` (nothing without it)."""
         if self._trace_events is not None and self.trace_out is not None:
