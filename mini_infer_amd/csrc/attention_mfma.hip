@@ -673,7 +673,8 @@ extern "C" int mi_attn_mfma_supported(int head_dim, int page_size) {
 // those of the whole step (cu_seqlens_q holds token numbers of the whole step);
 // `first_token` is the run's first token and `num_tokens` the run's token count.
 // With num_splits > 1, part_acc holds (first_token+num_tokens)*q_heads*num_splits*head_dim
-// floats and part_ml (first_token+num_tokens)*q_heads*num_splits*2.
+// floats and part_ml (first_token+num_tokens)*q_heads*num_splits*2; `combine` = 0 leaves the
+// key ranges' results there for the caller's next kernel to combine (`out` is not written).
 extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_pages,
                             const void* vt_pages, const int* block_table, int max_blocks,
                             const int* cu_seqlens_q, const int* positions, int num_requests,
@@ -681,7 +682,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
                             float* part_acc, float* part_ml, int q_heads, int kv_heads,
                             int head_dim, int page_size, int num_pages, float scale, int window,
                             int num_splits, int decode_only, int one_tile_per_request,
-                            int first_token, hipStream_t stream) {
+                            int first_token, int combine, hipStream_t stream) {
   MI_REQUIRE(first_token >= 0, "attn_mfma: first_token=%d is negative", first_token);
   MI_REQUIRE(num_tokens >= 0 && num_requests >= 0 && num_tiles >= 0,
              "attn_mfma: bad sizes tokens=%d requests=%d tiles=%d", num_tokens, num_requests, num_tiles);
@@ -757,7 +758,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
 #undef MI_LAUNCH_P
 #undef MI_LAUNCH
   MI_CHECK_LAUNCH("attn_mfma");
-  if (num_splits > 1) {
+  if (num_splits > 1 && combine) {
     const int64_t first_slot = (int64_t)first_token * q_heads * num_splits;
     return mi_attn_reduce_bf16(part_acc + first_slot * head_dim, part_ml + first_slot * 2,
                                (bf16_t*)out + (int64_t)first_token * out_row_stride, out_row_stride,

@@ -42,6 +42,13 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 // In every case the sums are rounded to bfloat16 before the activation or rotation,
 // exactly as when the product and the second step run as two kernels.
 enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2 };
+// Where the activations come from: a matrix in memory, or (PRO_ATTN, at most 2 rows) the
+// uncombined key ranges of attn_mfma: each wave first combines its own columns of the
+// attention output (what attn_reduce would have written) into LDS, so the combining launch
+// between the attention and its output projection is saved at the smallest batches.
+enum { PRO_NONE = 0, PRO_ATTN = 1 };
+#define SK_PRO_ROWS 2
+#define SK_PRO_SLICE 1024  // activations a wave holds per row: K <= 8 * 1024
 
 struct RopeArgs {  // EPI_ROPE only
   const float* cos_t;  // [m, head_dim/2]
@@ -50,9 +57,14 @@ struct RopeArgs {  // EPI_ROPE only
   bf16_t* k_pages;  // [pages][kv_heads][page_size][head_dim]
   bf16_t* v_pages;  // the same, or [pages][kv_heads][head_dim][page_size] if v_transposed
   int q_heads, kv_heads, head_dim, page_size, v_transposed;
+  // PRO_ATTN: partial accumulators [row][head][split][head_dim], (max in natural-log units,
+  // sum) pairs [row][head][split][2], as attn_mfma leaves them; K = attn_heads * attn_head_dim
+  const float* part_acc;
+  const float* part_ml;
+  int num_splits, attn_heads, attn_head_dim;
 };
 
-template <int NT, int U, int EPI>
+template <int NT, int U, int EPI, int PRO = PRO_NONE>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t ldw,
     bf16_t* __restrict__ c, int64_t ldc, int m, int n, int k, int features_per_block, const RopeArgs rope) {
@@ -101,6 +113,60 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   // activations: lane reads token `col`; lanes past M re-read the last token (the same
   // cache lines as its own lane, so no extra traffic) and their columns are never stored
   const bf16_t* ap = a + (int64_t)min(col, m - 1) * lda + quad * 8;
+  __shared__ __attribute__((aligned(16))) bf16_t a_own[PRO == PRO_ATTN ? SK_WAVES : 1][SK_PRO_ROWS][PRO == PRO_ATTN ? SK_PRO_SLICE : 8];
+  // PRO_ATTN: the weights of the first U k-steps are requested before the activations are
+  // made, so that the trips to the key ranges' results hide behind the first trip to memory
+  bf16x8_t w_first[PRO == PRO_ATTN ? U : 1][WT];
+  const bool first_ahead = PRO == PRO_ATTN && s_begin + U <= s_end;
+  if constexpr (PRO == PRO_ATTN) {
+    if (first_ahead) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int t = 0; t < WT; ++t)
+          w_first[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[t] + (int64_t)(s_begin + u) * 32);
+    }
+  }
+  if constexpr (PRO == PRO_ATTN) {
+    // this wave's columns [32*s_begin, 32*s_end) of the attention output, 8 at a time per
+    // lane: the key ranges' accumulators weighted by exp(max - overall max), added in range
+    // order, divided by the weighted sum of their sums (the arithmetic of attn_reduce_kernel)
+    const int chunks = (s_end - s_begin) * 4;
+    const int head_dim = rope.attn_head_dim, splits = rope.num_splits;
+    for (int idx = lane; idx < m * chunks; idx += MI_WAVE) {
+      const int row = idx / chunks, chunk = idx % chunks;
+      const int k0 = s_begin * 32 + chunk * 8;
+      const int head = k0 / head_dim, dim = k0 % head_dim;
+      const int64_t base = ((int64_t)row * rope.attn_heads + head) * splits;
+      const float* ml = rope.part_ml + base * 2;
+      const float* pa = rope.part_acc + base * head_dim + dim;
+      // (requesting every range's values before the first use measured slower than this loop)
+      float m_all = -INFINITY;
+#pragma unroll 8
+      for (int sp = 0; sp < splits; ++sp) m_all = fmaxf(m_all, ml[sp * 2]);
+      float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      float l_all = 0.f;
+#pragma unroll 4
+      for (int sp = 0; sp < splits; ++sp) {
+        const float weight = expf(ml[sp * 2] - m_all);
+        l_all += ml[sp * 2 + 1] * weight;
+        const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(pa + (int64_t)sp * head_dim);
+        const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(pa + (int64_t)sp * head_dim + 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          o[j] += lo[j] * weight;
+          o[4 + j] += hi[j] * weight;
+        }
+      }
+      const float inv = 1.f / l_all;
+      bf16x8_t packed;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) packed[j] = (bf16_t)(o[j] * inv);
+      *reinterpret_cast<bf16x8_t*>(&a_own[wave][row][chunk * 8]) = packed;
+    }
+    __syncthreads();
+  }
+  const bf16_t* own = &a_own[PRO == PRO_ATTN ? wave : 0][PRO == PRO_ATTN ? min(col, m - 1) : 0][quad * 8];
 
   f32x4_t acc[WT];
 #pragma unroll
@@ -113,9 +179,12 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
-      for (int t = 0; t < WT; ++t)
-        w_reg[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[t] + (int64_t)(s + u) * 32);
-      a_reg[u] = *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)(s + u) * 32);
+      for (int t = 0; t < WT; ++t) {
+        if (PRO == PRO_ATTN && first_ahead && s == s_begin) w_reg[u][t] = w_first[PRO == PRO_ATTN ? u : 0][t];
+        else w_reg[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[t] + (int64_t)(s + u) * 32);
+      }
+      if constexpr (PRO == PRO_ATTN) a_reg[u] = *reinterpret_cast<const bf16x8_t*>(own + (s + u - s_begin) * 32);
+      else a_reg[u] = *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)(s + u) * 32);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -124,7 +193,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_reg[u][t], a_reg[u], acc[t], 0, 0, 0);
   }
   for (; s < s_end; ++s) {  // fewer than U k-steps left
-    const bf16x8_t a_tail = *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)s * 32);
+    const bf16x8_t a_tail = PRO == PRO_ATTN ? *reinterpret_cast<const bf16x8_t*>(own + (s - s_begin) * 32)
+                                            : *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)s * 32);
 #pragma unroll
     for (int t = 0; t < WT; ++t) {
       const bf16x8_t w_tail = *reinterpret_cast<const bf16x8_t*>(wp[t] + (int64_t)s * 32);
@@ -290,6 +360,47 @@ extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, in
   return MI_OK;
 }
 
+// c[m, n] = attention output [m, heads*head_dim] . w^T, the attention output still lying in
+// attn_mfma's uncombined key ranges (part_acc, part_ml as that kernel leaves them, rows
+// 0..m-1): at most 2 rows, heads*head_dim at most 8192.
+extern "C" int mi_gemm_skinny_attn_bf16(const float* part_acc, const float* part_ml, int num_splits, int heads,
+                                        int head_dim, const void* w, int64_t ldw, void* c, int64_t ldc, int m,
+                                        int n, hipStream_t stream) {
+  MI_REQUIRE(part_acc && part_ml && num_splits >= 1 && num_splits <= 64,
+             "gemm_skinny_attn_bf16: needs the partial buffers of 1..64 key ranges, got %d", num_splits);
+  MI_REQUIRE(heads >= 1 && head_dim >= 32 && head_dim % 32 == 0,
+             "gemm_skinny_attn_bf16: takes head_dim a multiple of 32; got heads=%d head_dim=%d", heads, head_dim);
+  const int k = heads * head_dim;
+  MI_REQUIRE(m >= 1 && m <= SK_PRO_ROWS && n >= 1 && ldw % 8 == 0 && ldw >= k && ldc >= n,
+             "gemm_skinny_attn_bf16: takes 1 <= m <= %d, weight rows aligned to 16 bytes; got m=%d n=%d k=%d ldw=%lld",
+             SK_PRO_ROWS, m, n, k, (long long)ldw);
+  MI_REQUIRE(ceil_div(k / 32, SK_WAVES) * 32 <= SK_PRO_SLICE,
+             "gemm_skinny_attn_bf16: heads*head_dim=%d is more than %d", k, SK_WAVES * SK_PRO_SLICE);
+  const bf16_t* ap = (const bf16_t*)w;  // never read: the activations are made in the kernel
+  const int64_t lda = ldw;
+  const bf16_t* wp = (const bf16_t*)w;
+  bf16_t* cp = (bf16_t*)c;
+  RopeArgs args = {};
+  args.part_acc = part_acc;
+  args.part_ml = part_ml;
+  args.num_splits = num_splits;
+  args.attn_heads = heads;
+  args.attn_head_dim = head_dim;
+  const int cus = compute_units();
+  MI_REQUIRE(cus > 0, "gemm_skinny_attn_bf16: cannot read the device's compute unit count");
+  const int fpb = features_per_block_for(n, cus, 4);
+  const int blocks = ceil_div(n, fpb);
+  const int threads = 64 * SK_WAVES;
+  switch (ceil_div(fpb, 16)) {
+    case 1: gemm_skinny_bf16_kernel<1, 8, EPI_STORE, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args); break;
+    case 2: gemm_skinny_bf16_kernel<2, 8, EPI_STORE, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args); break;
+    case 3: gemm_skinny_bf16_kernel<3, 4, EPI_STORE, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args); break;
+    default: gemm_skinny_bf16_kernel<4, 2, EPI_STORE, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args); break;
+  }
+  MI_CHECK_LAUNCH("gemm_skinny_attn_bf16");
+  return MI_OK;
+}
+
 // out[m, n] = silu(a . gate^T) * (a . up^T) with w = [gate; up] stacked, [2n, k].
 extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* out,
                                           int64_t ldo, int m, int n, int k, hipStream_t stream) {
@@ -334,7 +445,7 @@ extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* 
   MI_REQUIRE(cos_t && sin_t, "gemm_skinny_rope_bf16: needs the rotation tables");
   MI_REQUIRE(kv_heads == 0 || (slot_mapping && k_pages && v_pages && page_size > 0 && num_pages > 0),
              "gemm_skinny_rope_bf16: pages and slots are needed to write keys and values");
-  RopeArgs rope;
+  RopeArgs rope = {};
   rope.cos_t = cos_t;
   rope.sin_t = sin_t;
   rope.slot_mapping = slot_mapping;

@@ -534,6 +534,63 @@ def attention_splits(work_items: int, max_seq_len: int, target: int = 2048, min_
     return int(min(by_fill, by_len, 64))
 
 
+@dataclasses.dataclass
+class AttentionPieces:
+    """An attention output that has not been combined yet: the results of `splits` key ranges
+    per (token, head) as `attn_mfma` leaves them (`paged_attention(..., combine=False)`).
+    `linear_from_attention` multiplies them with the output projection, combining on its way;
+    `finish()` combines them as the attention would have."""
+
+    part_acc: torch.Tensor  # [tokens * heads * splits, head_dim] float32
+    part_ml: torch.Tensor  # [tokens * heads * splits, 2] float32: maximum (natural log units), sum
+    splits: int
+    tokens: int
+    heads: int
+    head_dim: int
+    dtype: torch.dtype
+
+    def finish(self) -> torch.Tensor:
+        acc = self.part_acc.view(self.tokens, self.heads, self.splits, self.head_dim)
+        ml = self.part_ml.view(self.tokens, self.heads, self.splits, 2)
+        weight = torch.exp(ml[..., 0] - ml[..., 0].max(dim=-1, keepdim=True).values)
+        total = (acc * weight[..., None]).sum(dim=2) / (ml[..., 1] * weight).sum(dim=-1, keepdim=True)
+        return total.reshape(self.tokens, self.heads * self.head_dim).to(self.dtype)
+
+
+ATTENTION_PIECES_MAX_ROWS = 2
+
+
+def linear_from_attention(pieces: AttentionPieces, weight: torch.Tensor) -> torch.Tensor:
+    """`attention output @ weight.T` for at most 2 tokens, from the uncombined key ranges: one
+    kernel instead of the combining kernel and the product."""
+    _need_cuda(pieces.part_acc, pieces.part_ml, weight)
+    k = pieces.heads * pieces.head_dim
+    if (
+        weight.dtype != torch.bfloat16
+        or weight.dim() != 2
+        or weight.shape[1] != k
+        or weight.stride(1) != 1
+        or weight.stride(0) % 8 != 0
+        or not 1 <= pieces.tokens <= ATTENTION_PIECES_MAX_ROWS
+        or pieces.head_dim % 32 != 0
+        or k > 8192
+    ):
+        raise KernelShapeError(
+            f"linear_from_attention takes 1 or 2 tokens, head_dim a multiple of 32, heads*head_dim <= 8192 and a "
+            f"bfloat16 weight [N, {k}]; got {pieces.tokens} tokens, head_dim {pieces.head_dim}, weight {tuple(weight.shape)} {weight.dtype}"
+        )
+    n = weight.shape[0]
+    out = torch.empty((pieces.tokens, n), dtype=torch.bfloat16, device=weight.device)
+    lib = library.load()
+    library.check(
+        lib.mi_gemm_skinny_attn_bf16(
+            _ptr(pieces.part_acc), _ptr(pieces.part_ml), pieces.splits, pieces.heads, pieces.head_dim,
+            _ptr(weight), weight.stride(0), _ptr(out), out.stride(0), pieces.tokens, n, _stream(),
+        )
+    )
+    return out
+
+
 def paged_attention(
     q: torch.Tensor,
     k_pages: torch.Tensor,
@@ -552,8 +609,12 @@ def paged_attention(
     max_seq_len: int,
     v_transposed: bool = False,
     force_plain: bool = False,
-) -> torch.Tensor:
+    combine: bool = True,
+) -> torch.Tensor | AttentionPieces:
     """Causal attention of every token over its request's pages; returns [T, q_heads*head_dim].
+
+    With `combine=False` a step of single tokens whose keys are cut into ranges (the
+    matrix-core kernel) comes back as `AttentionPieces`, for `linear_from_attention`.
 
     `q` is [T, >= q_heads*head_dim] with the rotated queries in its first columns
     (rows may be strided, so the merged projection's buffer can be passed as it is).
@@ -615,7 +676,7 @@ def paged_attention(
         q_lens = [host_cu_seqlens_q[b + 1] - host_cu_seqlens_q[b] for b in range(num_requests)]
         max_blocks = block_table.shape[1]
 
-        def run(first: int, last: int) -> None:
+        def run(first: int, last: int, leave_pieces: bool = False) -> AttentionPieces | None:
             """Requests [first, last) of the step in one launch."""
             lens = q_lens[first:last]
             count = last - first
@@ -643,9 +704,13 @@ def paged_attention(
                     _ptr(cu_seqlens_q) + 4 * first, _ptr(positions), count, run_tokens,
                     num_tiles, _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads,
                     head_dim, page_size, num_pages, float(scale), int(window or 0), splits,
-                    int(decode_only), int(one_tile_per_request), first_token, _stream(),
+                    int(decode_only), int(one_tile_per_request), first_token,
+                    0 if (leave_pieces and splits > 1) else 1, _stream(),
                 )
             )
+            if leave_pieces and splits > 1:
+                return AttentionPieces(part_acc, part_ml, splits, run_tokens, q_heads, head_dim, q.dtype)
+            return None
 
         # Leading requests that bring a single token (a scheduler puts its decoding requests
         # first) run in the decode shape, where waves split the keys; inside the 128-row
@@ -658,7 +723,9 @@ def paged_attention(
             run(0, leading_single)
             run(leading_single, num_requests)
         else:
-            run(0, num_requests)
+            pieces = run(0, num_requests, leave_pieces=not combine and leading_single == num_requests)
+            if pieces is not None:
+                return pieces
         return out
 
     splits = attention_splits(tokens * kv_heads * math.ceil(group / 4), max_seq_len)

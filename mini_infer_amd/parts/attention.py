@@ -89,7 +89,7 @@ class GQAttention(Mixer):
                 q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
                 v_transposed=cache.v_transposed,
             )
-            return self.out.forward(self._attend(queries, ctx, cache), partial_ok=self.emit_partial_sums)
+            return self._project(self._attend(queries, ctx, cache))
         if writes_cache:
             qkv = self.qkv.forward(x)
             kv_heads, slots = self.num_kv_heads, ctx.slot_mapping[cache.group]
@@ -113,15 +113,26 @@ class GQAttention(Mixer):
                 q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
                 rotary_dim=0, interleaved=False, v_transposed=cache.v_transposed,
             )
-        return self.out.forward(self._attend(qkv, ctx, cache), partial_ok=self.emit_partial_sums)
+        return self._project(self._attend(qkv, ctx, cache))
 
-    def _attend(self, queries: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
-        """Attention of the rotated queries (the first columns of `queries`) over the cache pages."""
+    def _project(self, attended):
+        """The output projection of what `_attend` returned."""
+        if isinstance(attended, ops.AttentionPieces):
+            assert self.out.weight is not None
+            return ops.linear_from_attention(attended, self.out.weight)
+        return self.out.forward(attended, partial_ok=self.emit_partial_sums)
+
+    def _attend(self, queries: torch.Tensor, ctx: StepContext, cache: LayerCache):
+        """Attention of the rotated queries (the first columns of `queries`) over the cache pages.
+        At the smallest batches the key ranges may come back uncombined, for the output
+        projection to combine on its way (one launch less a layer)."""
+        few = ctx.num_tokens <= ops.ATTENTION_PIECES_MAX_ROWS and self.num_heads * self.head_dim <= 8192
+        few = few and self.head_dim % 32 == 0 and queries.dtype == torch.bfloat16
         return ops.paged_attention(
             queries, cache.k_pages, cache.v_pages, ctx.block_tables[cache.group], ctx.token_request,
             ctx.positions, ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
-            max_seq_len=ctx.max_seq_len, v_transposed=cache.v_transposed,
+            max_seq_len=ctx.max_seq_len, v_transposed=cache.v_transposed, combine=not few,
         )
 
 

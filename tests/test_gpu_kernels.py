@@ -539,6 +539,33 @@ def test_paged_attention_long_context_in_many_key_ranges():
     assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(torch.bfloat16, 2)
 
 
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,lengths", [(32, 8, 128, [3000]), (6, 2, 64, [700, 2049]), (3, 1, 32, [517])])
+def test_output_projection_from_uncombined_key_ranges(q_heads, kv_heads, head_dim, lengths):
+    """One or two single tokens: the attention leaves its key ranges uncombined and the output
+    projection combines them on its way; the same numbers as combining first."""
+    from mini_infer_amd import ops
+
+    case = _paged_case(torch.bfloat16, q_heads, kv_heads, head_dim, 16, lengths, [1] * len(lengths), seed=41,
+                       v_transposed=True)
+    args = (case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"],
+            case["positions"], case["cu"], case["host_cu"])
+    kwargs = dict(q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=0.3, window=None,
+                  max_seq_len=max(lengths), v_transposed=True)
+    whole = ops.paged_attention(*args, **kwargs)
+    pieces = ops.paged_attention(*args, **kwargs, combine=False)
+    assert isinstance(pieces, ops.AttentionPieces) and pieces.splits > 1 and pieces.tokens == len(lengths)
+    assert (pieces.finish().float() - whole.float()).abs().max() < 2e-2
+    for n in (q_heads * head_dim, 1000, 24):
+        w = _rand(n, q_heads * head_dim, dtype=torch.bfloat16, seed=42, scale=0.1)
+        assert torch.equal(ops.linear_from_attention(pieces, w), ops.linear(whole, w))
+    # with nothing to combine, or more than single tokens, the attention comes back whole
+    short = _paged_case(torch.bfloat16, q_heads, kv_heads, head_dim, 16, [40], [1], seed=43, v_transposed=True)
+    out = ops.paged_attention(short["q"], short["k_pages"], short["v_pages"], short["block_table"], short["token_request"],
+                              short["positions"], short["cu"], short["host_cu"], q_heads=q_heads, kv_heads=kv_heads,
+                              head_dim=head_dim, scale=0.3, window=None, max_seq_len=40, v_transposed=True, combine=False)
+    assert isinstance(out, torch.Tensor)
+
+
 def test_kernels_refuse_what_they_do_not_take():
     from mini_infer_amd import ops
     from mini_infer_amd.exceptions import KernelShapeError
