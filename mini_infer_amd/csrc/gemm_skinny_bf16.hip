@@ -42,13 +42,12 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 // In every case the sums are rounded to bfloat16 before the activation or rotation,
 // exactly as when the product and the second step run as two kernels.
 enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2 };
-// Where the activations come from: a matrix in memory, or (PRO_ATTN, at most 2 rows) the
+// Where the activations come from: a matrix in memory, or (PRO_ATTN, few rows) the
 // uncombined key ranges of attn_mfma: each wave first combines its own columns of the
 // attention output (what attn_reduce would have written) into LDS, so the combining launch
 // between the attention and its output projection is saved at the smallest batches.
 enum { PRO_NONE = 0, PRO_ATTN = 1 };
-#define SK_PRO_ROWS 2
-#define SK_PRO_SLICE 1024  // activations a wave holds per row: K <= 8 * 1024
+#define SK_PRO_VALUES 4096  // activations a wave makes and holds: rows * (K / 8 waves) at most
 
 struct RopeArgs {  // EPI_ROPE only
   const float* cos_t;  // [m, head_dim/2]
@@ -113,7 +112,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   // activations: lane reads token `col`; lanes past M re-read the last token (the same
   // cache lines as its own lane, so no extra traffic) and their columns are never stored
   const bf16_t* ap = a + (int64_t)min(col, m - 1) * lda + quad * 8;
-  __shared__ __attribute__((aligned(16))) bf16_t a_own[PRO == PRO_ATTN ? SK_WAVES : 1][SK_PRO_ROWS][PRO == PRO_ATTN ? SK_PRO_SLICE : 8];
+  __shared__ __attribute__((aligned(16))) bf16_t a_own[PRO == PRO_ATTN ? SK_WAVES : 1][PRO == PRO_ATTN ? SK_PRO_VALUES : 8];
+  const int own_stride = per_wave * 32;  // elements from one row of this wave's columns to the next
   // PRO_ATTN: the weights of the first U k-steps are requested before the activations are
   // made, so that the trips to the key ranges' results hide behind the first trip to memory
   bf16x8_t w_first[PRO == PRO_ATTN ? U : 1][WT];
@@ -162,11 +162,11 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
       bf16x8_t packed;
 #pragma unroll
       for (int j = 0; j < 8; ++j) packed[j] = (bf16_t)(o[j] * inv);
-      *reinterpret_cast<bf16x8_t*>(&a_own[wave][row][chunk * 8]) = packed;
+      *reinterpret_cast<bf16x8_t*>(&a_own[wave][row * own_stride + chunk * 8]) = packed;
     }
     __syncthreads();
   }
-  const bf16_t* own = &a_own[PRO == PRO_ATTN ? wave : 0][PRO == PRO_ATTN ? min(col, m - 1) : 0][quad * 8];
+  const bf16_t* own = &a_own[PRO == PRO_ATTN ? wave : 0][(PRO == PRO_ATTN ? min(col, m - 1) * own_stride : 0) + quad * 8];
 
   f32x4_t acc[WT];
 #pragma unroll
@@ -362,7 +362,14 @@ extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, in
 
 // c[m, n] = attention output [m, heads*head_dim] . w^T, the attention output still lying in
 // attn_mfma's uncombined key ranges (part_acc, part_ml as that kernel leaves them, rows
-// 0..m-1): at most 2 rows, heads*head_dim at most 8192.
+// 0..m-1): few rows, m * heads*head_dim at most 32768 (8 rows of 4096; see
+// mi_gemm_skinny_attn_bf16_supported).
+extern "C" int mi_gemm_skinny_attn_bf16_supported(int m, int heads, int head_dim) {
+  if (m < 1 || m > SK_MAX_ROWS || heads < 1 || head_dim < 32 || head_dim % 32 != 0) return 0;
+  const int k = heads * head_dim;
+  return m * ceil_div(k / 32, SK_WAVES) * 32 <= SK_PRO_VALUES ? 1 : 0;
+}
+
 extern "C" int mi_gemm_skinny_attn_bf16(const float* part_acc, const float* part_ml, int num_splits, int heads,
                                         int head_dim, const void* w, int64_t ldw, void* c, int64_t ldc, int m,
                                         int n, hipStream_t stream) {
@@ -371,11 +378,11 @@ extern "C" int mi_gemm_skinny_attn_bf16(const float* part_acc, const float* part
   MI_REQUIRE(heads >= 1 && head_dim >= 32 && head_dim % 32 == 0,
              "gemm_skinny_attn_bf16: takes head_dim a multiple of 32; got heads=%d head_dim=%d", heads, head_dim);
   const int k = heads * head_dim;
-  MI_REQUIRE(m >= 1 && m <= SK_PRO_ROWS && n >= 1 && ldw % 8 == 0 && ldw >= k && ldc >= n,
-             "gemm_skinny_attn_bf16: takes 1 <= m <= %d, weight rows aligned to 16 bytes; got m=%d n=%d k=%d ldw=%lld",
-             SK_PRO_ROWS, m, n, k, (long long)ldw);
-  MI_REQUIRE(ceil_div(k / 32, SK_WAVES) * 32 <= SK_PRO_SLICE,
-             "gemm_skinny_attn_bf16: heads*head_dim=%d is more than %d", k, SK_WAVES * SK_PRO_SLICE);
+  MI_REQUIRE(n >= 1 && ldw % 8 == 0 && ldw >= k && ldc >= n,
+             "gemm_skinny_attn_bf16: weight rows must be aligned to 16 bytes; got n=%d k=%d ldw=%lld", n, k,
+             (long long)ldw);
+  MI_REQUIRE(mi_gemm_skinny_attn_bf16_supported(m, heads, head_dim),
+             "gemm_skinny_attn_bf16: rows x (heads*head_dim / 8) must be at most %d; got m=%d k=%d", SK_PRO_VALUES, m, k);
   const bf16_t* ap = (const bf16_t*)w;  // never read: the activations are made in the kernel
   const int64_t lda = ldw;
   const bf16_t* wp = (const bf16_t*)w;

@@ -557,11 +557,20 @@ class AttentionPieces:
         return total.reshape(self.tokens, self.heads * self.head_dim).to(self.dtype)
 
 
-ATTENTION_PIECES_MAX_ROWS = 2
+def attention_pieces_pay(tokens: int, heads: int, head_dim: int) -> bool:
+    """Whether a step of `tokens` single tokens leaves its attention uncombined for the output
+    projection (`paged_attention(combine=False)` + `linear_from_attention`).  Every block of
+    that projection reads all the key ranges' results (tokens x heads x ranges x head_dim
+    floats), which costs more than the saved launch as soon as there are several tokens:
+    measured at Llama-3.1-8B sizes, a single token runs 1 % faster this way, 8 tokens 6 %
+    slower.  So: one token."""
+    if tokens != 1 or heads < 1 or head_dim < 32 or head_dim % 32 != 0:
+        return False
+    return bool(library.load().mi_gemm_skinny_attn_bf16_supported(tokens, heads, head_dim))
 
 
 def linear_from_attention(pieces: AttentionPieces, weight: torch.Tensor) -> torch.Tensor:
-    """`attention output @ weight.T` for at most 2 tokens, from the uncombined key ranges: one
+    """`attention output @ weight.T` for a few tokens, from the uncombined key ranges: one
     kernel instead of the combining kernel and the product."""
     _need_cuda(pieces.part_acc, pieces.part_ml, weight)
     k = pieces.heads * pieces.head_dim
@@ -571,12 +580,10 @@ def linear_from_attention(pieces: AttentionPieces, weight: torch.Tensor) -> torc
         or weight.shape[1] != k
         or weight.stride(1) != 1
         or weight.stride(0) % 8 != 0
-        or not 1 <= pieces.tokens <= ATTENTION_PIECES_MAX_ROWS
-        or pieces.head_dim % 32 != 0
-        or k > 8192
+        or not library.load().mi_gemm_skinny_attn_bf16_supported(pieces.tokens, pieces.heads, pieces.head_dim)
     ):
         raise KernelShapeError(
-            f"linear_from_attention takes 1 or 2 tokens, head_dim a multiple of 32, heads*head_dim <= 8192 and a "
+            f"linear_from_attention takes few tokens (tokens x heads*head_dim <= 32768), head_dim a multiple of 32 and a "
             f"bfloat16 weight [N, {k}]; got {pieces.tokens} tokens, head_dim {pieces.head_dim}, weight {tuple(weight.shape)} {weight.dtype}"
         )
     n = weight.shape[0]

@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -35,6 +35,7 @@ _SIGNATURES: dict[str, list] = {
     "mi_gemm_mid_partial_bf16": [_P, c_int64, _P, c_int64, _P, c_int, c_int, c_int, _P],
     "mi_gemm_mid_bf16_ranges": [c_int, c_int],
     "mi_gemm_mid_bf16_supported": [c_int, c_int, c_int, c_int64, c_int64],
+    "mi_gemm_skinny_attn_bf16_supported": [c_int, c_int, c_int],
     "mi_gemm_skinny_attn_bf16": [_P, _P, c_int, c_int, c_int, _P, c_int64, _P, c_int64, c_int, c_int, _P],
     "mi_gemm_skinny_swiglu_bf16": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_gemm_skinny_rope_bf16": [

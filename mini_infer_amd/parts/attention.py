@@ -126,8 +126,7 @@ class GQAttention(Mixer):
         """Attention of the rotated queries (the first columns of `queries`) over the cache pages.
         At the smallest batches the key ranges may come back uncombined, for the output
         projection to combine on its way (one launch less a layer)."""
-        few = ctx.num_tokens <= ops.ATTENTION_PIECES_MAX_ROWS and self.num_heads * self.head_dim <= 8192
-        few = few and self.head_dim % 32 == 0 and queries.dtype == torch.bfloat16
+        few = queries.dtype == torch.bfloat16 and ops.attention_pieces_pay(ctx.num_tokens, self.num_heads, self.head_dim)
         return ops.paged_attention(
             queries, cache.k_pages, cache.v_pages, ctx.block_tables[cache.group], ctx.token_request,
             ctx.positions, ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=self.num_heads,

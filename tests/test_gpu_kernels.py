@@ -539,9 +539,13 @@ def test_paged_attention_long_context_in_many_key_ranges():
     assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(torch.bfloat16, 2)
 
 
-@pytest.mark.parametrize("q_heads,kv_heads,head_dim,lengths", [(32, 8, 128, [3000]), (6, 2, 64, [700, 2049]), (3, 1, 32, [517])])
+@pytest.mark.parametrize(
+    "q_heads,kv_heads,head_dim,lengths",
+    [(32, 8, 128, [3000]), (6, 2, 64, [700, 2049]), (3, 1, 32, [517]), (32, 8, 128, [2100, 2500, 3000, 2048, 4000, 2222, 3100, 2900]),
+     (6, 2, 64, [700, 2049, 333, 900, 1200, 800, 650, 1500, 400, 512, 2000])],
+)
 def test_output_projection_from_uncombined_key_ranges(q_heads, kv_heads, head_dim, lengths):
-    """One or two single tokens: the attention leaves its key ranges uncombined and the output
+    """A few single tokens: the attention leaves its key ranges uncombined and the output
     projection combines them on its way; the same numbers as combining first."""
     from mini_infer_amd import ops
 
@@ -553,6 +557,7 @@ def test_output_projection_from_uncombined_key_ranges(q_heads, kv_heads, head_di
                   max_seq_len=max(lengths), v_transposed=True)
     whole = ops.paged_attention(*args, **kwargs)
     pieces = ops.paged_attention(*args, **kwargs, combine=False)
+    assert ops.attention_pieces_pay(1, q_heads, head_dim)
     assert isinstance(pieces, ops.AttentionPieces) and pieces.splits > 1 and pieces.tokens == len(lengths)
     assert (pieces.finish().float() - whole.float()).abs().max() < 2e-2
     for n in (q_heads * head_dim, 1000, 24):
@@ -564,6 +569,7 @@ def test_output_projection_from_uncombined_key_ranges(q_heads, kv_heads, head_di
                               short["positions"], short["cu"], short["host_cu"], q_heads=q_heads, kv_heads=kv_heads,
                               head_dim=head_dim, scale=0.3, window=None, max_seq_len=40, v_transposed=True, combine=False)
     assert isinstance(out, torch.Tensor)
+    assert not ops.attention_pieces_pay(2, 32, 128) and not ops.attention_pieces_pay(1, 4, 48)
 
 
 def test_kernels_refuse_what_they_do_not_take():
