@@ -23,11 +23,11 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define MID_KC 8  // k-steps of 32 per piece
 #define MID_AROW (MID_KC * 32 + 8)  // elements: rows 16 bytes apart in the banks, so 16 rows read side by side
 
-template <int MT, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void gemm_mid_partial_kernel(
+template <int MT>
+__global__ __launch_bounds__(64 * MID_WAVES) void gemm_mid_partial_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t ldw,
     float* __restrict__ part, int m, int n, int k, int pieces_per_range) {
-  constexpr int THREADS = 64 * WAVES;
+  constexpr int THREADS = 64 * MID_WAVES;
   constexpr int ROWS = 16 * MT;
   constexpr int A_IDS = ROWS * MID_KC * 4;  // 16-byte chunks of one piece of the activations
   constexpr int A_PER = A_IDS / THREADS;
@@ -37,7 +37,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_partial_kernel(
   const int wave = threadIdx.x / MI_WAVE;
   const int lane = threadIdx.x % MI_WAVE;
   const int col = lane % 16, quad = lane / 16;
-  const int n0 = blockIdx.x * (16 * WAVES) + wave * 16;
+  const int n0 = blockIdx.x * (16 * MID_WAVES) + wave * 16;
   const int ksteps = k / 32;
   const int s_begin = min((int)blockIdx.y * pieces_per_range * MID_KC, ksteps);
   const int s_end = min(s_begin + pieces_per_range * MID_KC, ksteps);
@@ -161,8 +161,8 @@ extern "C" int mi_gemm_mid_partial_bf16(const void* a, int64_t lda, const void* 
   const int per_range = ceil_div(pieces, ranges);
   const dim3 grid(ceil_div(n, 16 * MID_WAVES), ranges);
 #define MID_GO(MT_)                                                                                    \
-  gemm_mid_partial_kernel<MT_, MID_WAVES><<<grid, 64 * MID_WAVES, 0, stream>>>((const bf16_t*)a, lda, \
-                                                                              (const bf16_t*)w, ldw, part, m, n, k, per_range)
+  gemm_mid_partial_kernel<MT_><<<grid, 64 * MID_WAVES, 0, stream>>>((const bf16_t*)a, lda, (const bf16_t*)w, ldw, \
+                                                                   part, m, n, k, per_range)
   if (m <= 16) MID_GO(1);
   else if (m <= 32) MID_GO(2);
   else MID_GO(4);
