@@ -379,15 +379,17 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
 // The same for the usual layout (halves paired, every size a multiple of 4), four
 // elements per thread and step: 8- and 16-byte loads and stores instead of single
 // elements.  Arithmetic and rounding are those of the kernel above.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_vec;
+
 template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_write_vec4_kernel(
     T* __restrict__ qkv, int64_t row_stride, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const int* __restrict__ slot_mapping, T* __restrict__ k_pages,
     T* __restrict__ v_pages, int q_heads, int kv_heads, int head_dim, int rotary_dim, int page_size,
-    int v_transposed) {
+    int v_transposed, int num_tokens, int blocks_y) {
   const int t = blockIdx.x;
   const int first = blockIdx.y * blockDim.x + threadIdx.x;
-  const int stride = blockDim.x * gridDim.y;
+  const int stride = blockDim.x * blocks_y;
   const int half = rotary_dim / 2;
   const int half4 = half / 4;
   T* row = qkv + (int64_t)t * row_stride;
@@ -438,6 +440,37 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec4_kernel(
     load4(k_row + h * head_dim + d, x);
     store4(k_pages + (((int64_t)page * kv_heads + h) * page_size + off) * head_dim + d, x);
   }
+  if (v_transposed && page_size % 8 == 0) {
+    // Transposed value pages keep a dim's slots side by side: where this step's tokens fill a
+    // whole page in order (a prompt's portion), the page's FIRST token writes every dim's row
+    // of the page at once (page_size elements in a row instead of one), the others nothing.
+    const int lead = t - off;
+    bool whole_page = lead >= 0 && lead + page_size <= num_tokens;
+    if (whole_page) {
+      for (int i = 0; i < page_size; ++i) whole_page = whole_page && slot_mapping[lead + i] == page * page_size + i;
+    }
+    if (whole_page) {
+      if (off != 0) return;
+      const int64_t v_off = (int64_t)(q_heads + kv_heads) * head_dim;
+      for (int e = first; e < kv_heads * head_dim; e += stride) {
+        const int h = e / head_dim, d = e % head_dim;
+        T* dst = v_pages + ((int64_t)page * kv_heads + h) * page_size * head_dim + (int64_t)d * page_size;
+        const T* src = qkv + (int64_t)lead * row_stride + v_off + h * head_dim + d;
+        for (int i0 = 0; i0 < page_size; i0 += 8) {
+          if constexpr (sizeof(T) == 2) {
+            bf16x8_vec x;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = src[(int64_t)(i0 + i) * row_stride];
+            *reinterpret_cast<bf16x8_vec*>(dst + i0) = x;
+          } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dst[i0 + i] = src[(int64_t)(i0 + i) * row_stride];
+          }
+        }
+      }
+      return;
+    }
+  }
   const int dim4 = head_dim / 4;
   for (int e = first; e < kv_heads * dim4; e += stride) {
     const int h = e / dim4, d = (e % dim4) * 4;
@@ -480,11 +513,11 @@ extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const 
     if (dtype == MI_F32) {
       rope_kv_write_vec4_kernel<float><<<grid, 256, 0, stream>>>(
           (float*)qkv, row_stride, cos_t, sin_t, slot_mapping, (float*)k_pages, (float*)v_pages,
-          q_heads, kv_heads, head_dim, rotary_dim, page_size, v_transposed);
+          q_heads, kv_heads, head_dim, rotary_dim, page_size, v_transposed, num_tokens, blocks_y);
     } else {
       rope_kv_write_vec4_kernel<bf16_t><<<grid, 256, 0, stream>>>(
           (bf16_t*)qkv, row_stride, cos_t, sin_t, slot_mapping, (bf16_t*)k_pages, (bf16_t*)v_pages,
-          q_heads, kv_heads, head_dim, rotary_dim, page_size, v_transposed);
+          q_heads, kv_heads, head_dim, rotary_dim, page_size, v_transposed, num_tokens, blocks_y);
     }
     MI_CHECK_LAUNCH("rope_kv_write");
     return MI_OK;

@@ -333,6 +333,46 @@ def test_rope_kv_write(dtype, q_heads, kv_heads, head_dim, rotary_dim, interleav
         assert torch.equal(qkv[0, : q_heads * head_dim], original[0, : q_heads * head_dim])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page_size", [16, 8])
+def test_rope_kv_write_whole_pages_of_transposed_values(dtype, page_size):
+    """Tokens that fill a page in order have their transposed values written a whole page at a
+    time by the page's first token; pages filled out of order, from the middle, or only in
+    part go token by token.  All give what the plain layout gives, transposed."""
+    from mini_infer_amd import ops
+
+    q_heads, kv_heads, head_dim, num_pages = 4, 2, 32, 7
+    ps = page_size
+    slots = (
+        list(range(2 * ps, 3 * ps))  # page 2, in order: written at once
+        + [0 * ps + i for i in np.random.default_rng(0).permutation(ps)]  # page 0, out of order
+        + list(range(4 * ps + 3, 4 * ps + 3 + 5))  # page 4 from its middle
+        + list(range(5 * ps, 5 * ps + ps // 2))  # half of page 5
+        + [-1]  # a token that is not written
+        + list(range(6 * ps, 7 * ps))  # page 6, in order, at the very end of the step
+        + list(range(3 * ps, 3 * ps + ps - 1))  # page 3 but for its last slot
+    )
+    tokens = len(slots)
+    qkv = _rand(tokens, (q_heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=21)
+    positions = torch.arange(tokens, dtype=torch.int32, device=DEV)
+    cos, sin = ops.rope_table(positions, torch.from_numpy(pl.inv_freq_default(head_dim, 10000.0)).to(DEV))
+    slot_t = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    k_a = torch.zeros((num_pages, kv_heads, ps, head_dim), dtype=dtype, device=DEV)
+    v_a = torch.zeros_like(k_a)
+    ops.rope_kv_write(qkv.clone(), cos, sin, slot_t, k_a, v_a, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+                      rotary_dim=head_dim, interleaved=False)
+    k_b = torch.zeros_like(k_a)
+    v_b = torch.zeros((num_pages, kv_heads, head_dim, ps), dtype=dtype, device=DEV)
+    ops.rope_kv_write(qkv.clone(), cos, sin, slot_t, k_b, v_b, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
+                      rotary_dim=head_dim, interleaved=False, v_transposed=True)
+    assert torch.equal(k_a, k_b) and torch.equal(v_b.transpose(2, 3), v_a)
+    values = qkv[:, (q_heads + kv_heads) * head_dim :].reshape(tokens, kv_heads, head_dim)
+    for t, slot in enumerate(slots):
+        if slot >= 0:
+            assert torch.equal(v_a[slot // ps, :, slot % ps], values[t])
+    assert int((v_a != 0).any(dim=-1).sum()) == sum(1 for s in slots if s >= 0) * kv_heads  # nothing else was written
+
+
 def _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=0, v_transposed=False):
     """Random keys/values scattered over shuffled pages; queries are the last q_len positions."""
     rng = np.random.default_rng(seed)
