@@ -1,4 +1,4 @@
-// Weight-streaming matrix product for up to 64 rows, left as float32 sums over ranges of K:
+// Weight-streaming matrix product for up to 128 rows, left as float32 sums over ranges of K:
 // part[s][M][N] = sum over the s-th range of K of A[M, k] * W[N, k], bfloat16 in.
 //
 // The product is bound by reading W once, but the activations do not come for free: a
@@ -11,7 +11,7 @@
 // ahead.  Cutting K across blocks is what fills the GPU when N is small; the pieces are
 // added up, in order, by the kernel that consumes the product (add_rmsnorm).  Measured on
 // MI355X: 4096 x 14336 in 24.5 us at 1 to 16 rows (gemm_skinny_bf16: 27 / 31 / 37 us at
-// 1 / 8 / 16 rows), 25 / 29 us at 32 / 64 rows (vendor library: 34 / 41 us).
+// 1 / 8 / 16 rows), 25 / 29 / 39 us at 32 / 64 / 128 rows (vendor library: 34 / 41 / 75 us).
 //
 // This stands where the reference's engine calls the vendor BLAS (distributed/linear.py:167).
 #include "common.h"
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(64 * MID_WAVES) void gemm_mid_partial_kernel(
 }
 
 extern "C" int mi_gemm_mid_bf16_supported(int m, int n, int k, int64_t lda, int64_t ldw) {
-  return (m >= 1 && m <= 64 && n >= 1 && k >= 32 && k % 32 == 0 && lda % 8 == 0 && ldw % 8 == 0) ? 1 : 0;
+  return (m >= 1 && m <= 128 && n >= 1 && k >= 32 && k % 32 == 0 && lda % 8 == 0 && ldw % 8 == 0) ? 1 : 0;
 }
 
 // How many ranges K is cut into for these sizes on the current device (the caller sizes
@@ -152,7 +152,7 @@ extern "C" int mi_gemm_mid_bf16_ranges(int n, int k) {
 extern "C" int mi_gemm_mid_partial_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, float* part,
                                         int m, int n, int k, hipStream_t stream) {
   MI_REQUIRE(mi_gemm_mid_bf16_supported(m, n, k, lda, ldw),
-             "gemm_mid_partial_bf16: takes 1 <= m <= 64, k a multiple of 32, rows aligned to 16 bytes; "
+             "gemm_mid_partial_bf16: takes 1 <= m <= 128, k a multiple of 32, rows aligned to 16 bytes; "
              "got m=%d n=%d k=%d lda=%lld ldw=%lld", m, n, k, (long long)lda, (long long)ldw);
   MI_REQUIRE(lda >= k && ldw >= k, "gemm_mid_partial_bf16: a row stride is shorter than its row");
   const int ranges = mi_gemm_mid_bf16_ranges(n, k);
@@ -165,7 +165,8 @@ extern "C" int mi_gemm_mid_partial_bf16(const void* a, int64_t lda, const void* 
                                                                    part, m, n, k, per_range)
   if (m <= 16) MID_GO(1);
   else if (m <= 32) MID_GO(2);
-  else MID_GO(4);
+  else if (m <= 64) MID_GO(4);
+  else MID_GO(8);
 #undef MID_GO
   MI_CHECK_LAUNCH("gemm_mid_partial_bf16");
   return MI_OK;

@@ -321,7 +321,7 @@ def skinny_gemm_takes(m: int, k: int, lda: int, ldw: int) -> bool:
     return 1 <= m <= SKINNY_MAX_ROWS and k >= 32 and k % 32 == 0 and lda % 8 == 0 and ldw % 8 == 0
 
 
-PARTIAL_SUMS_MAX_ROWS = 64
+PARTIAL_SUMS_MAX_ROWS = 128
 
 
 def partial_sums_pay(m: int, n: int, k: int) -> bool:
@@ -337,6 +337,9 @@ def partial_sums_pay(m: int, n: int, k: int) -> bool:
         3072 x 3072  (3B o)        8 / 8     9 / 8    11 / 9     16 / 11
         8192 x 8192  (70B o)      29 / 36   33 / 36   31 / 38    34 / 40
 
+    and at 96 / 128 rows 63 / 75 against 36 / 39 (8B down), 22 / 24 against 16 / 18 (8B o),
+    121 / 201 against 130 / 131 (70B down)
+
     so: a long K from 5 rows on (with fewer rows the step as a whole ran 0.5 % slower this
     way at 8B sizes), a small square-ish product from 12 rows on, nothing else.  Whole
     steps at 8B sizes: batch 8 / 16 / 64 run 1.6 / 5 / 2.8 % faster."""
@@ -348,7 +351,7 @@ def partial_sums_pay(m: int, n: int, k: int) -> bool:
 
 
 def linear_partial_sums(x: torch.Tensor, weight: torch.Tensor) -> PartialSums:
-    """`x @ weight.T` for up to 64 bfloat16 rows as float32 sums over ranges of K."""
+    """`x @ weight.T` for up to 128 bfloat16 rows as float32 sums over ranges of K."""
     _need_cuda(x, weight)
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or x.dim() != 2 or weight.dim() != 2:
         raise KernelShapeError("linear_partial_sums takes 2-D bfloat16 tensors")
@@ -362,7 +365,7 @@ def linear_partial_sums(x: torch.Tensor, weight: torch.Tensor) -> PartialSums:
         or not lib.mi_gemm_mid_bf16_supported(m, n, k, x.stride(0), weight.stride(0))
     ):
         raise KernelShapeError(
-            f"linear_partial_sums takes 1 to 64 rows, K a multiple of 32, rows aligned to 16 bytes; "
+            f"linear_partial_sums takes 1 to 128 rows, K a multiple of 32, rows aligned to 16 bytes; "
             f"got x {tuple(x.shape)} strides {x.stride()}, weight {tuple(weight.shape)} strides {weight.stride()}"
         )
     ranges = lib.mi_gemm_mid_bf16_ranges(n, k)
@@ -383,7 +386,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, partial_ok: bool = False) -> t
     the vendor GEMM library through torch, as the reference's engine does
     (distributed/linear.py:167, `F.linear` -> the vendor BLAS).
     With `partial_ok` the result may come as `PartialSums` where that pays
-    (`partial_sums_pay`: up to 64 rows, few features, a long K).
+    (`partial_sums_pay`: up to 128 rows, few features, a long K).
     """
     if x.dtype == torch.float32:
         return gemm_f32(x, weight)

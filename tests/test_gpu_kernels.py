@@ -128,7 +128,7 @@ def test_gemm_skinny_bf16(m, n, k):
 @pytest.mark.parametrize(
     "m,n,k",
     [(1, 4096, 14336), (8, 1000, 8192 + 32), (16, 4096, 4096), (17, 1003, 4096), (33, 136, 608), (64, 4096, 14336),
-     (47, 5, 32), (64, 260, 8192 - 224)],
+     (47, 5, 32), (64, 260, 8192 - 224), (128, 4096, 4096), (101, 200, 1024 + 64)],
 )
 def test_linear_in_partial_sums_then_norm_is_linear_then_norm(m, n, k):
     """A product left as sums over ranges of K, added up by the norm that follows it: the
@@ -165,15 +165,15 @@ def test_linear_leaves_partial_sums_only_where_asked_and_where_it_pays():
     assert isinstance(ops.linear(a, w), torch.Tensor)
     assert not ops.partial_sums_pay(8, 64, 4096) and ops.partial_sums_pay(12, 64, 4096)
     assert not ops.partial_sums_pay(4, 64, 12288) and not ops.partial_sums_pay(16, 3072, 8192)
-    assert not ops.partial_sums_pay(65, 64, 12288) and not ops.partial_sums_pay(8, 28672, 12288)
+    assert not ops.partial_sums_pay(129, 64, 12288) and not ops.partial_sums_pay(8, 28672, 12288)
     assert isinstance(ops.linear(a[:, :4096].contiguous(), w[:, :4096].contiguous(), partial_ok=True), torch.Tensor)
     assert isinstance(ops.linear(a.float(), w.float(), partial_ok=True), torch.Tensor)
     partial = ops.linear(a, w, partial_ok=True)
     with pytest.raises(KernelShapeError, match="partial sums"):
         ops.add_rmsnorm(ops.PartialSums(partial.pieces[:, :1].contiguous(), torch.bfloat16), _rand(8, 64),
                         _rand(64, dtype=torch.bfloat16), 1e-5)
-    with pytest.raises(KernelShapeError, match="1 to 64 rows"):
-        ops.linear_partial_sums(_rand(65, 64, dtype=torch.bfloat16), _rand(16, 64, dtype=torch.bfloat16))
+    with pytest.raises(KernelShapeError, match="1 to 128 rows"):
+        ops.linear_partial_sums(_rand(129, 64, dtype=torch.bfloat16), _rand(16, 64, dtype=torch.bfloat16))
 
 
 @pytest.mark.parametrize(
