@@ -62,3 +62,41 @@ def test_real_widths_under_three_schedules(wide, dtype):
             ru.assert_close(got[rid], expected[rid], dtype, f"8B widths, {name}, request {rid}")
         runner.cache.check()
     assert runner.num_free_blocks() == 8
+
+
+def test_single_tokens_over_a_longer_context_at_real_widths(wide, monkeypatch):
+    """One request of 600 tokens, the last 10 one by one in bfloat16 through the replayed decode
+    step: at these widths and this context a single token's attention is left in its key ranges
+    and combined by the output projection, and the down product is summed up by the next norm
+    from 5 rows on (the 7-token portion)."""
+    import mini_infer_amd.ops as ops
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.ops import kernels
+
+    calls = {"from_attention": 0, "partial_sums": 0}
+    from_attention, partial_sums = ops.linear_from_attention, kernels.linear_partial_sums
+
+    def count_from_attention(*args):
+        calls["from_attention"] += 1
+        return from_attention(*args)
+
+    def count_partial_sums(*args):
+        calls["partial_sums"] += 1
+        return partial_sums(*args)
+
+    monkeypatch.setattr(ops, "linear_from_attention", count_from_attention)
+    monkeypatch.setattr(kernels, "linear_partial_sums", count_partial_sums)
+    folder, _, _ = wide
+    tokens = tiny.random_tokens(WIDE, 600, seed=5)
+    expected = plain_llama.llama_logits(WIDE, tiny.make_weights(WIDE, seed=8), np.array(tokens))  # the fixture's weights
+    runner = ModelRunner.from_pretrained(folder, dtype="bfloat16", num_blocks=40, block_size=16)
+    got = [runner.step([StepEntry("r", tokens[:583], [582])]).cpu().numpy()]
+    got.append(runner.step([StepEntry("r", tokens[583:590], list(range(7)))]).cpu().numpy())
+    for at in range(590, 600):
+        got.append(runner.step([StepEntry("r", tokens[at : at + 1], [0])]).cpu().numpy())
+    seen = expected.copy()
+    seen[582:600] = np.concatenate(got)
+    ru.assert_close(seen, expected, "bfloat16", "8B widths, 600 tokens")
+    assert calls["from_attention"] >= 1 and calls["partial_sums"] >= 1  # (a replayed step calls nothing)
+    runner.free_request("r")
+    assert runner.num_free_blocks() == 40
