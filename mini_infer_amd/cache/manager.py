@@ -1,7 +1,7 @@
 """The cache manager: pages of keys and values, block tables, state slots.
 
-Layer calls whose needs agree (same key/value heads, head size and window) form
-a *group*.  Each group has its own page storage, its own pool of page ids and,
+Layer calls whose needs agree (same key/value heads, key and value widths, window
+and value layout) form a *group*.  Each group has its own page storage, its own pool of page ids and,
 per request, its own block table; pages are shared by all calls of the group
 (one id addresses the same page in every call's storage, as the reference's
 block ids are global across layers: cache/block_pool.py:338-351).
@@ -15,9 +15,11 @@ Life of a request:
                    the pages no future query can see
   free_request     every page and the state slot go back; ids are reused at once
 
-Storage layout per group: [calls, 2 (k, v), num_pages, kv_heads, page_size * head_dim];
-a key chunk is [page_size][head_dim]; a value chunk is the same, or transposed
-([head_dim][page_size]) where the matrix-core attention kernel will read it.
+Storage per group: keys [calls, num_pages, kv_heads, page_size * head_dim] and values
+[calls, num_pages, kv_heads, page_size * value dim], sized apart (a mixer may keep
+values of another width than its keys, or none).  A key chunk is
+[page_size][head_dim]; a value chunk is [page_size][value dim], or transposed
+([value dim][page_size]) if the mixer that reads it asked for that layout.
 """
 
 from __future__ import annotations
@@ -31,7 +33,6 @@ import torch
 from mini_infer_amd.cache.page_pool import PagePool
 from mini_infer_amd.cache.state_slots import StateSlots
 from mini_infer_amd.exceptions import OutOfMemoryError
-from mini_infer_amd.ops.kernels import mfma_attention_supported
 from mini_infer_amd.parts.base import CacheNeeds, LayerCache, StateNeeds
 
 RELEASED = -1  # block-table entry of a page a window has passed
@@ -45,8 +46,10 @@ class PageGroup:
     head_dim: int
     window: int | None
     pool: PagePool
-    storage: torch.Tensor | None = None
-    v_transposed: bool = False  # values stored [head_dim][slot] inside a page (matrix-core attention)
+    value_dim: int = 0  # width of a value row; 0: the group keeps no values
+    v_transposed: bool = False  # values stored [dim][slot] inside a page, as its mixers asked
+    k_storage: torch.Tensor | None = None
+    v_storage: torch.Tensor | None = None
     tables: dict[Hashable, list[int]] = dataclasses.field(default_factory=dict)
 
     def first_live_page(self, length: int, page_size: int) -> int:
@@ -98,16 +101,21 @@ class CacheManager:
             if need is None:
                 continue
             if need.pages is not None:
-                key = (need.pages.num_kv_heads, need.pages.head_dim, need.pages.window)
+                pages = need.pages
+                if pages.num_kv_heads <= 0 or pages.head_dim <= 0 or pages.value_dim < 0:
+                    raise ValueError(f"call {call}: impossible page needs {pages}")
+                key = (pages.num_kv_heads, pages.head_dim, pages.value_dim, pages.window, pages.v_transposed)
                 group = by_shape.get(key)
                 if group is None:
                     group = PageGroup(
                         index=len(self.groups),
                         calls=[],
-                        num_kv_heads=need.pages.num_kv_heads,
-                        head_dim=need.pages.head_dim,
-                        window=need.pages.window,
+                        num_kv_heads=pages.num_kv_heads,
+                        head_dim=pages.head_dim,
+                        window=pages.window,
                         pool=PagePool(num_pages),
+                        value_dim=pages.value_dim,
+                        v_transposed=pages.v_transposed,
                     )
                     by_shape[key] = group
                     self.groups.append(group)
@@ -116,13 +124,15 @@ class CacheManager:
             if need.state is not None:
                 state_needs[call] = need.state
         for group in self.groups:
-            group.v_transposed = mfma_attention_supported(dtype, group.head_dim, page_size)
             if allocate_storage:
-                group.storage = torch.zeros(
-                    (len(group.calls), 2, num_pages, group.num_kv_heads, page_size * group.head_dim),
-                    dtype=dtype,
-                    device=self.device,
+                calls, heads = len(group.calls), group.num_kv_heads
+                group.k_storage = torch.zeros(
+                    (calls, num_pages, heads, page_size * group.head_dim), dtype=dtype, device=self.device
                 )
+                if group.value_dim > 0:
+                    group.v_storage = torch.zeros(
+                        (calls, num_pages, heads, page_size * group.value_dim), dtype=dtype, device=self.device
+                    )
         self.states = StateSlots(max_requests, state_needs, self.device, allocate_storage)
         self._num_calls = len(needs)
         self._lengths: dict[Hashable, int] = {}
@@ -193,6 +203,18 @@ class CacheManager:
         for request_id, new_tokens in extents.items():
             for group, count in zip(self.groups, self.pages_needed(request_id, new_tokens)):
                 group.tables[request_id].extend(group.pool.allocate_many(count))
+
+    def cancel_reservation(self, extents: dict[Hashable, int]) -> None:
+        """Undo a `reserve` whose step did not happen: pages past what each request's
+        committed length needs go back; lengths were never advanced."""
+        for request_id in extents:
+            keep = self.pages_for_tokens(self._lengths[request_id])
+            for group in self.groups:
+                table = group.tables[request_id]
+                while len(table) > keep:
+                    page = table.pop()
+                    if page != RELEASED:
+                        group.pool.free(page)
 
     def commit(self, extents: dict[Hashable, int]) -> None:
         """Advance lengths after a step and give back what windows have passed."""
@@ -284,13 +306,12 @@ class CacheManager:
             for i, call in enumerate(group.calls):
                 caches[call].group = group.index
                 caches[call].v_transposed = group.v_transposed
-                if group.storage is not None:
-                    pages, heads = self.num_pages, group.num_kv_heads
-                    caches[call].k_pages = group.storage[i, 0].view(pages, heads, self.page_size, group.head_dim)
-                    if group.v_transposed:
-                        caches[call].v_pages = group.storage[i, 1].view(pages, heads, group.head_dim, self.page_size)
-                    else:
-                        caches[call].v_pages = group.storage[i, 1].view(pages, heads, self.page_size, group.head_dim)
+                pages, heads = self.num_pages, group.num_kv_heads
+                if group.k_storage is not None:
+                    caches[call].k_pages = group.k_storage[i].view(pages, heads, self.page_size, group.head_dim)
+                if group.v_storage is not None:
+                    shape = (group.value_dim, self.page_size) if group.v_transposed else (self.page_size, group.value_dim)
+                    caches[call].v_pages = group.v_storage[i].view(pages, heads, *shape)
         for call, tensor in self.states.tensors.items():
             caches[call].state = tensor
         return caches

@@ -7,7 +7,9 @@
 //
 // Semantics follow the reference's oracle (cache/packed_attention.py:296-338):
 // query head h reads key/value head h / (Hq/Hkv); a query at absolute position p
-// sees keys 0..p, or p-window+1..p with a window.
+// sees keys 0..p, or p-window+1..p with a window.  With `slopes` (one float per
+// query head, may be null) the score of the key at position j gets
+// slopes[h] * (j - p) added before the softmax: a bias linear in the distance.
 //
 // Layout: q rows [token][head][head_dim] with a row stride; pages
 // [num_pages][kv_heads][page_size][head_dim]; block_table[request][i] is the page
@@ -29,7 +31,8 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     const T* __restrict__ v_pages, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ token_request, const int* __restrict__ positions, T* __restrict__ out,
     int64_t out_row_stride, float* __restrict__ part_acc, float* __restrict__ part_ml, int q_heads,
-    int kv_heads, int head_dim, int page_size, float scale, int window, int num_splits) {
+    int kv_heads, int head_dim, int page_size, float scale, int window, int num_splits,
+    const float* __restrict__ slopes) {
   extern __shared__ float q_lds[];  // [GT][head_dim], pre-multiplied by the scale
   constexpr int KV = 16 / sizeof(T);  // elements in a 16-byte load
 
@@ -67,6 +70,9 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     for (int v = 0; v < VPL; ++v) acc[g][v] = 0.f;
   }
   const bool owns_dims = lane * VPL < head_dim;
+  float slope[GT];
+#pragma unroll
+  for (int g = 0; g < GT; ++g) slope[g] = (slopes != nullptr && g < nh) ? slopes[head0 + g] : 0.f;
 
   for (int base = a; base < b; base += MI_WAVE) {
     const int key = base + lane;
@@ -90,6 +96,9 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
           for (int g = 0; g < GT; ++g) s[g] += q_lds[g * head_dim + d + e] * kf;
         }
       }
+      const float distance = (float)(key - pos);
+#pragma unroll
+      for (int g = 0; g < GT; ++g) s[g] += slope[g] * distance;
     }
     float p[GT];
 #pragma unroll
@@ -235,7 +244,7 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
                                int64_t out_row_stride, float* part_acc, float* part_ml,
                                int num_tokens, int q_heads, int kv_heads, int head_dim,
                                int page_size, float scale, int window, int num_splits,
-                               hipStream_t stream) {
+                               const float* slopes, hipStream_t stream) {
   const int group = q_heads / kv_heads;
   dim3 grid(num_tokens, kv_heads * ceil_div(group, GT), num_splits);
   const size_t lds = sizeof(float) * GT * head_dim;
@@ -243,7 +252,7 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
   attn_generic_kernel<T, VPL><<<grid, MI_WAVE, lds, stream>>>(                                    \
       (const T*)q, q_row_stride, (const T*)k_pages, (const T*)v_pages, block_table, max_blocks,   \
       token_request, positions, (T*)out, out_row_stride, part_acc, part_ml, q_heads, kv_heads,    \
-      head_dim, page_size, scale, window, num_splits)
+      head_dim, page_size, scale, window, num_splits, slopes)
   if (head_dim <= 64) MI_ATTN_LAUNCH(1);
   else if (head_dim <= 128) MI_ATTN_LAUNCH(2);
   else MI_ATTN_LAUNCH(4);
@@ -258,15 +267,9 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
   return MI_OK;
 }
 
-// part_acc holds num_tokens*q_heads*num_splits*head_dim floats and part_ml
-// num_tokens*q_heads*num_splits*2 floats; both may be null when num_splits == 1.
-extern "C" int mi_attn_generic(int dtype, const void* q, int64_t q_row_stride, const void* k_pages,
-                               const void* v_pages, const int* block_table, int max_blocks,
-                               const int* token_request, const int* positions, void* out,
-                               int64_t out_row_stride, float* part_acc, float* part_ml,
-                               int num_tokens, int q_heads, int kv_heads, int head_dim,
-                               int page_size, int num_pages, float scale, int window,
-                               int num_splits, hipStream_t stream) {
+static int attn_generic_check(int dtype, int64_t q_row_stride, int max_blocks, int64_t out_row_stride,
+                              int num_tokens, int q_heads, int kv_heads, int head_dim, int page_size,
+                              int num_pages, int window, int num_splits) {
   MI_REQUIRE(num_tokens >= 0 && q_heads > 0 && kv_heads > 0, "attn_generic: bad sizes tokens=%d q_heads=%d kv_heads=%d",
              num_tokens, q_heads, kv_heads);
   MI_REQUIRE(q_heads % kv_heads == 0, "attn_generic: q_heads=%d is not a multiple of kv_heads=%d",
@@ -279,21 +282,37 @@ extern "C" int mi_attn_generic(int dtype, const void* q, int64_t q_row_stride, c
              "attn_generic: the cache has too many key rows for 32-bit row indices");
   MI_REQUIRE(window >= 0, "attn_generic: window=%d must be 0 (none) or positive", window);
   MI_REQUIRE(num_splits >= 1 && num_splits <= 64, "attn_generic: num_splits=%d must be 1..64", num_splits);
-  MI_REQUIRE(num_splits == 1 || (part_acc && part_ml), "attn_generic: split keys need partial buffers");
   MI_REQUIRE(q_row_stride >= (int64_t)q_heads * head_dim && out_row_stride >= (int64_t)q_heads * head_dim,
              "attn_generic: row strides shorter than q_heads*head_dim");
   MI_REQUIRE(kv_heads * ceil_div(q_heads / kv_heads, GT) <= 65535, "attn_generic: too many heads");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "attn_generic: unknown dtype %d", dtype);
+  return MI_OK;
+}
+
+// part_acc holds num_tokens*q_heads*num_splits*head_dim floats and part_ml
+// num_tokens*q_heads*num_splits*2 floats; both may be null when num_splits == 1.
+// `slopes` (q_heads floats) may be null.
+extern "C" int mi_attn_generic(int dtype, const void* q, int64_t q_row_stride, const void* k_pages,
+                               const void* v_pages, const int* block_table, int max_blocks,
+                               const int* token_request, const int* positions, void* out,
+                               int64_t out_row_stride, float* part_acc, float* part_ml,
+                               int num_tokens, int q_heads, int kv_heads, int head_dim,
+                               int page_size, int num_pages, float scale, int window,
+                               int num_splits, const float* slopes, hipStream_t stream) {
+  const int bad = attn_generic_check(dtype, q_row_stride, max_blocks, out_row_stride, num_tokens, q_heads,
+                                     kv_heads, head_dim, page_size, num_pages, window, num_splits);
+  if (bad != MI_OK) return bad;
+  MI_REQUIRE(num_splits == 1 || (part_acc && part_ml), "attn_generic: split keys need partial buffers");
   if (num_tokens == 0) return MI_OK;
   if (dtype == MI_F32)
     return attn_generic_launch<float>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
                                       token_request, positions, out, out_row_stride, part_acc, part_ml,
                                       num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
-                                      num_splits, stream);
+                                      num_splits, slopes, stream);
   return attn_generic_launch<bf16_t>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
                                      token_request, positions, out, out_row_stride, part_acc, part_ml,
                                      num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
-                                     num_splits, stream);
+                                     num_splits, slopes, stream);
 }
 
 // The combining step alone, for partials written by the matrix-core kernel.

@@ -70,7 +70,7 @@ class ModelRunner:
         self.block_size = block_size
         self.num_blocks = num_blocks
         self.cache = CacheManager(
-            model.cache_needs(),
+            model.cache_needs(block_size),
             page_size=block_size,
             num_pages=num_blocks,
             max_requests=max_concurrent,
@@ -153,7 +153,10 @@ class ModelRunner:
         Rows come in the order of `entries` and, within an entry, of its `want`.
         The tensor may be reused by the next step: read or copy it before calling
         `step` again.  Requests seen for the first time are admitted.  Raises `OutOfMemoryError`
-        before anything changes if the pages for this step are not there.
+        before anything changes if the pages for this step are not there; any other failure
+        (a kernel that refuses a size, an error on the device) gives the step's pages back
+        and forgets the requests it admitted, so lengths and free pages are what they were.
+        State of fixed size that a mixer had already updated in place is not restored.
 
         `device_tokens` (int32, on the device) holds token ids the host has not read yet,
         e.g. what `sample_tokens` returned for the last step; an entry with `device_row`
@@ -206,19 +209,30 @@ class ModelRunner:
                 self.cache.free_request(request_id)
             raise
 
-        index = self.cache.build_step_index([(e.request_id, len(e.tokens)) for e in entries])
-        rows = np.fromiter(
-            (int(index.cu_seqlens_q[b]) + w for b, e in enumerate(entries) for w in e.want),
-            dtype=np.int32,
-        )
-        token_ids = token_ids.astype(np.int32)
-        if self.decode_graphs is not None and self.decode_graphs.takes(index, rows, device_tokens):
-            logits = self.decode_graphs.run(token_ids, index, from_rows, device_tokens)
-        else:
-            ctx, from_rows_device = self._to_device(token_ids, rows, index, from_rows)
-            if from_rows_device is not None:
-                ops.take_device_tokens(ctx.token_ids, from_rows_device, device_tokens, self.vocab_size)
-            logits = self.model.forward(ctx, self._layer_caches)
+        # From here on pages are reserved: whatever fails below (building the index, the copy
+        # to the device, a kernel that refuses a size) gives them back, so that the cache is
+        # as it was before the step (the reference's rollback on a failed step:
+        # scheduler/continuous_scheduler.py:418-445).  Keys and values the failed step may
+        # have written lie past every request's length and are overwritten later.
+        try:
+            index = self.cache.build_step_index([(e.request_id, len(e.tokens)) for e in entries])
+            rows = np.fromiter(
+                (int(index.cu_seqlens_q[b]) + w for b, e in enumerate(entries) for w in e.want),
+                dtype=np.int32,
+            )
+            token_ids = token_ids.astype(np.int32)
+            if self.decode_graphs is not None and self.decode_graphs.takes(index, rows, device_tokens):
+                logits = self.decode_graphs.run(token_ids, index, from_rows, device_tokens)
+            else:
+                ctx, from_rows_device = self._to_device(token_ids, rows, index, from_rows)
+                if from_rows_device is not None:
+                    ops.take_device_tokens(ctx.token_ids, from_rows_device, device_tokens, self.vocab_size)
+                logits = self.model.forward(ctx, self._layer_caches)
+        except BaseException:
+            self.cache.cancel_reservation(extents)
+            for request_id in admitted:
+                self.cache.free_request(request_id)
+            raise
         self.cache.commit(extents)
         return logits
 
@@ -242,7 +256,7 @@ class ModelRunner:
         if from_rows is not None:
             pieces.append(from_rows)
         sizes = [int(p.size) for p in pieces]
-        staging = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=True)
+        staging = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=self.device.type == "cuda")
         host = staging.numpy()
         offset = 0
         for piece, size in zip(pieces, sizes):

@@ -1,7 +1,7 @@
 """A decoder-only language model assembled from a `ModelSpec`.
 
-Embedding -> layer calls in `spec.order` -> final norm at the requested rows ->
-output head, the reference's `LlamaForCausalLM.forward`
+Embedding part -> layer calls in `spec.order` -> final norm at the requested rows ->
+head part, the reference's `LlamaForCausalLM.forward`
 (models/llama/llama.py:149-172) with `run_decoder_layers`
 (models/blocks/transformer_block.py:123-153), but driven by data: nothing here
 names an architecture.
@@ -20,8 +20,7 @@ from mini_infer_amd.parts.base import (
     StepContext,
     TensorGetter,
 )
-from mini_infer_amd.parts.embedding import OutputHead, TokenEmbedding
-from mini_infer_amd.registry import BLOCKS, NORMS
+from mini_infer_amd.registry import BLOCKS, EMBEDDINGS, HEADS, NORMS
 
 
 class DecoderModel:
@@ -32,19 +31,15 @@ class DecoderModel:
         self.dtype = dtype
         self.device = torch.device(device)
         shared: dict = {}
-        self.embedding = TokenEmbedding(spec.vocab_size, spec.hidden_size, spec.embedding_name, dtype, device)
+        embedding = spec.embedding_description()
+        self.embedding = EMBEDDINGS.lookup(embedding["kind"])(embedding, dtype, device, shared)
+        shared["embedding"] = self.embedding  # a tied head finds its table here
         self.blocks: list[Block] = [
             BLOCKS.lookup(layer.block["kind"])(layer.block, dtype, device, shared) for layer in spec.layers
         ]
         self.final_norm = NORMS.lookup(spec.final_norm["kind"])(spec.final_norm, dtype, device, shared)
-        self.head = OutputHead(
-            spec.hidden_size,
-            spec.vocab_size,
-            spec.head_name,
-            dtype,
-            device,
-            tied_to=self.embedding if spec.tie_word_embeddings else None,
-        )
+        head = spec.head_description()
+        self.head = HEADS.lookup(head["kind"])(head, dtype, device, shared)
         # a product whose output only ever meets norms that can add up its pieces may leave them apart
         if self.final_norm.takes_partial_sums and all(block.takes_partial_sums for block in self.blocks):
             for block in self.blocks:
@@ -78,10 +73,10 @@ class DecoderModel:
 
     # -- cache ----------------------------------------------------------------
 
-    def cache_needs(self) -> list[CacheNeeds | None]:
+    def cache_needs(self, page_size: int) -> list[CacheNeeds | None]:
         """Per call in `order`: what its own cache must hold, or None if it reads another's."""
         return [
-            None if call.reads_cache_of is not None else self.blocks[call.layer].mixer.cache_needs()
+            None if call.reads_cache_of is not None else self.blocks[call.layer].mixer.cache_needs(page_size)
             for call in self.spec.order
         ]
 
@@ -89,7 +84,7 @@ class DecoderModel:
 
     def forward(self, ctx: StepContext, caches: list[LayerCache]) -> torch.Tensor:
         """Logits [len(ctx.logit_rows), vocab] float32.  `caches[i]` belongs to call i."""
-        residual = self.embedding.forward(ctx.token_ids)
+        residual = self.embedding.forward(ctx)
         delta: torch.Tensor | None = None
         for i, call in enumerate(self.spec.order):
             own = call.reads_cache_of is None
@@ -98,4 +93,4 @@ class DecoderModel:
         if ctx.logit_rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         h = self.final_norm.forward(delta, residual, rows=ctx.logit_rows)
-        return self.head.forward(h)
+        return self.head.forward(h, ctx)

@@ -38,6 +38,23 @@ class ModelSpec:
     head_name: str
     tie_word_embeddings: bool
     max_position_embeddings: int | None = None
+    # How the residual stream starts and how it ends, by kind like every other part
+    # ({"kind": ..., ...}).  None: the plain table lookup under `embedding_name`, and the
+    # plain product with the matrix under `head_name` (the table itself when tied).
+    embedding: dict[str, Any] | None = None
+    head: dict[str, Any] | None = None
+
+    def embedding_description(self) -> dict[str, Any]:
+        if self.embedding is not None:
+            return self.embedding
+        return {"kind": "token_embedding", "vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
+                "name": self.embedding_name}
+
+    def head_description(self) -> dict[str, Any]:
+        if self.head is not None:
+            return self.head
+        return {"kind": "linear_head", "vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
+                "name": self.head_name, "tied": self.tie_word_embeddings}
 
     def __post_init__(self) -> None:
         for i, call in enumerate(self.order):

@@ -55,6 +55,9 @@ def _check_v_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, v_transposed: b
 
 
 MFMA_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
+# what the plain attention kernel (and so the engine as a whole) takes
+ATTENTION_HEAD_DIM_STEP = 16
+ATTENTION_MAX_HEAD_DIM = 256
 
 
 def mfma_attention_supported(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
@@ -629,8 +632,13 @@ def paged_attention(
     v_transposed: bool = False,
     force_plain: bool = False,
     combine: bool = True,
+    slopes: torch.Tensor | None = None,
 ) -> torch.Tensor | AttentionPieces:
     """Causal attention of every token over its request's pages; returns [T, q_heads*head_dim].
+
+    `slopes` (float32 [q_heads], optional): the score of head h for the key at position j
+    seen from position p gets `slopes[h] * (j - p)` added before the softmax.  Only the
+    plain kernel knows it.
 
     With `combine=False` a step of single tokens whose keys are cut into ranges (the
     matrix-core kernel) comes back as `AttentionPieces`, for `linear_from_attention`.
@@ -682,6 +690,13 @@ def paged_attention(
         )
     if v_transposed and force_plain:
         raise KernelShapeError("the plain attention kernel reads value pages that are not transposed")
+    if slopes is not None:
+        _need_cuda(slopes)
+        _need_contiguous("slopes", slopes)
+        if slopes.dtype != torch.float32 or slopes.numel() != q_heads:
+            raise KernelShapeError(f"slopes must be float32 [{q_heads}], got {slopes.dtype} x {slopes.numel()}")
+        if use_mfma:
+            raise KernelShapeError("the matrix-core attention kernel takes no score slopes; keep values untransposed")
 
     def partials(splits: int, rows: int = tokens) -> tuple[torch.Tensor | None, torch.Tensor | None]:
         if splits == 1:
@@ -754,7 +769,7 @@ def paged_attention(
             _dtype_code(q), _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             block_table.shape[1], _ptr(token_request), _ptr(positions), _ptr(out), out.stride(0),
             _ptr(part_acc), _ptr(part_ml), tokens, q_heads, kv_heads, head_dim, page_size, num_pages,
-            float(scale), int(window or 0), splits, _stream(),
+            float(scale), int(window or 0), splits, _ptr(slopes), _stream(),
         )
     )
     return out

@@ -1,10 +1,12 @@
 """Parts a layer is put together from.  Importing this package registers the built-in kinds."""
 
-from mini_infer_amd.parts import attention, block, feed_forward, norm, position  # noqa: F401
+from mini_infer_amd.parts import attention, block, embedding, feed_forward, norm, position  # noqa: F401
 from mini_infer_amd.parts.base import (
     Block,
     CacheNeeds,
+    Embedding,
     FeedForward,
+    Head,
     LayerCache,
     Mixer,
     Norm,
@@ -12,6 +14,7 @@ from mini_infer_amd.parts.base import (
     ParamSpec,
     Part,
     PositionEncoding,
+    RotaryTables,
     StateNeeds,
     StepContext,
 )
@@ -19,7 +22,9 @@ from mini_infer_amd.parts.base import (
 __all__ = [
     "Block",
     "CacheNeeds",
+    "Embedding",
     "FeedForward",
+    "Head",
     "LayerCache",
     "Mixer",
     "Norm",
@@ -27,6 +32,7 @@ __all__ = [
     "ParamSpec",
     "Part",
     "PositionEncoding",
+    "RotaryTables",
     "StateNeeds",
     "StepContext",
 ]

@@ -21,11 +21,11 @@ from mini_infer_amd.parts.base import (
     Mixer,
     PagedKVNeeds,
     ParamSpec,
+    PositionEncoding,
     StepContext,
     TensorGetter,
 )
 from mini_infer_amd.parts.linear import Linear
-from mini_infer_amd.parts.position import RotaryPosition
 from mini_infer_amd.registry import POSITION_ENCODINGS, register_mixer
 
 
@@ -38,7 +38,7 @@ class GQAttention(Mixer):
         num_heads: int,
         num_kv_heads: int,
         head_dim: int,
-        position: RotaryPosition | None,
+        position: PositionEncoding | None,
         dtype: torch.dtype,
         device,
         *,
@@ -50,6 +50,11 @@ class GQAttention(Mixer):
             raise ValueError(f"num_heads={num_heads} is not a multiple of num_kv_heads={num_kv_heads}")
         if window is not None and window <= 0:
             raise ValueError(f"window must be positive, got {window}")
+        if head_dim <= 0 or head_dim % ops.ATTENTION_HEAD_DIM_STEP != 0 or head_dim > ops.ATTENTION_MAX_HEAD_DIM:
+            raise ValueError(
+                f"head_dim={head_dim}: the attention kernels take head sizes in steps of "
+                f"{ops.ATTENTION_HEAD_DIM_STEP} up to {ops.ATTENTION_MAX_HEAD_DIM}"
+            )
         self.hidden_size = hidden_size
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads
@@ -57,6 +62,12 @@ class GQAttention(Mixer):
         self.position = position
         self.window = window
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        # per-head slopes of a score bias linear in the distance, if the encoding has one
+        self.slopes = position.score_slopes(num_heads) if position is not None else None
+        if self.slopes is not None and (
+            self.slopes.dtype != torch.float32 or tuple(self.slopes.shape) != (num_heads,)
+        ):
+            raise ValueError(f"score slopes must be float32 [{num_heads}], got {self.slopes.dtype} {tuple(self.slopes.shape)}")
         q_width, kv_width = num_heads * head_dim, num_kv_heads * head_dim
         self.qkv = Linear(hidden_size, [q_width, kv_width, kv_width], ["q_proj", "k_proj", "v_proj"], dtype, device)
         self.out = Linear(q_width, hidden_size, "o_proj", dtype, device)
@@ -68,8 +79,13 @@ class GQAttention(Mixer):
         self.qkv.load_params(prefix, get)
         self.out.load_params(prefix, get)
 
-    def cache_needs(self) -> CacheNeeds:
-        return CacheNeeds(pages=PagedKVNeeds(self.num_kv_heads, self.head_dim, self.window))
+    def cache_needs(self, page_size: int) -> CacheNeeds:
+        # values lie transposed inside a page where the matrix-core kernel will read them
+        # (that kernel knows no score bias: such layers keep the plain layout and kernel)
+        transposed = self.slopes is None and ops.mfma_attention_supported(self.dtype, self.head_dim, page_size)
+        return CacheNeeds(
+            pages=PagedKVNeeds(self.num_kv_heads, self.head_dim, self.window, v_transposed=transposed)
+        )
 
     def forward(
         self, x: torch.Tensor, ctx: StepContext, cache: LayerCache, writes_cache: bool = True
@@ -77,14 +93,14 @@ class GQAttention(Mixer):
         assert cache.group is not None and cache.k_pages is not None and cache.v_pages is not None
         q_width = self.num_heads * self.head_dim
         assert self.qkv.weight is not None
-        if self.position is not None and ops.qkv_rope_write_takes(
-            x, self.qkv.weight, self.head_dim, self.position.rotary_dim, self.position.interleaved
+        rotary = self.position.rotary(ctx) if self.position is not None else None
+        if rotary is not None and ops.qkv_rope_write_takes(
+            x, self.qkv.weight, self.head_dim, rotary.rotary_dim, rotary.interleaved
         ):
             # few rows (decode): projection, rotation and cache write are one kernel
-            cos, sin = self.position.tables(ctx)
             kv_heads = self.num_kv_heads if writes_cache else 0
             queries = ops.qkv_rope_write(
-                x, self.qkv.weight if writes_cache else self.qkv.weight[:q_width], cos, sin,
+                x, self.qkv.weight if writes_cache else self.qkv.weight[:q_width], rotary.cos, rotary.sin,
                 ctx.slot_mapping[cache.group] if writes_cache else None, cache.k_pages, cache.v_pages,
                 q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
                 v_transposed=cache.v_transposed,
@@ -95,24 +111,18 @@ class GQAttention(Mixer):
             kv_heads, slots = self.num_kv_heads, ctx.slot_mapping[cache.group]
         else:
             # reads another call's keys and values: only q is projected
-            assert self.qkv.weight is not None
             qkv = ops.linear(x, self.qkv.weight[:q_width])
             kv_heads, slots = 0, None
-        if self.position is not None:
-            cos, sin = self.position.tables(ctx)
-            ops.rope_kv_write(
-                qkv, cos, sin, slots, cache.k_pages, cache.v_pages,
-                q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
-                rotary_dim=self.position.rotary_dim, interleaved=self.position.interleaved,
-                v_transposed=cache.v_transposed,
-            )
+        if rotary is not None:
+            cos, sin, rotary_dim, interleaved = rotary.cos, rotary.sin, rotary.rotary_dim, rotary.interleaved
         else:
-            empty = torch.empty((ctx.num_tokens, 0), dtype=torch.float32, device=x.device)
-            ops.rope_kv_write(
-                qkv, empty, empty, slots, cache.k_pages, cache.v_pages,
-                q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
-                rotary_dim=0, interleaved=False, v_transposed=cache.v_transposed,
-            )
+            cos = sin = torch.empty((ctx.num_tokens, 0), dtype=torch.float32, device=x.device)
+            rotary_dim, interleaved = 0, False
+        ops.rope_kv_write(
+            qkv, cos, sin, slots, cache.k_pages, cache.v_pages,
+            q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
+            rotary_dim=rotary_dim, interleaved=interleaved, v_transposed=cache.v_transposed,
+        )
         return self._project(self._attend(qkv, ctx, cache))
 
     def _project(self, attended):
@@ -131,7 +141,7 @@ class GQAttention(Mixer):
             queries, cache.k_pages, cache.v_pages, ctx.block_tables[cache.group], ctx.token_request,
             ctx.positions, ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
-            max_seq_len=ctx.max_seq_len, v_transposed=cache.v_transposed, combine=not few,
+            max_seq_len=ctx.max_seq_len, v_transposed=cache.v_transposed, combine=not few, slopes=self.slopes,
         )
 
 

@@ -66,11 +66,25 @@ class Part:
 
 @dataclasses.dataclass(frozen=True)
 class PagedKVNeeds:
-    """Keys and values per token, kept in pages.  `window=None` keeps all of them."""
+    """What a mixer keeps per token in pages: per key/value head one key row of `head_dim`
+    values and one value row of `v_head_dim` values (None: as wide as the keys; 0: no value
+    stream at all, the mixer keeps a single stream and gets no value pages).
+
+    `window=None` keeps every token; with a window, pages that no future query can see
+    are given back.  `v_transposed` is the layout of a value page, chosen by the mixer
+    for the kernel that will read it: `[slot][dim]` (False) or `[dim][slot]` (True).
+    Layer calls whose needs are equal share one page group.
+    """
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    v_head_dim: int | None = None
+    v_transposed: bool = False
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclasses.dataclass(frozen=True)
@@ -93,7 +107,9 @@ class LayerCache:
 
     group: int | None = None  # which page group's block table and write slots apply
     k_pages: torch.Tensor | None = None  # [num_pages, kv_heads, page_size, head_dim]
-    v_pages: torch.Tensor | None = None  # same, or [num_pages, kv_heads, head_dim, page_size] if transposed
+    # [num_pages, kv_heads, page_size, value dim], or [num_pages, kv_heads, value dim, page_size]
+    # if transposed; None for a mixer that asked for no value stream
+    v_pages: torch.Tensor | None = None
     v_transposed: bool = False
     state: torch.Tensor | None = None  # [max_requests, *state shape]
 
@@ -165,8 +181,37 @@ class Norm(Part):
         raise NotImplementedError
 
 
+@dataclasses.dataclass
+class RotaryTables:
+    """Rotation of the first `rotary_dim` dims of every query and key head by the angle of
+    its token: `cos`, `sin` are float32 [T, rotary_dim/2] for the step's tokens;
+    `interleaved` pairs dim 2j with 2j+1, otherwise j with j + rotary_dim/2."""
+
+    cos: torch.Tensor
+    sin: torch.Tensor
+    rotary_dim: int
+    interleaved: bool = False
+
+
 class PositionEncoding(Part):
-    """Describes how a mixer encodes positions; rotary kinds expose `inv_freq`."""
+    """How a mixer learns where its tokens are.  An attention mixer asks two things of it,
+    each of which may answer None ("not my way of encoding positions"):
+
+    `rotary(ctx)`: tables to rotate queries and keys with before the scores are taken.
+
+    `score_slopes(num_heads)`: a float32 tensor [num_heads] on the device; the score of
+    query head h at position p for the key at position j gets `slopes[h] * (j - p)` added
+    before the softmax (a penalty linear in the distance for positive slopes).
+
+    An encoding that acts elsewhere (learned positions added to the embedding, say) is an
+    `Embedding` part's business and answers None to both.
+    """
+
+    def rotary(self, ctx: "StepContext") -> RotaryTables | None:
+        return None
+
+    def score_slopes(self, num_heads: int) -> torch.Tensor | None:
+        return None
 
 
 class Mixer(Part):
@@ -177,7 +222,9 @@ class Mixer(Part):
 
     emit_partial_sums = False
 
-    def cache_needs(self) -> CacheNeeds:
+    def cache_needs(self, page_size: int) -> CacheNeeds:
+        """What the cache manager must keep for one call of this mixer, given its page size
+        (a mixer may choose its page layout by it)."""
         return CacheNeeds()
 
     def forward(
@@ -192,6 +239,26 @@ class FeedForward(Part):
     emit_partial_sums = False
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    """Starts the float32 residual stream of a step: `forward(ctx)` -> [T, hidden] float32
+    from `ctx.token_ids` (and, if it wishes, `ctx.positions`)."""
+
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """Ends a step: `forward(h, ctx)` takes the normalized rows [rows, hidden] in the compute
+    dtype and returns logits [rows, vocab] in float32.  `optional_names(prefix)` lists
+    tensors a checkpoint may hold without the head needing them."""
+
+    def optional_names(self, prefix: str) -> set[str]:
+        return set()
+
+    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
 
 

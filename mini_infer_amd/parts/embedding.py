@@ -4,6 +4,10 @@ Embedding: a row lookup that starts the float32 residual stream
 (models/llama/llama.py:159 of the reference).  Head: `logits = h @ W.T` on the
 requested rows only (llama.py:169-171); with tied embeddings the head's matrix is
 the embedding table and the checkpoint holds no `lm_head.weight` (llama.py:143-147).
+
+Both are chosen by kind like every other part, so a model whose stream starts or
+ends differently (a scaled embedding, learned positions added to it, capped logits)
+registers a part of its own and names it in its `ModelSpec`.
 """
 
 from __future__ import annotations
@@ -11,10 +15,11 @@ from __future__ import annotations
 import torch
 
 from mini_infer_amd import ops
-from mini_infer_amd.parts.base import ParamSpec, Part, TensorGetter
+from mini_infer_amd.parts.base import Embedding, Head, ParamSpec, StepContext, TensorGetter
+from mini_infer_amd.registry import register_embedding, register_head
 
 
-class TokenEmbedding(Part):
+class TokenEmbedding(Embedding):
     graph_safe = True
 
     def __init__(self, vocab_size: int, hidden_size: int, name: str, dtype: torch.dtype, device) -> None:
@@ -30,12 +35,12 @@ class TokenEmbedding(Part):
     def load_params(self, prefix: str, get: TensorGetter) -> None:
         self.weight = get(prefix + self.name).contiguous()
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, ctx: StepContext) -> torch.Tensor:
         assert self.weight is not None, "embedding used before its table was loaded"
-        return ops.embed_gather(self.weight, token_ids)
+        return ops.embed_gather(self.weight, ctx.token_ids)
 
 
-class OutputHead(Part):
+class OutputHead(Head):
     graph_safe = True
 
     def __init__(
@@ -74,6 +79,25 @@ class OutputHead(Part):
         assert w is not None, "output head used before its matrix was loaded"
         return w
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, ctx: StepContext | None = None) -> torch.Tensor:
         """Logits [rows, vocab] in float32."""
         return ops.linear(h, self.weight).float()
+
+
+@register_embedding("token_embedding")
+def build_token_embedding(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> TokenEmbedding:
+    return TokenEmbedding(int(desc["vocab_size"]), int(desc["hidden_size"]), str(desc["name"]), dtype, device)
+
+
+@register_head("linear_head")
+def build_linear_head(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> OutputHead:
+    """`desc["tied"]`: the head's matrix is the table of the model's embedding part (which the
+    model leaves under `shared["embedding"]` before it builds the head)."""
+    tied_to = None
+    if desc.get("tied", False):
+        tied_to = (shared or {}).get("embedding")
+        if tied_to is None or not hasattr(tied_to, "weight"):
+            raise ValueError("a tied output head needs the model's embedding part to hold a `weight` table")
+    return OutputHead(
+        int(desc["hidden_size"]), int(desc["vocab_size"]), str(desc["name"]), dtype, device, tied_to=tied_to
+    )

@@ -5,8 +5,8 @@ reference), optionally rescaled the llama3 way (rope.py:200-225).  The table
 stays float32 whatever the compute dtype (rope.py:368-390), and the angles
 `position * inv_freq` and their cos/sin are float32 too.
 
-A mixer asks this part for the cos/sin tables of a step; they are computed once
-per step and shared by all layers that use the same encoding.
+A mixer asks this part for the cos/sin tables of a step (`rotary(ctx)`); they are
+computed once per step and shared by all layers that use the same encoding.
 """
 
 from __future__ import annotations
@@ -16,7 +16,7 @@ import math
 import torch
 
 from mini_infer_amd import ops
-from mini_infer_amd.parts.base import PositionEncoding, StepContext
+from mini_infer_amd.parts.base import PositionEncoding, RotaryTables, StepContext
 from mini_infer_amd.registry import register_position_encoding
 
 
@@ -92,6 +92,10 @@ class RotaryPosition(PositionEncoding):
         if key not in ctx.shared:
             ctx.shared[key] = ops.rope_table(ctx.positions, self.inv_freq)
         return ctx.shared[key]
+
+    def rotary(self, ctx: StepContext) -> RotaryTables:
+        cos, sin = self.tables(ctx)
+        return RotaryTables(cos, sin, self.rotary_dim, self.interleaved)
 
 
 @register_position_encoding("rotary")

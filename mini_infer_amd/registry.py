@@ -59,12 +59,14 @@ def _load_builtins() -> None:
 
 # name in config.json's `architectures[0]` -> Architecture (models/architecture.py)
 ARCHITECTURES: Registry[Any] = Registry("architecture")
-# kind -> callable(description: dict, dtype, device) -> part
+# kind -> callable(description: dict, dtype, device, shared: dict | None) -> part
 MIXERS: Registry[Callable[..., Any]] = Registry("mixer")
 FEED_FORWARDS: Registry[Callable[..., Any]] = Registry("feed-forward")
 NORMS: Registry[Callable[..., Any]] = Registry("norm")
 POSITION_ENCODINGS: Registry[Callable[..., Any]] = Registry("position encoding")
 BLOCKS: Registry[Callable[..., Any]] = Registry("block arrangement")
+EMBEDDINGS: Registry[Callable[..., Any]] = Registry("embedding")
+HEADS: Registry[Callable[..., Any]] = Registry("output head")
 
 
 def _decorator(registry: Registry[Any], name: str) -> Callable[[T], T]:
@@ -97,3 +99,11 @@ def register_position_encoding(kind: str) -> Callable[[T], T]:
 
 def register_block(kind: str) -> Callable[[T], T]:
     return _decorator(BLOCKS, kind)
+
+
+def register_embedding(kind: str) -> Callable[[T], T]:
+    return _decorator(EMBEDDINGS, kind)
+
+
+def register_head(kind: str) -> Callable[[T], T]:
+    return _decorator(HEADS, kind)

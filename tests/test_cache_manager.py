@@ -228,3 +228,27 @@ def test_random_orders_lose_no_page(seed, window):
     assert all(m.num_free_pages(g.index) == 12 for g in m.groups)
     assert m.states.num_free == 4
     assert reused
+
+
+def test_keys_and_values_are_sized_apart_and_layout_is_what_the_mixer_declared():
+    needs = [
+        CacheNeeds(pages=PagedKVNeeds(2, 16, v_head_dim=40)),
+        CacheNeeds(pages=PagedKVNeeds(2, 16, v_head_dim=40)),
+        CacheNeeds(pages=PagedKVNeeds(2, 16, v_transposed=True)),
+        CacheNeeds(pages=PagedKVNeeds(1, 24, v_head_dim=0)),
+    ]
+    manager = CacheManager(needs, page_size=4, num_pages=6, max_requests=2, dtype=torch.float32, allocate_storage=True)
+    assert [g.calls for g in manager.groups] == [[0, 1], [2], [3]]
+    wide, transposed, single = manager.groups
+    assert wide.k_storage.shape == (2, 6, 2, 4 * 16) and wide.v_storage.shape == (2, 6, 2, 4 * 40)
+    assert single.v_storage is None
+    caches = manager.layer_caches()
+    assert caches[0].k_pages.shape == (6, 2, 4, 16) and caches[0].v_pages.shape == (6, 2, 4, 40)
+    assert caches[2].v_pages.shape == (6, 2, 16, 4) and caches[2].v_transposed and not caches[0].v_transposed
+    assert caches[3].k_pages.shape == (6, 1, 4, 24) and caches[3].v_pages is None
+    # views of one call do not overlap another call's
+    caches[0].v_pages.fill_(1.0)
+    assert caches[1].v_pages.abs().sum() == 0 and caches[0].k_pages.abs().sum() == 0
+    with pytest.raises(ValueError):
+        CacheManager([CacheNeeds(pages=PagedKVNeeds(0, 16))], page_size=4, num_pages=2, max_requests=1,
+                     allocate_storage=False)

@@ -131,7 +131,7 @@ def test_attention_part_in_two_portions(dtype, window):
             "head_dim": head_dim, "window": window,
             "position": {"kind": "rotary", "head_dim": head_dim, "theta": 100.0}}
     mixer = MIXERS.lookup("gqa_attention")(desc, TORCH[dtype], DEV, {})
-    needs = mixer.cache_needs()
+    needs = mixer.cache_needs(4)
     assert (needs.pages.num_kv_heads, needs.pages.head_dim, needs.pages.window) == (kv_heads, head_dim, window)
     rng = np.random.default_rng(1)
     w = {f"a.{n}_proj.weight": tiny.bf16_round(rng.standard_normal(s) / 6) for n, s in
@@ -490,9 +490,51 @@ def test_tokens_left_on_the_device_give_the_steps_of_tokens_from_the_host(tmp_pa
 
 
 def test_model_with_a_host_looping_part_is_not_graphed(tmp_path):
-    from mini_infer_amd.parts import Mixer
+    """A model holding a part that does not declare itself `graph_safe` (here a pass-through
+    feed-forward defined in the test) gets no decode graphs: its single-token steps run eagerly."""
+    import copy
+    import dataclasses
 
-    assert Mixer.graph_safe is False
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.models.spec import LayerSpec
+    from mini_infer_amd.parts import FeedForward
+    from mini_infer_amd.registry import ARCHITECTURES, FEED_FORWARDS
+
+    class Nothing(FeedForward):
+        def forward(self, x, ctx):
+            assert len(ctx.host_seq_lens) == ctx.num_requests  # the host lists a looping part would read
+            return torch.zeros_like(x)
+
+    FEED_FORWARDS.register("nothing", lambda desc, dtype_, device, shared=None: Nothing(dtype_, device))
+
+    def with_toy(spec):
+        layers = list(spec.layers)
+        block = copy.deepcopy(layers[1].block)
+        block["feed_forward"] = {"kind": "nothing"}
+        layers[1] = LayerSpec(layers[1].prefix, block)
+        return dataclasses.replace(spec, layers=layers)
+
+    _register_variant("NotGraphedTestLM", with_toy)
+    try:
+        cfg = dict(tiny.TINY_A, architectures=["NotGraphedTestLM"])
+        weights = tiny.make_weights(cfg, 59)
+        for n in ("gate", "up", "down"):
+            del weights[f"model.layers.1.mlp.{n}_proj.weight"]
+        folder = tiny.write_model_dir(tmp_path / "notgraphed", cfg, weights)
+        runner = ModelRunner.from_pretrained(folder, dtype="bfloat16", num_blocks=8, block_size=4)
+        assert not runner.model.graph_safe and runner.decode_graphs is None
+        runner.step([StepEntry("a", [1, 2, 3], [2])])
+        for token in (4, 5, 6):
+            assert runner.step([StepEntry("a", [token], [0])]).shape == (1, cfg["vocab_size"])
+        # the same folder's plain Llama sibling does record its decode steps
+        plain_cfg, _, _, plain_folder = _folder(tmp_path, "A", 59)
+        graphed = ModelRunner.from_pretrained(plain_folder, dtype="bfloat16", num_blocks=8, block_size=4)
+        graphed.step([StepEntry("a", [1, 2, 3], [2])])
+        graphed.step([StepEntry("a", [4], [0])])
+        assert graphed.decode_graphs is not None and graphed.decode_graphs.replays == 1
+    finally:
+        ARCHITECTURES.unregister("NotGraphedTestLM")
+        FEED_FORWARDS.unregister("nothing")
 
 
 def test_step_refuses_bad_batches(tmp_path):
@@ -624,7 +666,7 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path, dtype):
         def load_params(self, prefix, get):
             self.weight = get(prefix + "mix.weight")
 
-        def cache_needs(self):
+        def cache_needs(self, page_size):
             return CacheNeeds(state=StateNeeds((hidden,), torch.float32))
 
         def forward(self, x, ctx, cache, writes_cache=True):
@@ -809,23 +851,21 @@ def test_toy_position_encoding_registers_builds_and_steps(tmp_path, dtype):
 
     from mini_infer_amd.engine import ModelRunner
     from mini_infer_amd.models.spec import LayerSpec
-    from mini_infer_amd.parts import PositionEncoding
+    from mini_infer_amd.parts import PositionEncoding, RotaryTables
     from mini_infer_amd.registry import ARCHITECTURES, POSITION_ENCODINGS
 
     squeeze = 4.0
 
     class SqueezedRotary(PositionEncoding):
-        interleaved = False
-
         def __init__(self, desc, dtype_, device):
             super().__init__(dtype_, device)
             self.rotary_dim = int(desc["head_dim"])
             table = pl.inv_freq_default(self.rotary_dim, float(desc["theta"]))
             self.inv_freq = torch.from_numpy(table).to(device)
 
-        def tables(self, ctx):
+        def rotary(self, ctx):
             angle = (ctx.positions.float() / squeeze)[:, None] * self.inv_freq[None, :]
-            return torch.cos(angle).contiguous(), torch.sin(angle).contiguous()
+            return RotaryTables(torch.cos(angle).contiguous(), torch.sin(angle).contiguous(), self.rotary_dim, False)
 
     POSITION_ENCODINGS.register("squeezed_rotary", lambda desc, dtype_, device, shared=None: SqueezedRotary(desc, dtype_, device))
 
@@ -869,6 +909,273 @@ def test_toy_position_encoding_registers_builds_and_steps(tmp_path, dtype):
     finally:
         ARCHITECTURES.unregister("ToyPositionTestLM")
         POSITION_ENCODINGS.unregister("squeezed_rotary")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_distance_penalty_in_place_of_rotation_registers_builds_and_steps(tmp_path, dtype):
+    """A position encoding defined here that rotates nothing: it answers the attention part's
+    other question, with per-head slopes of a score penalty linear in the distance.  Layer 1
+    uses it (its values stay untransposed and the plain kernel runs, in bfloat16 too); layer 0
+    keeps its rotation, so the two layers live in page groups of their own."""
+    import copy
+    import dataclasses
+
+    from mini_infer_amd.engine import ModelRunner
+    from mini_infer_amd.models.spec import LayerSpec
+    from mini_infer_amd.parts import PositionEncoding
+    from mini_infer_amd.registry import ARCHITECTURES, POSITION_ENCODINGS
+
+    class DistancePenalty(PositionEncoding):
+        def score_slopes(self, num_heads):
+            return torch.tensor([0.5 ** (h + 1) for h in range(num_heads)], dtype=torch.float32, device=self.device)
+
+    POSITION_ENCODINGS.register("distance_penalty", lambda desc, dtype_, device, shared=None: DistancePenalty(dtype_, device))
+
+    def with_toy(spec):
+        layers = list(spec.layers)
+        block = copy.deepcopy(layers[1].block)
+        block["mixer"]["position"] = {"kind": "distance_penalty"}
+        layers[1] = LayerSpec(layers[1].prefix, block)
+        return dataclasses.replace(spec, layers=layers)
+
+    _register_variant("ToyPenaltyTestLM", with_toy)
+    try:
+        cfg = dict(tiny.TINY_B, architectures=["ToyPenaltyTestLM"], num_hidden_layers=2)
+        weights = tiny.make_weights(cfg, 65)
+        folder = tiny.write_model_dir(tmp_path / "penalty", cfg, weights)
+        heads, kv_heads, head_dim = 3, 1, 32
+
+        def penalized_attention(h, q_layer):
+            t = h.shape[0]
+            w = {n: weights[q_layer + f"self_attn.{n}_proj.weight"].astype(np.float64) for n in "qkvo"}
+            q = (h @ w["q"].T).reshape(t, heads, head_dim)
+            k = (h @ w["k"].T).reshape(t, kv_heads, head_dim)
+            v = (h @ w["v"].T).reshape(t, kv_heads, head_dim)
+            out = np.zeros((t, heads, head_dim))
+            for head in range(heads):
+                scores = q[:, head] @ k[:, 0].T / math.sqrt(head_dim)
+                distance = np.arange(t)[None, :] - np.arange(t)[:, None]  # j - p
+                scores = scores + 0.5 ** (head + 1) * distance
+                scores = np.where(distance > 0, -np.inf, scores)
+                probs = np.exp(scores - scores.max(axis=-1, keepdims=True))
+                out[:, head] = (probs / probs.sum(axis=-1, keepdims=True)) @ v[:, 0]
+            return out.reshape(t, heads * head_dim) @ w["o"].T
+
+        def plain(tokens):
+            eps = cfg["rms_norm_eps"]
+            r = pl.embedding(weights["model.embed_tokens.weight"], np.array(tokens))
+            cos, sin = pl.rope_tables(np.arange(len(tokens)), pl.config_inv_freq(cfg))
+            for layer in range(2):
+                q = f"model.layers.{layer}."
+                h = pl.rms_norm(r, weights[q + "input_layernorm.weight"], eps)
+                if layer == 0:
+                    a, _ = pl.attention_layer(h, *(weights[q + f"self_attn.{n}_proj.weight"] for n in "qkvo"),
+                                              cos, sin, heads, kv_heads, head_dim)
+                else:
+                    a = penalized_attention(h, q)
+                r = r + a
+                r = r + pl.swiglu(pl.rms_norm(r, weights[q + "post_attention_layernorm.weight"], eps),
+                                  *(weights[q + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            return pl.rms_norm(r, weights["model.norm.weight"], eps) @ weights["lm_head.weight"].astype(np.float64).T
+
+        requests = {f"d{i}": tiny.random_tokens(cfg, n, seed=30 + i) for i, n in enumerate((70, 9, 33))}
+        expected = {rid: plain(t) for rid, t in requests.items()}
+        # the penalty matters: without it (and without rotation) layer 1 gives other logits
+        runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=24, block_size=16, max_concurrent=3)
+        groups = runner.cache.groups
+        if dtype == "bfloat16":
+            assert [g.v_transposed for g in groups] == [True, False] and [g.calls for g in groups] == [[0], [1]]
+        else:
+            assert len(groups) == 1 and not groups[0].v_transposed
+        got = ru.run_schedule(runner, requests, ru.schedule_mixed(requests, seed=7, tail=5))
+        for rid in requests:
+            ru.assert_close(got[rid], expected[rid], dtype, f"penalty {rid}")
+        runner.cache.check()
+    finally:
+        ARCHITECTURES.unregister("ToyPenaltyTestLM")
+        POSITION_ENCODINGS.unregister("distance_penalty")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_with_keys_and_values_of_different_widths(tmp_path, dtype):
+    """A paged mixer defined here keeps narrow keys (8 per token) and wide values (24): it
+    declares both widths, the cache manager sizes the two streams apart and hands the
+    mixer pages of each, and the mixer reads and writes them through the step's block
+    tables and write slots.  No framework file knows it."""
+    import copy
+    import dataclasses
+
+    from mini_infer_amd.engine import ModelRunner
+    from mini_infer_amd.models.spec import LayerSpec
+    from mini_infer_amd.parts import CacheNeeds, Mixer, PagedKVNeeds, ParamSpec
+    from mini_infer_amd.registry import ARCHITECTURES, MIXERS
+
+    hidden, k_dim, v_dim = tiny.TINY_A["hidden_size"], 8, 24
+
+    class NarrowKeysWideValues(Mixer):
+        def param_specs(self, prefix):
+            return {prefix + "k.weight": ParamSpec((k_dim, hidden)), prefix + "q.weight": ParamSpec((k_dim, hidden)),
+                    prefix + "v.weight": ParamSpec((v_dim, hidden)), prefix + "o.weight": ParamSpec((hidden, v_dim))}
+
+        def load_params(self, prefix, get):
+            self.w = {n: get(prefix + n + ".weight").float() for n in "qkvo"}
+
+        def cache_needs(self, page_size):
+            return CacheNeeds(pages=PagedKVNeeds(1, k_dim, v_head_dim=v_dim))
+
+        def forward(self, x, ctx, cache, writes_cache=True):
+            page = ctx.page_size
+            assert cache.k_pages.shape[1:] == (1, page, k_dim) and cache.v_pages.shape[1:] == (1, page, v_dim)
+            xf = x.float()
+            q, k, v = xf @ self.w["q"].T, xf @ self.w["k"].T, xf @ self.w["v"].T
+            slots = ctx.slot_mapping[cache.group].long()
+            cache.k_pages[slots // page, 0, slots % page] = k.to(x.dtype)
+            cache.v_pages[slots // page, 0, slots % page] = v.to(x.dtype)
+            out = torch.empty((x.shape[0], v_dim), dtype=torch.float32, device=x.device)
+            table = ctx.block_tables[cache.group]
+            for b in range(ctx.num_requests):
+                first, last = ctx.host_cu_seqlens_q[b], ctx.host_cu_seqlens_q[b + 1]
+                length = ctx.host_seq_lens[b]
+                pages = table[b, : -(-length // page)].long()
+                keys = cache.k_pages[pages, 0].reshape(-1, k_dim)[:length].float()
+                values = cache.v_pages[pages, 0].reshape(-1, v_dim)[:length].float()
+                scores = q[first:last] @ keys.T
+                positions = ctx.positions[first:last].long()
+                hidden_keys = torch.arange(length, device=x.device)[None, :] > positions[:, None]
+                out[first:last] = torch.softmax(scores.masked_fill(hidden_keys, float("-inf")), dim=-1) @ values
+            return (out @ self.w["o"].T).to(x.dtype)
+
+    MIXERS.register("narrow_keys_wide_values", lambda desc, dtype_, device, shared=None: NarrowKeysWideValues(dtype_, device))
+
+    def with_toy(spec):
+        layers = list(spec.layers)
+        block = copy.deepcopy(layers[0].block)
+        block["mixer"] = {"kind": "narrow_keys_wide_values"}
+        layers[0] = LayerSpec(layers[0].prefix, block)
+        return dataclasses.replace(spec, layers=layers)
+
+    _register_variant("ToyWidthsTestLM", with_toy)
+    try:
+        cfg = dict(tiny.TINY_A, architectures=["ToyWidthsTestLM"])
+        weights = tiny.make_weights(cfg, 66)
+        for n in "qkvo":
+            del weights[f"model.layers.0.self_attn.{n}_proj.weight"]
+        rng = np.random.default_rng(8)
+        p = "model.layers.0.self_attn."
+        for n, shape in (("q", (k_dim, hidden)), ("k", (k_dim, hidden)), ("v", (v_dim, hidden)), ("o", (hidden, v_dim))):
+            weights[p + n + ".weight"] = tiny.bf16_round(rng.standard_normal(shape) / math.sqrt(shape[1]))
+        folder = tiny.write_model_dir(tmp_path / "widths", cfg, weights)
+        rounded = (lambda a: tiny.bf16_round(a).astype(np.float64)) if dtype == "bfloat16" else (lambda a: a)
+
+        def plain(tokens):
+            eps = cfg["rms_norm_eps"]
+            t = len(tokens)
+            r = pl.embedding(weights["model.embed_tokens.weight"], np.array(tokens))
+            h = rounded(pl.rms_norm(r, weights["model.layers.0.input_layernorm.weight"], eps))
+            w = {n: weights[p + n + ".weight"].astype(np.float64) for n in "qkvo"}
+            q, k, v = h @ w["q"].T, rounded(h @ w["k"].T), rounded(h @ w["v"].T)
+            scores = np.where(np.arange(t)[None, :] > np.arange(t)[:, None], -np.inf, q @ k.T)
+            probs = np.exp(scores - scores.max(axis=-1, keepdims=True))
+            r = r + rounded(((probs / probs.sum(axis=-1, keepdims=True)) @ v) @ w["o"].T)
+            q0 = "model.layers.0."
+            r = r + pl.swiglu(pl.rms_norm(r, weights[q0 + "post_attention_layernorm.weight"], eps),
+                              *(weights[q0 + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            q1 = "model.layers.1."
+            cos, sin = pl.rope_tables(np.arange(t), pl.config_inv_freq(cfg))
+            a, _ = pl.attention_layer(pl.rms_norm(r, weights[q1 + "input_layernorm.weight"], eps),
+                                      *(weights[q1 + f"self_attn.{n}_proj.weight"] for n in "qkvo"), cos, sin, 4, 2, 16)
+            r = r + a
+            r = r + pl.swiglu(pl.rms_norm(r, weights[q1 + "post_attention_layernorm.weight"], eps),
+                              *(weights[q1 + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            return pl.rms_norm(r, weights["model.norm.weight"], eps) @ weights["model.embed_tokens.weight"].astype(np.float64).T
+
+        requests = {f"w{i}": tiny.random_tokens(cfg, n, seed=40 + i) for i, n in enumerate((19, 8, 27, 12))}
+        expected = {rid: plain(t) for rid, t in requests.items()}
+        runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=20, block_size=4, max_concurrent=4)
+        groups = runner.cache.groups
+        assert [(g.head_dim, g.value_dim) for g in groups] == [(k_dim, v_dim), (16, 16)]
+        assert groups[0].k_storage.shape[-1] == 4 * k_dim and groups[0].v_storage.shape[-1] == 4 * v_dim
+        got = ru.run_schedule(runner, requests, ru.schedule_mixed(requests, seed=8, tail=4))
+        for rid in requests:
+            ru.assert_close(got[rid], expected[rid], dtype, f"widths {rid}")
+        runner.cache.check()
+        assert all(g.pool.num_free == 20 for g in groups)
+    finally:
+        ARCHITECTURES.unregister("ToyWidthsTestLM")
+        MIXERS.unregister("narrow_keys_wide_values")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_embedding_and_head_register_and_take_the_places_of_the_built_in_ones(tmp_path, dtype):
+    """How the residual stream starts and ends is a part like any other: an embedding defined
+    here adds a learned row per position to the token's row, and a head defined here caps the
+    logits with a tanh.  The model's spec names them by kind; no framework file changes."""
+    import dataclasses
+
+    from mini_infer_amd import ops
+    from mini_infer_amd.engine import ModelRunner
+    from mini_infer_amd.parts import Embedding, Head, ParamSpec
+    from mini_infer_amd.registry import ARCHITECTURES, EMBEDDINGS, HEADS
+
+    cfg = dict(tiny.TINY_A, architectures=["ToyEndsTestLM"], max_position_embeddings=64)
+    hidden, vocab, cap = cfg["hidden_size"], cfg["vocab_size"], 100.0
+
+    class TokensPlusPositions(Embedding):
+        def param_specs(self, prefix):
+            return {"model.embed_tokens.weight": ParamSpec((vocab, hidden)),
+                    "model.embed_positions.weight": ParamSpec((64, hidden))}
+
+        def load_params(self, prefix, get):
+            self.weight = get("model.embed_tokens.weight").contiguous()
+            self.rows = get("model.embed_positions.weight").contiguous()
+
+        def forward(self, ctx):
+            return ops.embed_gather(self.weight, ctx.token_ids) + ops.embed_gather(self.rows, ctx.positions)
+
+    class CappedHead(Head):
+        def __init__(self, dtype_, device, embedding):
+            super().__init__(dtype_, device)
+            self.embedding = embedding
+
+        def forward(self, h, ctx):
+            return cap * torch.tanh(ops.linear(h, self.embedding.weight).float() / cap)
+
+    EMBEDDINGS.register("tokens_plus_positions", lambda desc, dtype_, device, shared=None: TokensPlusPositions(dtype_, device))
+    HEADS.register("capped_head", lambda desc, dtype_, device, shared=None: CappedHead(dtype_, device, shared["embedding"]))
+    _register_variant("ToyEndsTestLM", lambda spec: dataclasses.replace(
+        spec, embedding={"kind": "tokens_plus_positions"}, head={"kind": "capped_head"}))
+    try:
+        weights = tiny.make_weights(cfg, 67)
+        weights["model.embed_positions.weight"] = tiny.bf16_round(np.random.default_rng(9).standard_normal((64, hidden)))
+        folder = tiny.write_model_dir(tmp_path / "ends", cfg, weights)
+
+        def plain(tokens):
+            eps = cfg["rms_norm_eps"]
+            r = pl.embedding(weights["model.embed_tokens.weight"], np.array(tokens))
+            r = r + weights["model.embed_positions.weight"][: len(tokens)].astype(np.float64)
+            cos, sin = pl.rope_tables(np.arange(len(tokens)), pl.config_inv_freq(cfg))
+            for layer in range(2):
+                q = f"model.layers.{layer}."
+                a, _ = pl.attention_layer(
+                    pl.rms_norm(r, weights[q + "input_layernorm.weight"], eps),
+                    *(weights[q + f"self_attn.{n}_proj.weight"] for n in "qkvo"), cos, sin, 4, 2, 16)
+                r = r + a
+                r = r + pl.swiglu(pl.rms_norm(r, weights[q + "post_attention_layernorm.weight"], eps),
+                                  *(weights[q + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            logits = pl.rms_norm(r, weights["model.norm.weight"], eps) @ weights["model.embed_tokens.weight"].astype(np.float64).T
+            return cap * np.tanh(logits / cap)
+
+        requests = {f"e{i}": tiny.random_tokens(cfg, n, seed=50 + i) for i, n in enumerate((21, 5, 14))}
+        expected = {rid: plain(t) for rid, t in requests.items()}
+        assert np.abs(expected["e0"] - pl.llama_logits(cfg, weights, np.array(requests["e0"]))).max() > 1e-1
+        runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=24, block_size=4, max_concurrent=3)
+        got = ru.run_schedule(runner, requests, ru.schedule_mixed(requests, seed=9, tail=5))
+        for rid in requests:
+            ru.assert_close(got[rid], expected[rid], dtype, f"ends {rid}")
+    finally:
+        ARCHITECTURES.unregister("ToyEndsTestLM")
+        EMBEDDINGS.unregister("tokens_plus_positions")
+        HEADS.unregister("capped_head")
 
 
 _LONG = {}

@@ -313,3 +313,60 @@ def test_trace_out_holds_one_event_per_step_with_its_kind_and_sizes(tmp_path):
     assert events[-1]["args"]["phase"] == "decode"
     assert all(e["ph"] == "X" and e["name"] == "step" and e["dur"] >= 0 for e in events)
     assert events[0]["ts"] == 0 and all(a["ts"] <= b["ts"] for a, b in zip(events, events[1:]))
+
+
+# -- a step that fails leaves the cache as it was ------------------------------------------------
+
+
+class _FailingModel:
+    """Stands where a `DecoderModel` stands in a `ModelRunner`: logits of zeros, or an error on demand."""
+
+    graph_safe = False
+    dtype = torch.float32
+    device = torch.device("cpu")
+
+    class spec:  # noqa: N801 - attribute-compatible with ModelSpec
+        vocab_size = VOCAB
+
+    def __init__(self):
+        self.fail_with = None
+        self.positions_seen = []
+
+    def cache_needs(self, page_size):
+        return [CacheNeeds(pages=PagedKVNeeds(1, 16))]
+
+    def forward(self, ctx, caches):
+        if self.fail_with is not None:
+            raise self.fail_with
+        self.positions_seen.append(ctx.positions.tolist())
+        return torch.zeros((ctx.logit_rows.numel(), VOCAB))
+
+
+def test_a_step_that_raises_leaves_lengths_pages_and_admissions_as_they_were():
+    from mini_infer_amd.engine.batch import StepEntry
+    from mini_infer_amd.engine.model_runner import ModelRunner
+    from mini_infer_amd.exceptions import KernelShapeError
+
+    model = _FailingModel()
+    runner = ModelRunner(model, None, num_blocks=8, block_size=4, max_concurrent=3, cuda_graph=False)
+    runner.step([StepEntry("old", [1, 2, 3, 4, 5, 6], [5])])
+    free_before = runner.num_free_blocks()
+    assert free_before == 8 - 2 and runner.cache.length("old") == 6
+
+    model.fail_with = KernelShapeError("a kernel refuses this size")
+    with pytest.raises(KernelShapeError):
+        # "old" would grow into a third page, "new" would be admitted with two pages
+        runner.step([StepEntry("old", [7, 8, 9], [2]), StepEntry("new", [1, 2, 3, 4, 5], [4])])
+    runner.cache.check()
+    assert runner.num_free_blocks() == free_before
+    assert runner.cache.length("old") == 6 and not runner.has_request("new")
+    assert runner.cache.states.num_free == 2
+
+    model.fail_with = None
+    runner.step([StepEntry("old", [7, 8, 9], [2]), StepEntry("new", [1, 2, 3], [2])])
+    assert model.positions_seen[-1] == [6, 7, 8, 0, 1, 2]
+    assert runner.cache.length("old") == 9 and runner.cache.length("new") == 3
+    runner.cache.check()
+    runner.free_request("old")
+    runner.free_request("new")
+    assert runner.num_free_blocks() == 8
