@@ -15,8 +15,11 @@
 // [num_pages][kv_heads][page_size][head_dim]; block_table[request][i] is the page
 // of that request's keys i*page_size .. (i+1)*page_size-1.
 #include "common.h"
+#include "entry_points.h"
 
 #include <math.h>
+
+#include <mutex>
 
 #define GT 4  // query heads handled together by one wave
 
@@ -327,4 +330,81 @@ extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, 
                                                             num_splits);
   MI_CHECK_LAUNCH("attn_reduce");
   return MI_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// The same attention for callers that cannot allocate: the partial results of the key
+// ranges lie in an array of the library's own.
+//
+// `scratch` below is, in host code, only a stand-in for the device symbol: its device
+// address differs per GPU and is asked for once per device with hipGetSymbolAddress;
+// host code passes that address, never the array's name, to kernels.
+
+#define MI_MAX_DEVICES 64
+
+static __device__ __align__(256) unsigned char scratch[MI_ATTN_STATIC_SCRATCH_BYTES];
+
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[MI_MAX_DEVICES] = {};
+
+// The address of this device's copy of `scratch` (asked for at the first call on the device).
+static int scratch_of_current_device(float** ptr) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess || device < 0 || device >= MI_MAX_DEVICES) {
+    mi_set_error("attn_generic_static: cannot tell the current device (%s, device %d)",
+                 hipGetErrorString(err), device);
+    return MI_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* address = nullptr;
+    err = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || address == nullptr) {
+      mi_set_error("attn_generic_static: hipGetSymbolAddress failed on device %d: %s", device,
+                   hipGetErrorString(err));
+      return MI_ERR_LAUNCH;
+    }
+    g_scratch_ptr[device] = address;
+  }
+  *ptr = (float*)g_scratch_ptr[device];
+  return MI_OK;
+}
+
+extern "C" int mi_attn_generic_static(int dtype, const void* q, int64_t q_row_stride, const void* k_pages,
+                                      const void* v_pages, const int* block_table, int max_blocks,
+                                      const int* token_request, const int* positions, void* out,
+                                      int64_t out_row_stride, int num_tokens, int q_heads, int kv_heads,
+                                      int head_dim, int page_size, int num_pages, float scale, int window,
+                                      int num_splits, const float* slopes, hipStream_t stream) {
+  const int bad = attn_generic_check(dtype, q_row_stride, max_blocks, out_row_stride, num_tokens, q_heads,
+                                     kv_heads, head_dim, page_size, num_pages, window, num_splits);
+  if (bad != MI_OK) return bad;
+  if (num_tokens == 0) return MI_OK;
+  const int64_t slots = (int64_t)num_tokens * q_heads * num_splits;
+  const int64_t bytes = slots * (head_dim + 2) * (int64_t)sizeof(float);
+  if (num_splits > 1 && bytes > (int64_t)MI_ATTN_STATIC_SCRATCH_BYTES) {
+    mi_set_error("attn_generic_static: %d tokens x %d heads x %d key ranges x head_dim %d need %lld bytes "
+                 "of partial results, the library's array holds %u",
+                 num_tokens, q_heads, num_splits, head_dim, (long long)bytes, MI_ATTN_STATIC_SCRATCH_BYTES);
+    return MI_ERR_LIMIT;
+  }
+  float* part_acc = nullptr;
+  float* part_ml = nullptr;
+  if (num_splits > 1) {
+    float* base = nullptr;
+    const int status = scratch_of_current_device(&base);
+    if (status != MI_OK) return status;
+    part_acc = base;                     // [slots][head_dim]
+    part_ml = base + slots * head_dim;  // [slots][2]
+  }
+  if (dtype == MI_F32)
+    return attn_generic_launch<float>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
+                                      token_request, positions, out, out_row_stride, part_acc, part_ml,
+                                      num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
+                                      num_splits, slopes, stream);
+  return attn_generic_launch<bf16_t>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
+                                     token_request, positions, out, out_row_stride, part_acc, part_ml,
+                                     num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
+                                     num_splits, slopes, stream);
 }
