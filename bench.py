@@ -255,7 +255,7 @@ def main() -> int:
     import torch
 
     from mini_infer_amd.engine import ModelRunner, StepEntry
-    from mini_infer_amd.sampling import SamplingParams, sample_tokens
+    from mini_infer_amd.sampling import sample_from_slots
 
     model_name, sizes = SIZES[args.sizes]
     full_layers = sizes["num_hidden_layers"]
@@ -275,7 +275,11 @@ def main() -> int:
         max_concurrent=max(batches),
     )
     rng = np.random.default_rng(0)
-    greedy = SamplingParams()
+
+    def sample(logits) -> torch.Tensor:
+        """The greedy choice of every row on the device: each request's sampling state (greedy
+        by default) is read from its state slot, as the scheduler's sampling does."""
+        return sample_from_slots(logits, runner.last_row_slots, runner.cache.states.table)
 
     def sync() -> None:
         torch.cuda.synchronize()
@@ -290,8 +294,7 @@ def main() -> int:
         for rid in ids:
             prompt = rng.integers(0, cfg["vocab_size"], size=PROMPT_LEN).tolist()
             logits = prefill(rid, prompt)
-            last.append(int(sample_tokens(logits, [greedy], [0], [0]).tolist()[0]))
-        params, seeds = [greedy] * batch, [0] * batch
+            last.append(int(sample(logits).tolist()[0]))
         host_ids = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         copied = [torch.cuda.Event(), torch.cuda.Event()]
 
@@ -304,7 +307,7 @@ def main() -> int:
             else:
                 entries = [StepEntry(rid, [0], [0], device_row=row) for row, rid in enumerate(ids)]
             logits = runner.step(entries, device_tokens=ids_on_device)
-            sampled = sample_tokens(logits, params, seeds, [draw] * batch)
+            sampled = sample(logits)
             host_ids[draw % 2].copy_(sampled, non_blocking=True)
             copied[draw % 2].record()
             return sampled

@@ -4,6 +4,8 @@
   random-weights  write a model folder (config.json + model.safetensors) from a
                   config.json and a seed
   replay          the trace replay tool (same as bin/trace_run)
+  make-trace      print a trace for it: random token ids cut into steps by one of the
+                  schedule families (whole, decode, portions, mixed)
 
 Engine options carry the reference's constructor names (engine/model_runner.py:84-100,
 scheduler/continuous_scheduler.py:168-177): --num-blocks, --block-size,
@@ -18,18 +20,19 @@ import argparse
 import json
 import sys
 
-from mini_infer_amd.config import DEFAULT_BLOCK_SIZE, DEFAULT_NUM_BLOCKS
+from mini_infer_amd.config import EngineConfig
 
 
 def _add_engine_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--device", default="cuda:0")
-    parser.add_argument("--num-blocks", type=int, default=DEFAULT_NUM_BLOCKS)
-    parser.add_argument("--block-size", type=int, default=DEFAULT_BLOCK_SIZE)
-    parser.add_argument("--max-concurrent", type=int, default=16)
-    parser.add_argument("--max-num-batched-tokens", type=int, default=2048)
-    parser.add_argument("--chunk-size", type=int, default=256)
-    parser.add_argument("--decode-headroom-blocks", type=int, default=8)
+    defaults = EngineConfig()
+    parser.add_argument("--num-blocks", type=int, default=defaults.num_blocks)
+    parser.add_argument("--block-size", type=int, default=defaults.block_size)
+    parser.add_argument("--max-concurrent", type=int, default=defaults.max_concurrent)
+    parser.add_argument("--max-num-batched-tokens", type=int, default=defaults.max_num_batched_tokens)
+    parser.add_argument("--chunk-size", type=int, default=defaults.chunk_size)
+    parser.add_argument("--decode-headroom-blocks", type=int, default=defaults.decode_headroom_blocks)
     parser.add_argument("--trace-out", default=None, help="write a Chrome trace of the steps to this file")
 
 
@@ -44,8 +47,9 @@ def _generate(args: argparse.Namespace) -> int:
         prompts.append([int(t) for t in ids.replace(",", " ").split()])
     if not prompts:
         raise SystemExit("give --prompt TEXT or --prompt-ids '1 2 3' (either may repeat)")
-    llm = LLM(
-        args.model,
+    from mini_infer_amd.config import EngineConfig
+
+    engine = EngineConfig(
         dtype=args.dtype,
         device=args.device,
         num_blocks=args.num_blocks,
@@ -57,6 +61,7 @@ def _generate(args: argparse.Namespace) -> int:
         seed=args.seed,
         trace_out=args.trace_out,
     )
+    llm = LLM(args.model, engine=engine)
     params = SamplingParams(
         temperature=args.temperature,
         top_k=args.top_k,
@@ -102,6 +107,25 @@ def _replay(args: argparse.Namespace) -> int:
     return replay.run(args)
 
 
+def _make_trace(args: argparse.Namespace) -> int:
+    import numpy as np
+
+    from mini_infer_amd.engine import trace
+
+    rng = np.random.default_rng(args.seed)
+    lengths = [int(n) for n in args.lengths.replace(",", " ").split()]
+    requests = {f"r{i}": rng.integers(0, args.vocab_size, size=n).tolist() for i, n in enumerate(lengths)}
+    schedule = trace.make_schedule(args.family, requests, seed=args.seed, tail=args.tail)
+    for line in trace.to_trace_lines(requests, schedule):
+        print(line)
+    print(
+        f"{len(schedule)} steps, at most {trace.peak_pages(requests, schedule, 64) * 64} tokens live "
+        f"(each request rounded up to 64)",
+        file=sys.stderr,
+    )
+    return 0
+
+
 def main(argv: list[str] | None = None) -> int:
     parser = argparse.ArgumentParser(prog="python -m mini_infer_amd", description=__doc__.split("\n\n")[0])
     commands = parser.add_subparsers(dest="command", required=True)
@@ -132,6 +156,16 @@ def main(argv: list[str] | None = None) -> int:
 
     rep = commands.add_parser("replay", parents=[replay_parser()], add_help=False, help="trace replay")
     rep.set_defaults(run=_replay)
+
+    from mini_infer_amd.engine.trace import FAMILIES
+
+    mk = commands.add_parser("make-trace", help="print a replay trace of random token ids")
+    mk.add_argument("--family", choices=FAMILIES, default="mixed")
+    mk.add_argument("--lengths", required=True, help="request lengths, e.g. '150,40,97,1'")
+    mk.add_argument("--vocab-size", type=int, required=True)
+    mk.add_argument("--seed", type=int, default=0)
+    mk.add_argument("--tail", type=int, default=32, help="tokens at the end of a request fed one by one")
+    mk.set_defaults(run=_make_trace)
 
     args = parser.parse_args(argv)
     return args.run(args)

@@ -159,6 +159,12 @@ class CacheManager:
     def state_slot(self, request_id: Hashable) -> int:
         return self._slots[request_id]
 
+    def set_sampling(self, request_id: Hashable, *, temperature: float, top_k: int, top_p: float,
+                     seed: int, draw: int = 0) -> None:
+        """Write the request's sampling state into its slot (see `StateSlots.set_sampling`)."""
+        self.states.set_sampling(self._slots[request_id], temperature=temperature, top_k=top_k, top_p=top_p,
+                                 seed=seed, draw=draw)
+
     def live_requests(self) -> list[Hashable]:
         return list(self._lengths)
 
@@ -215,12 +221,15 @@ class CacheManager:
                     page = table.pop()
                     if page != RELEASED:
                         group.pool.free(page)
+            # the step's first kernel may already have written the new position on the device
+            self.states.push(self._slots[request_id])
 
     def commit(self, extents: dict[Hashable, int]) -> None:
         """Advance lengths after a step and give back what windows have passed."""
         for request_id, new_tokens in extents.items():
             length = self._lengths[request_id] + new_tokens
             self._lengths[request_id] = length
+            self.states.set_position(self._slots[request_id], length)
             for group in self.groups:
                 if group.window is None:
                     continue
@@ -250,6 +259,8 @@ class CacheManager:
                 if page != RELEASED:
                     group.pool.free(page)
         self._lengths[request_id] = length
+        self.states.set_position(self._slots[request_id], length)
+        self.states.push(self._slots[request_id])
 
     # -- per-step index -------------------------------------------------------
 

@@ -1,19 +1,47 @@
 """Slots for per-request state of fixed size.
 
-Beside the paged keys and values, a request owns one row in each state tensor
-for as long as it lives: `[max_requests, *shape]` per layer call that asked for
-state.  A row is zeroed when it is handed out.  The reference keeps such state
-in a separate cache family (cache/state_cache.py:130-333); here it lives next to
-the pages so one manager admits and frees a request as a whole.  Llama needs no
-state tensors; the slot itself (the row index) still exists for every request.
+Beside the paged keys and values, a request owns one slot for as long as it lives.
+The reference keeps such state in a separate cache family
+(cache/state_cache.py:130-333); here it lives next to the pages so one manager
+admits and frees a request as a whole.  A slot is
+
+  * one row of the *slot table*, `[max_requests, 8]` int32 on the device with a copy
+    on the host: the request's position (tokens in the cache) and the state of its
+    sampling (seed, index of the next draw, temperature, top-k, top-p).  Kernels
+    read a request's row by its slot id: the sampling kernel takes its settings
+    from there and advances the draw index itself, the first kernel of a step
+    writes the positions.  The host copy is what the scheduler plans with; both
+    are advanced by the same events, so they agree whenever the device is idle;
+  * one row in each state tensor a mixer asked for, `[max_requests, *shape]` per
+    layer call, zeroed when the slot is handed out (Llama asks for none).
 """
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from mini_infer_amd.exceptions import OutOfMemoryError
 from mini_infer_amd.parts.base import StateNeeds
+
+# int32 words of a slot-table row (the layout the kernels read)
+SLOT_WORDS = 8
+SLOT_POSITION = 0
+SLOT_SEED_LO = 1
+SLOT_SEED_HI = 2
+SLOT_DRAW = 3
+SLOT_TEMPERATURE = 4  # float32 bits
+SLOT_TOP_K = 5
+SLOT_TOP_P = 6  # float32 bits
+
+
+def _float_bits(value: float) -> int:
+    return int(np.array([value], dtype=np.float32).view(np.int32)[0])
+
+
+def _as_i32(value: int) -> int:
+    """The int32 holding the unsigned 32-bit pattern `value`."""
+    return int(np.array([value & 0xFFFFFFFF], dtype=np.uint32).view(np.int32)[0])
 
 
 class StateSlots:
@@ -30,7 +58,10 @@ class StateSlots:
         self._free: list[int] = list(range(max_requests - 1, -1, -1))
         self._owner: list[object | None] = [None] * max_requests
         self.tensors: dict[int, torch.Tensor] = {}
+        self.host = np.zeros((max_requests, SLOT_WORDS), dtype=np.int32)
+        self.table: torch.Tensor | None = None
         if allocate_storage:
+            self.table = torch.zeros((max_requests, SLOT_WORDS), dtype=torch.int32, device=device)
             for call, need in needs.items():
                 self.tensors[call] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
 
@@ -39,10 +70,14 @@ class StateSlots:
         return len(self._free)
 
     def allocate(self, owner: object) -> int:
+        """A free slot, its table row and state rows zeroed: position 0, draw 0, greedy."""
         if not self._free:
             raise OutOfMemoryError(f"all {self.max_requests} request slots are in use")
         slot = self._free.pop()
         self._owner[slot] = owner
+        self.host[slot] = 0
+        self.host[slot, SLOT_TOP_P] = _float_bits(1.0)
+        self.push(slot)
         for tensor in self.tensors.values():
             tensor[slot].zero_()
         return slot
@@ -57,6 +92,49 @@ class StateSlots:
 
     def owner(self, slot: int) -> object | None:
         return self._owner[slot]
+
+    # -- the slot table -----------------------------------------------------------
+
+    def push(self, slot: int) -> None:
+        """Send the host's copy of a row to the device (ordered after the work already queued)."""
+        if self.table is not None:
+            self.table[slot].copy_(torch.from_numpy(self.host[slot].copy()))
+
+    def set_sampling(
+        self, slot: int, *, temperature: float, top_k: int, top_p: float, seed: int, draw: int = 0
+    ) -> None:
+        """The sampling state of the request in `slot`: its settings, its seed (64 unsigned
+        bits) and the index of its next draw (0 for a new request, the number of tokens it
+        already drew when it is admitted again after a preemption)."""
+        row = self.host[slot]
+        row[SLOT_SEED_LO] = _as_i32(seed)
+        row[SLOT_SEED_HI] = _as_i32(seed >> 32)
+        row[SLOT_DRAW] = _as_i32(draw)
+        row[SLOT_TEMPERATURE] = _float_bits(temperature)
+        row[SLOT_TOP_K] = int(top_k)
+        row[SLOT_TOP_P] = _float_bits(top_p)
+        self.push(slot)
+
+    def set_position(self, slot: int, position: int) -> None:
+        """Host copy only: on the device the first kernel of the step writes the same value."""
+        self.host[slot, SLOT_POSITION] = position
+
+    def count_draw(self, slot: int) -> None:
+        """Host copy only: the sampling kernel advances the device's copy itself."""
+        self.host[slot, SLOT_DRAW] = _as_i32(int(self.host[slot, SLOT_DRAW]) + 1)
+
+    def position(self, slot: int) -> int:
+        return int(self.host[slot, SLOT_POSITION])
+
+    def draws(self, slot: int) -> int:
+        return int(self.host[slot, SLOT_DRAW]) & 0xFFFFFFFF
+
+    def seed(self, slot: int) -> int:
+        lo = int(self.host[slot, SLOT_SEED_LO]) & 0xFFFFFFFF
+        hi = int(self.host[slot, SLOT_SEED_HI]) & 0xFFFFFFFF
+        return (hi << 32) | lo
+
+    # -- checks ---------------------------------------------------------------------
 
     def check(self) -> None:
         if len(set(self._free)) != len(self._free):

@@ -1,5 +1,9 @@
 from mini_infer_amd.config.engine_config import (
     DEFAULT_BLOCK_SIZE,
+    DEFAULT_CHUNK_SIZE,
+    DEFAULT_DECODE_HEADROOM_BLOCKS,
+    DEFAULT_MAX_CONCURRENT,
+    DEFAULT_MAX_NUM_BATCHED_TOKENS,
     DEFAULT_NUM_BLOCKS,
     EngineConfig,
 )
@@ -12,6 +16,10 @@ from mini_infer_amd.config.model_config import (
 
 __all__ = [
     "DEFAULT_BLOCK_SIZE",
+    "DEFAULT_CHUNK_SIZE",
+    "DEFAULT_DECODE_HEADROOM_BLOCKS",
+    "DEFAULT_MAX_CONCURRENT",
+    "DEFAULT_MAX_NUM_BATCHED_TOKENS",
     "DEFAULT_NUM_BLOCKS",
     "EngineConfig",
     "Llama3RopeScaling",

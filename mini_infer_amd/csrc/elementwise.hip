@@ -101,6 +101,49 @@ extern "C" int mi_take_device_tokens(int* ids, const int* from_rows, const int* 
 }
 
 // ---------------------------------------------------------------------------
+// The first kernel of a step: what `take_device_tokens` does (if `from_rows` is given), and
+// the position word of every request's state slot set to the request's length after the
+// step: slot_table[state_slots[b]][0] = seq_lens[b].  A negative slot (a padding row of a
+// recorded step) is skipped.  Slot rows are 8 int32 words.
+// ---------------------------------------------------------------------------
+
+__global__ void begin_step_kernel(int* __restrict__ ids, const int* __restrict__ from_rows,
+                                  const int* __restrict__ source, int n, int source_len, int vocab,
+                                  int* __restrict__ slot_table, const int* __restrict__ state_slots,
+                                  const int* __restrict__ seq_lens, int num_requests, int num_slots) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (from_rows != nullptr && i < n) {
+    const int row = from_rows[i];
+    if (row >= 0) {
+      const int token = source[min(row, source_len - 1)];
+      ids[i] = min(max(token, 0), vocab - 1);
+    }
+  }
+  if (slot_table != nullptr && i < num_requests) {
+    const int slot = state_slots[i];
+    if (slot >= 0 && slot < num_slots) slot_table[(int64_t)slot * 8] = seq_lens[i];
+  }
+}
+
+extern "C" int mi_begin_step(int* ids, const int* from_rows, const int* source, int n, int source_len, int vocab,
+                             int* slot_table, const int* state_slots, const int* seq_lens, int num_requests,
+                             int num_slots, hipStream_t stream) {
+  MI_REQUIRE(n >= 0 && num_requests >= 0 && vocab >= 1, "begin_step: bad sizes n=%d requests=%d vocab=%d", n,
+             num_requests, vocab);
+  MI_REQUIRE(from_rows == nullptr || (source != nullptr && source_len >= 1 && ids != nullptr),
+             "begin_step: tokens taken from the device need their source");
+  MI_REQUIRE(slot_table == nullptr || (state_slots != nullptr && seq_lens != nullptr && num_slots >= 1),
+             "begin_step: the slot table needs slot ids and lengths");
+  const int work = max(from_rows ? n : 0, slot_table ? num_requests : 0);
+  if (work == 0) return MI_OK;
+  begin_step_kernel<<<ceil_div(work, 256), 256, 0, stream>>>(ids, from_rows, source, n, source_len, vocab,
+                                                             slot_table, state_slots, seq_lens, num_requests,
+                                                             num_slots);
+  MI_CHECK_LAUNCH("begin_step");
+  return MI_OK;
+}
+
+// ---------------------------------------------------------------------------
 // residual add + RMSNorm
 //   s = residual[r] + delta[r]           (float32; stored back unless `rows` is given)
 //   out[b] = weight * s * rsqrt(mean(s^2) + eps)

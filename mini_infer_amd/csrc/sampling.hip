@@ -23,6 +23,16 @@
 #define SAMPLE_BATCH 16  // loads a thread has in flight
 #define MASS_ONE 1099511627776.0f  // 2^40
 
+// A request's row in the table of state slots (int32 words), as the cache manager lays it out.
+#define SLOT_WORDS 8
+#define SLOT_POSITION 0
+#define SLOT_SEED_LO 1
+#define SLOT_SEED_HI 2
+#define SLOT_DRAW 3
+#define SLOT_TEMPERATURE 4  // float bits
+#define SLOT_TOP_K 5
+#define SLOT_TOP_P 6  // float bits
+
 __device__ __forceinline__ uint32_t order_key(float x) {
   const uint32_t u = __float_as_uint(x);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
@@ -103,7 +113,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, const uint32_t* __restrict__ seed_lo,
     const uint32_t* __restrict__ seed_hi, const uint32_t* __restrict__ draw_index,
-    int* __restrict__ out) {
+    int* __restrict__ out, const int* __restrict__ slots, int* __restrict__ slot_table) {
   __shared__ ArgBest best_scratch[SAMPLE_WAVES];
   __shared__ uint32_t cnt[256];
   __shared__ unsigned long long mass[256];
@@ -114,7 +124,16 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
   const T* x = logits + (int64_t)row * row_stride;
-  const float temp = temperature[row];
+  // the row's settings: from the request's state slot, or from one array per setting
+  int* slot = slot_table ? slot_table + (int64_t)slots[row] * SLOT_WORDS : nullptr;
+  const float temp = slot ? __int_as_float(slot[SLOT_TEMPERATURE]) : temperature[row];
+  const int k = slot ? slot[SLOT_TOP_K] : top_k[row];
+  const float p = slot ? __int_as_float(slot[SLOT_TOP_P]) : top_p[row];
+  const uint32_t k0 = slot ? (uint32_t)slot[SLOT_SEED_LO] : seed_lo[row];
+  const uint32_t k1 = slot ? (uint32_t)slot[SLOT_SEED_HI] : seed_hi[row];
+  const uint32_t draw = slot ? (uint32_t)slot[SLOT_DRAW] : draw_index[row];
+  // every thread has read the draw index before thread 0 may advance it at the end
+  __syncthreads();
 
   if (temp == 0.f) {
     ArgBest mine = {-INFINITY, 0x7fffffff};  // rising index order: ties go to the first
@@ -122,7 +141,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       if (v > mine.val || mine.idx == 0x7fffffff) { mine.val = v; mine.idx = i; }
     });
     const ArgBest best = block_argbest(mine, best_scratch);
-    if (tid == 0) out[row] = best.idx;
+    if (tid == 0) {
+      out[row] = best.idx;
+      if (slot) slot[SLOT_DRAW] = (int)(draw + 1u);
+    }
     return;
   }
 
@@ -137,7 +159,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   uint32_t key_floor = 0;  // tokens whose key is below this are dropped
 
   // ---- top-k: the key of the k-th largest value ---------------------------
-  const int k = top_k[row];
   if (k > 0 && k < vocab) {
     uint32_t prefix = 0, mask = 0;
     uint32_t remaining = (uint32_t)k;
@@ -179,7 +200,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   }
 
   // ---- top-p: the smallest key whose mass-above is within top_p ------------
-  const float p = top_p[row];
   if (p < 1.f) {
     uint32_t prefix = 0, mask = 0;
     unsigned long long above = 0;
@@ -235,7 +255,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   }
 
   // ---- draw -----------------------------------------------------------------
-  const uint32_t k0 = seed_lo[row], k1 = seed_hi[row], draw = draw_index[row];
   ArgBest mine = {-INFINITY, 0x7fffffff};
   const int n_quads = (vocab + 3) / 4;
   constexpr int QUADS = 4;  // quads whose 16 loads are issued together
@@ -267,7 +286,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     }
   }
   const ArgBest best = block_argbest(mine, best_scratch);
-  if (tid == 0) out[row] = best.idx;
+  if (tid == 0) {
+    out[row] = best.idx;
+    if (slot) slot[SLOT_DRAW] = (int)(draw + 1u);
+  }
 }
 
 extern "C" int mi_sample(int dtype, const void* logits, int64_t row_stride, int num_rows, int vocab,
@@ -282,12 +304,38 @@ extern "C" int mi_sample(int dtype, const void* logits, int64_t row_stride, int 
   if (dtype == MI_F32) {
     sample_kernel<float><<<num_rows, SAMPLE_THREADS, 0, stream>>>(
         (const float*)logits, row_stride, vocab, temperature, top_k, top_p, seed_lo, seed_hi,
-        draw_index, out);
+        draw_index, out, nullptr, nullptr);
   } else {
     sample_kernel<bf16_t><<<num_rows, SAMPLE_THREADS, 0, stream>>>(
         (const bf16_t*)logits, row_stride, vocab, temperature, top_k, top_p, seed_lo, seed_hi,
-        draw_index, out);
+        draw_index, out, nullptr, nullptr);
   }
   MI_CHECK_LAUNCH("sample");
+  return MI_OK;
+}
+
+// The same choice with every row's settings read from its request's state slot:
+// `slots[row]` indexes `slot_table` [num_slots][8] (position, seed low, seed high, draw
+// index, temperature bits, top_k, top_p bits, unused).  The draw index of each sampled
+// slot is advanced by one, so the next call draws the request's next number without
+// the host sending anything.  A request appears in at most one row.
+extern "C" int mi_sample_slots(int dtype, const void* logits, int64_t row_stride, int num_rows, int vocab,
+                               const int* slots, int* slot_table, int* out, hipStream_t stream) {
+  MI_REQUIRE(num_rows >= 0 && vocab > 0, "sample_slots: bad sizes rows=%d vocab=%d", num_rows, vocab);
+  MI_REQUIRE(row_stride >= vocab, "sample_slots: row stride %lld is shorter than the vocabulary %d",
+             (long long)row_stride, vocab);
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "sample_slots: unknown dtype %d", dtype);
+  MI_REQUIRE(slots && slot_table, "sample_slots: needs the slot ids and the slot table");
+  if (num_rows == 0) return MI_OK;
+  if (dtype == MI_F32) {
+    sample_kernel<float><<<num_rows, SAMPLE_THREADS, 0, stream>>>(
+        (const float*)logits, row_stride, vocab, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, out,
+        slots, slot_table);
+  } else {
+    sample_kernel<bf16_t><<<num_rows, SAMPLE_THREADS, 0, stream>>>(
+        (const bf16_t*)logits, row_stride, vocab, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, out,
+        slots, slot_table);
+  }
+  MI_CHECK_LAUNCH("sample_slots");
   return MI_OK;
 }

@@ -97,7 +97,7 @@ class DecodeGraph:
         put(np.arange(b, dtype=np.int32), b)  # token_request: one token per row
         put(np.arange(b + 1, dtype=np.int32), b + 1)  # cu_seqlens_q
         put(index.seq_lens, b, pad=1)
-        put(index.state_slots, b)
+        put(index.state_slots, b, pad=-1)  # padding rows own no state slot
         put(np.arange(b, dtype=np.int32), b)  # logits wanted at every row
         for mapping, table in zip(index.slot_mapping, index.block_tables):
             put(mapping, b, pad=-1)  # padding rows write no keys or values
@@ -128,7 +128,8 @@ class DecodeGraph:
         gc.disable()
         try:
             with torch.cuda.graph(graph):
-                ops.take_device_tokens(self.ctx.token_ids, self.from_rows, self.device_tokens, self.runner.vocab_size)
+                ops.begin_step(self.ctx.token_ids, self.from_rows, self.device_tokens, self.runner.vocab_size,
+                               self.runner.cache.states.table, self.ctx.state_slots, self.ctx.seq_lens)
                 self.logits = model.forward(self.ctx, caches)
         finally:
             if collecting:
@@ -141,8 +142,9 @@ class DecodeGraph:
         index,
         from_rows: np.ndarray | None = None,
         device_tokens: torch.Tensor | None = None,
-    ) -> torch.Tensor:
-        """Logits [real rows, vocab] of this step; they live until the next replay."""
+    ) -> tuple[torch.Tensor, torch.Tensor]:
+        """Logits [real rows, vocab] of this step and the state-slot id of each row; both live
+        until the next replay."""
         self.fill(token_ids, index, from_rows)
         self.device.copy_(self.host, non_blocking=True)
         if from_rows is not None and device_tokens is not None:
@@ -153,7 +155,8 @@ class DecodeGraph:
         if self.graph is None:
             self.capture()
         self.graph.replay()
-        return self.logits[: len(index.request_ids)]
+        real = len(index.request_ids)
+        return self.logits[:real], self.ctx.state_slots[:real]
 
 
 class DecodeGraphs:
@@ -181,7 +184,7 @@ class DecodeGraphs:
         index,
         from_rows: np.ndarray | None = None,
         device_tokens: torch.Tensor | None = None,
-    ) -> torch.Tensor:
+    ) -> tuple[torch.Tensor, torch.Tensor]:
         batch = bucket_of(len(index.request_ids))
         width = bucket_of(max([t.shape[1] for t in index.block_tables] + [1]), MIN_WIDTH)
         key = (batch, width)

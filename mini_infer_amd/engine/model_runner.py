@@ -18,7 +18,7 @@ import torch
 
 from mini_infer_amd import ops
 from mini_infer_amd.cache.manager import CacheManager
-from mini_infer_amd.config import DEFAULT_BLOCK_SIZE, DEFAULT_NUM_BLOCKS, read_config_json
+from mini_infer_amd.config import DEFAULT_BLOCK_SIZE, DEFAULT_NUM_BLOCKS, EngineConfig, read_config_json
 from mini_infer_amd.engine.batch import StepEntry
 from mini_infer_amd.engine.decode_graph import DecodeGraphs
 from mini_infer_amd.models import DecoderModel, architecture_for
@@ -78,6 +78,9 @@ class ModelRunner:
             device=model.device,
         )
         self._layer_caches = self.cache.layer_caches()
+        self.engine_config: EngineConfig | None = None  # set when built from one
+        # state-slot id of every row of the logits the last step returned (int32, on the device)
+        self.last_row_slots: torch.Tensor | None = None
         # decode steps are replayed as HIP graphs where every part of the model allows it
         self.decode_graphs = DecodeGraphs(self, max_batch=64) if cuda_graph and model.graph_safe else None
 
@@ -88,6 +91,7 @@ class ModelRunner:
         cls,
         model_name: str | Path,
         *,
+        engine: EngineConfig | None = None,
         device: str = "cuda:0",
         dtype: str | torch.dtype | None = None,
         num_blocks: int = DEFAULT_NUM_BLOCKS,
@@ -95,15 +99,25 @@ class ModelRunner:
         max_concurrent: int = 16,
         cuda_graph: bool = True,
     ) -> "ModelRunner":
-        """Load the model folder `model_name` (config.json + safetensors) and build its cache."""
-        dev = require_gpu(device)
+        """Load the model folder `model_name` (config.json + safetensors) and build its cache.
+
+        The engine's knobs come as one `EngineConfig` (`engine=`) or as the keyword arguments
+        of the same names, from which one is made (and so checked) here."""
+        if engine is None:
+            engine = EngineConfig(
+                num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent, device=device,
+                dtype=str(resolve_dtype(dtype)).replace("torch.", ""), cuda_graph=cuda_graph,
+            )
+        dev = require_gpu(engine.device)
         raw = read_config_json(model_name)
         arch = architecture_for(raw)
         config = arch.parse_config(raw)
-        model = DecoderModel(arch.build_spec(config), resolve_dtype(dtype), dev)
+        model = DecoderModel(arch.build_spec(config), resolve_dtype(engine.dtype), dev)
         load_checkpoint(model, model_name)
-        return cls(model, config, num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent,
-                   cuda_graph=cuda_graph)
+        runner = cls(model, config, num_blocks=engine.num_blocks, block_size=engine.block_size,
+                     max_concurrent=engine.max_concurrent, cuda_graph=engine.cuda_graph)
+        runner.engine_config = engine
+        return runner
 
     @classmethod
     def from_random(
@@ -222,11 +236,16 @@ class ModelRunner:
             )
             token_ids = token_ids.astype(np.int32)
             if self.decode_graphs is not None and self.decode_graphs.takes(index, rows, device_tokens):
-                logits = self.decode_graphs.run(token_ids, index, from_rows, device_tokens)
+                logits, self.last_row_slots = self.decode_graphs.run(token_ids, index, from_rows, device_tokens)
             else:
-                ctx, from_rows_device = self._to_device(token_ids, rows, index, from_rows)
-                if from_rows_device is not None:
-                    ops.take_device_tokens(ctx.token_ids, from_rows_device, device_tokens, self.vocab_size)
+                row_slots = np.fromiter(
+                    (index.state_slots[b] for b, e in enumerate(entries) for _ in e.want), dtype=np.int32
+                )
+                ctx, from_rows_device, self.last_row_slots = self._to_device(token_ids, rows, index, from_rows, row_slots)
+                # tokens still on the device are taken from there, positions go into the state slots
+                if self.device.type == "cuda":
+                    ops.begin_step(ctx.token_ids, from_rows_device, device_tokens, self.vocab_size,
+                                   self.cache.states.table, ctx.state_slots, ctx.seq_lens)
                 logits = self.model.forward(ctx, self._layer_caches)
         except BaseException:
             self.cache.cancel_reservation(extents)
@@ -237,10 +256,10 @@ class ModelRunner:
         return logits
 
     def _to_device(
-        self, token_ids: np.ndarray, rows: np.ndarray, index, from_rows: np.ndarray | None = None
-    ) -> tuple[StepContext, torch.Tensor | None]:
+        self, token_ids: np.ndarray, rows: np.ndarray, index, from_rows: np.ndarray | None, row_slots: np.ndarray
+    ) -> tuple[StepContext, torch.Tensor | None, torch.Tensor]:
         """All of a step's integers in one pinned buffer and one copy to the device
-        (the step's context, and `from_rows` on the device if it was given)."""
+        (the step's context, `from_rows` on the device if it was given, and `row_slots`)."""
         pieces = [
             token_ids,
             index.positions,
@@ -249,6 +268,7 @@ class ModelRunner:
             index.seq_lens,
             index.state_slots,
             rows,
+            row_slots,
         ]
         for mapping, table in zip(index.slot_mapping, index.block_tables):
             pieces.append(mapping)
@@ -264,11 +284,11 @@ class ModelRunner:
             offset += size
         on_device = staging.to(self.device, non_blocking=True)
         views = list(torch.split(on_device, sizes))
-        token_ids_d, positions, token_request, cu, seq_lens, state_slots, rows_d = views[:7]
+        token_ids_d, positions, token_request, cu, seq_lens, state_slots, rows_d, row_slots_d = views[:8]
         slot_mapping, block_tables = [], []
         for g, table in enumerate(index.block_tables):
-            slot_mapping.append(views[7 + 2 * g])
-            block_tables.append(views[8 + 2 * g].view(table.shape))
+            slot_mapping.append(views[8 + 2 * g])
+            block_tables.append(views[9 + 2 * g].view(table.shape))
         ctx = StepContext(
             num_tokens=int(token_ids.size),
             num_requests=len(index.request_ids),
@@ -288,4 +308,4 @@ class ModelRunner:
             host_seq_lens=index.seq_lens.tolist(),
             host_state_slots=index.state_slots.tolist(),
         )
-        return ctx, (views[-1] if from_rows is not None else None)
+        return ctx, (views[-1] if from_rows is not None else None), row_slots_d

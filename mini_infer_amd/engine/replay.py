@@ -8,7 +8,9 @@ line:
 
 For a step with wanted places, `OUT/<step>.f32` holds the logits [wanted, vocab]
 as little-endian float32, in the order of the entries and of `want`.  After each
-step `done <step>` is printed and flushed.
+step `done <step>` is printed and flushed.  When the input ends, requests still live are
+ended, and the program checks that every page of the pool is free again (exit code 1 if
+one is lost, else 0).
 """
 
 from __future__ import annotations
@@ -84,6 +86,20 @@ def run(args: argparse.Namespace, lines=None, out=None) -> int:
             if runner.has_request(request_id):
                 runner.free_request(request_id)
         print(f"done {step}", file=out, flush=True)
+
+    # The input has ended: what the trace left live is given back, and then every page
+    # must be free again and none held twice: a page lost on the way is the engine's
+    # fault, never the trace's, and the only reason to end with another code than 0.
+    for request_id in runner.cache.live_requests():
+        runner.free_request(request_id)
+    try:
+        runner.cache.check()
+        lost = num_blocks - runner.num_free_blocks()
+        if lost:
+            raise AssertionError(f"{lost} of {num_blocks} pages are still held after every request ended")
+    except AssertionError as err:
+        print(f"trace_run: the cache is not whole at the end of the trace: {err}", file=sys.stderr, flush=True)
+        return 1
     return 0
 
 

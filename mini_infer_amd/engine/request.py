@@ -64,6 +64,9 @@ class RunningRequest:
     cancel_requested: bool = False
     admitted_order: int = -1
     preemptions: int = 0
+    # index of the request's next draw, as read from its state slot when it was preempted
+    # (while it runs, the slot itself holds the counter)
+    draws: int = 0
     steps: list[GenerationStep] = dataclasses.field(default_factory=list)
     done_event: threading.Event = dataclasses.field(default_factory=threading.Event)
     # asynchronous sampling: the request's newest token has been sampled but not read by the

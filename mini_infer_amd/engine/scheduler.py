@@ -40,6 +40,7 @@ import threading
 import time
 from typing import Any, Callable, Iterable, Iterator, Sequence
 
+from mini_infer_amd.config.engine_config import DEFAULT_CHUNK_SIZE, DEFAULT_DECODE_HEADROOM_BLOCKS, EngineConfig
 from mini_infer_amd.engine.batch import StepEntry
 from mini_infer_amd.engine.request import (
     GenerationResult,
@@ -50,15 +51,7 @@ from mini_infer_amd.engine.request import (
 )
 from mini_infer_amd.exceptions import EngineNotRunningError, OutOfMemoryError
 
-DEFAULT_DECODE_HEADROOM_BLOCKS = 8
-DEFAULT_CHUNK_SIZE = 256
 IDLE_SLEEP_SECONDS = 0.005
-
-
-def _device_sampler(logits, params, seeds, draws) -> list[int]:
-    from mini_infer_amd.sampling.sampler import sample_batch
-
-    return sample_batch(logits, params, seeds, draws)
 
 
 @dataclasses.dataclass(frozen=True)
@@ -172,7 +165,9 @@ class ContinuousScheduler:
             self.eos_token_ids = frozenset(int(t) for t in eos_token_id)
         self.tokenizer = tokenizer
         self.base_seed = base_seed
-        self._sample = sampler or _device_sampler
+        # None: the device's own sampler, which reads every request's settings, seed and draw
+        # index from its state slot; a callable `(logits, params, seeds, draws) -> ids` replaces it
+        self._sample = sampler
         # None: on where it can be (the runner takes tokens from the device and the sampler is the device's own)
         can_async = sampler is None and bool(getattr(runner, "supports_device_tokens", False))
         if async_sampling and not can_async:
@@ -196,6 +191,22 @@ class ContinuousScheduler:
         self.trace_out = trace_out
         self._trace_events: list[dict[str, Any]] | None = [] if trace_out is not None else None
         self._trace_start: float | None = None
+
+    @classmethod
+    def from_config(cls, runner: Any, engine: EngineConfig, **others: Any) -> "ContinuousScheduler":
+        """A scheduler with the knobs of `engine`; `others` are what an `EngineConfig` does not
+        hold (`eos_token_id`, `tokenizer`, `sampler`)."""
+        return cls(
+            runner,
+            max_concurrent=engine.max_concurrent,
+            decode_headroom_blocks=engine.decode_headroom_blocks,
+            chunk_size=engine.chunk_size,
+            max_num_batched_tokens=engine.max_num_batched_tokens,
+            base_seed=engine.seed,
+            async_sampling=engine.async_sampling,
+            trace_out=engine.trace_out,
+            **others,
+        )
 
     # -- submitting -----------------------------------------------------------
 
@@ -374,13 +385,10 @@ class ContinuousScheduler:
                 )
         if sampled_for:
             # (rows of requests that the late ids have just finished are sampled too and dropped)
-            params = [r.request.sampling_params for r in sampled_for]
-            seeds = [r.seed for r in sampled_for]
-            draws = [len(r.tokens_generated) for r in sampled_for]
             if self.async_sampling:
-                self._sample_later(logits, sampled_for, params, seeds, draws)
+                self._sample_later(logits, sampled_for)
             else:
-                token_ids = self._sample(logits, params, seeds, draws)
+                token_ids = self._sample_now(logits, sampled_for)
                 for running, token in zip(sampled_for, token_ids):
                     if running.state != RequestState.DONE:
                         self._accept_token(running, int(token))
@@ -390,13 +398,40 @@ class ContinuousScheduler:
 
     # -- asynchronous sampling ---------------------------------------------------------------
 
-    def _sample_later(self, logits, sampled_for, params, seeds, draws) -> None:
+    def _count_draws(self, sampled_for) -> None:
+        """The host's copy of each sampled request's draw index follows the device's."""
+        for running in sampled_for:
+            if running.state != RequestState.DONE and self.cache.has_request(running.request_id):
+                self.cache.states.count_draw(self.cache.state_slot(running.request_id))
+
+    def _sample_on_device(self, logits, sampled_for):
+        """One id per row, as an int32 device tensor: settings, seed and draw index of every
+        row come from its request's state slot, whose draw index the kernel advances."""
+        from mini_infer_amd.sampling.sampler import sample_from_slots
+
+        on_device = sample_from_slots(logits, self.runner.last_row_slots, self.cache.states.table)
+        self._count_draws(sampled_for)
+        return on_device
+
+    def _sample_now(self, logits, sampled_for) -> list[int]:
+        if self._sample is None:
+            return self._sample_on_device(logits, sampled_for).tolist()
+        states = self.cache.states
+        slots = [
+            self.cache.state_slot(r.request_id) if self.cache.has_request(r.request_id) else None for r in sampled_for
+        ]
+        params = [r.request.sampling_params for r in sampled_for]
+        seeds = [r.seed for r in sampled_for]
+        draws = [states.draws(slot) if slot is not None else 0 for slot in slots]
+        token_ids = self._sample(logits, params, seeds, draws)
+        self._count_draws(sampled_for)
+        return token_ids
+
+    def _sample_later(self, logits, sampled_for) -> None:
         """Sample on the device, start the copy of the ids to the host, read nothing yet."""
         import torch
 
-        from mini_infer_amd.sampling.sampler import sample_tokens
-
-        on_device = sample_tokens(logits, params, seeds, draws)
+        on_device = self._sample_on_device(logits, sampled_for)
         # One pinned buffer and one event for the scheduler's life: the ids of a step are read
         # (`_resolve_pending`) before the next step's ids are copied into the same place.
         if self._ids_on_host is None or self._ids_on_host.numel() < on_device.numel():
@@ -447,6 +482,16 @@ class ContinuousScheduler:
     def _free_pages(self) -> int:
         return self.runner.num_free_blocks()
 
+    def _promised_pages(self) -> int:
+        """Pages that requests already admitted will still take for the tokens they have not
+        fed yet (admission reserves nothing, so the pool's free count does not show them)."""
+        promised = 0
+        for running in self._running:
+            remaining = running.prefill_remaining
+            if remaining > 0 and self.cache.has_request(running.request_id):
+                promised += max(self.cache.pages_needed(running.request_id, remaining), default=0)
+        return promised
+
     def _admit_waiting(self) -> None:
         while len(self._running) < self.max_concurrent:
             with self._lock:
@@ -483,12 +528,20 @@ class ContinuousScheduler:
                 need_now,
                 min(need_now + self.decode_headroom_blocks, self._pages_for(to_feed + remaining_new - 1)),
             )
-            free = self._free_pages()
+            # what is free, less what the requests admitted before this one are about to take
+            free = self._free_pages() - self._promised_pages()
             if free < required and (self._running or free < need_now):
                 return
             with self._lock:
                 self._waiting.popleft()
             self.cache.add_request(running.request_id)
+            # the request's sampling state lives in its slot; a request that comes back after a
+            # preemption goes on with the draw index it had reached
+            params = running.request.sampling_params
+            self.cache.set_sampling(
+                running.request_id, temperature=params.temperature, top_k=params.top_k, top_p=params.top_p,
+                seed=running.seed, draw=running.draws,
+            )
             running.state = RequestState.PREFILLING
             running.tokens_fed = 0
             running.admitted_order = self._admitted
@@ -542,6 +595,7 @@ class ContinuousScheduler:
             return False
         victim = max(self._running, key=lambda r: r.admitted_order)
         self._running.remove(victim)
+        victim.draws = self.cache.states.draws(self.cache.state_slot(victim.request_id))
         self.cache.free_request(victim.request_id)
         if not self._running:
             self.stats["rejected"] += 1

@@ -120,6 +120,44 @@ def take_device_tokens(ids: torch.Tensor, from_rows: torch.Tensor, source: torch
     )
 
 
+SLOT_WORDS = 8  # int32 words of a request's row in the table of state slots
+
+
+def begin_step(
+    ids: torch.Tensor,
+    from_rows: torch.Tensor | None,
+    source: torch.Tensor | None,
+    vocab: int,
+    slot_table: torch.Tensor | None,
+    state_slots: torch.Tensor | None,
+    seq_lens: torch.Tensor | None,
+) -> None:
+    """The first kernel of a step.  With `from_rows`: `take_device_tokens`.  With
+    `slot_table` [slots, 8] int32: word 0 of row `state_slots[b]` becomes `seq_lens[b]`,
+    the request's length after this step (negative slots are skipped)."""
+    _need_cuda(ids, from_rows, source, slot_table, state_slots, seq_lens)
+    for name, t in (("ids", ids), ("from_rows", from_rows), ("source", source), ("slot_table", slot_table),
+                    ("state_slots", state_slots), ("seq_lens", seq_lens)):
+        _need_contiguous(name, t)
+        _need_int32(name, t)
+    if from_rows is not None and (source is None or source.numel() == 0 or from_rows.shape != ids.shape):
+        raise KernelShapeError("begin_step: from_rows is [n] like ids and needs a source of at least one row")
+    num_requests = num_slots = 0
+    if slot_table is not None:
+        if slot_table.dim() != 2 or slot_table.shape[1] != SLOT_WORDS or state_slots is None or seq_lens is None:
+            raise KernelShapeError(f"begin_step: the slot table is [slots, {SLOT_WORDS}] and needs state_slots and seq_lens")
+        if state_slots.numel() != seq_lens.numel():
+            raise KernelShapeError("begin_step: one slot id per request length")
+        num_requests, num_slots = state_slots.numel(), slot_table.shape[0]
+    lib = library.load()
+    library.check(
+        lib.mi_begin_step(
+            _ptr(ids), _ptr(from_rows), _ptr(source), ids.numel(), 0 if source is None else source.numel(), int(vocab),
+            _ptr(slot_table), _ptr(state_slots), _ptr(seq_lens), num_requests, num_slots, _stream(),
+        )
+    )
+
+
 @dataclasses.dataclass
 class PartialSums:
     """A product that has not been added up yet: `pieces` [S, T, N] float32 holds its sums
@@ -811,6 +849,30 @@ def sample(
             _dtype_code(logits), _ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature),
             _ptr(top_k), _ptr(top_p), _ptr(seed_lo), _ptr(seed_hi), _ptr(draw_index), _ptr(out),
             _stream(),
+        )
+    )
+    return out
+
+
+def sample_slots(logits: torch.Tensor, slots: torch.Tensor, slot_table: torch.Tensor) -> torch.Tensor:
+    """One token id per row of `logits` [B, V], each row's settings (temperature, top_k, top_p,
+    seed, draw index) read from row `slots[b]` of `slot_table` [slots, 8] int32; the draw
+    index of every sampled slot is advanced by one on the device."""
+    _need_cuda(logits, slots, slot_table)
+    if logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelShapeError("logits must be [rows, vocab] with unit inner stride")
+    rows, vocab = logits.shape
+    for name, t in (("slots", slots), ("slot_table", slot_table)):
+        _need_contiguous(name, t)
+        _need_int32(name, t)
+    if slots.numel() != rows or slot_table.dim() != 2 or slot_table.shape[1] != SLOT_WORDS:
+        raise KernelShapeError(f"sample_slots: one slot id per row and a table [slots, {SLOT_WORDS}]")
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    lib = library.load()
+    library.check(
+        lib.mi_sample_slots(
+            _dtype_code(logits), _ptr(logits), logits.stride(0), rows, vocab, _ptr(slots), _ptr(slot_table),
+            _ptr(out), _stream(),
         )
     )
     return out

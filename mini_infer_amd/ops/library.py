@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -23,6 +23,7 @@ _P = c_void_p
 _SIGNATURES: dict[str, list] = {
     "mi_embed_gather": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
     "mi_take_device_tokens": [_P, _P, _P, c_int, c_int, c_int, _P],
+    "mi_begin_step": [_P, _P, _P, c_int, c_int, c_int, _P, _P, _P, c_int, c_int, _P],
     "mi_add_rmsnorm": [c_int, _P, _P, _P, _P, _P, c_int, c_int, c_float, _P, c_int, c_int64, _P],
     "mi_rope_table": [_P, _P, _P, _P, c_int, c_int, _P],
     "mi_rope_kv_write": [
@@ -54,6 +55,7 @@ _SIGNATURES: dict[str, list] = {
     "mi_attn_mfma_tokens_per_tile": [c_int, c_int, c_int],
     "mi_attn_mfma_supported": [c_int, c_int],
     "mi_sample": [c_int, _P, c_int64, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P],
+    "mi_sample_slots": [c_int, _P, c_int64, c_int, c_int, _P, _P, _P, _P],
 }
 
 

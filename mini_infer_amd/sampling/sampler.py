@@ -56,6 +56,17 @@ def sample_tokens(
     )
 
 
+def sample_from_slots(logits: torch.Tensor, row_slots: torch.Tensor, slot_table: torch.Tensor) -> torch.Tensor:
+    """One id per row of `logits` as an int32 device tensor, every row's settings, seed and draw
+    index read on the device from its request's state slot (`row_slots[b]` of `slot_table`); the
+    kernel advances the draw index, so nothing about sampling travels from the host per step."""
+    if logits.dim() != 2 or row_slots.numel() != logits.shape[0]:
+        raise ValueError(
+            f"logits must be (batch, vocab) with one slot id per row; got {tuple(logits.shape)} and {row_slots.numel()} slots"
+        )
+    return ops.sample_slots(logits, row_slots, slot_table)
+
+
 def sample_batch(
     logits: torch.Tensor,
     params: Sequence[SamplingParams],

@@ -252,3 +252,31 @@ def test_keys_and_values_are_sized_apart_and_layout_is_what_the_mixer_declared()
     with pytest.raises(ValueError):
         CacheManager([CacheNeeds(pages=PagedKVNeeds(0, 16))], page_size=4, num_pages=2, max_requests=1,
                      allocate_storage=False)
+
+
+def test_slot_table_row_follows_the_request():
+    from mini_infer_amd import ops
+    from mini_infer_amd.cache import state_slots as layout
+
+    assert ops.SLOT_WORDS == layout.SLOT_WORDS  # the kernels and the manager agree on the row
+    m = _manager(storage=True)
+    m.add_request("a")
+    slot = m.state_slot("a")
+    assert m.states.table.shape == (4, layout.SLOT_WORDS) and m.states.table.dtype == torch.int32
+    m.set_sampling("a", temperature=0.7, top_k=40, top_p=0.95, seed=(5 << 32) | 0xFFFFFFFE, draw=3)
+    assert m.states.seed(slot) == (5 << 32) | 0xFFFFFFFE and m.states.draws(slot) == 3
+    m.reserve({"a": 6})
+    m.commit({"a": 6})
+    assert m.states.position(slot) == 6
+    m.truncate("a", 5)
+    assert m.states.position(slot) == 5
+    m.states.count_draw(slot)
+    assert m.states.draws(slot) == 4
+    # the device copy holds what was pushed (settings, seed, draw as set; position as truncated)
+    row = m.states.table[slot].tolist()
+    assert row[layout.SLOT_SEED_LO] == -2 and row[layout.SLOT_SEED_HI] == 5 and row[layout.SLOT_TOP_K] == 40
+    assert row[layout.SLOT_POSITION] == 5 and row[layout.SLOT_DRAW] == 3
+    m.free_request("a")
+    m.add_request("b")
+    assert m.state_slot("b") == slot and m.states.draws(slot) == 0 and m.states.position(slot) == 0
+    assert m.states.table[slot].tolist()[:4] == [0, 0, 0, 0]

@@ -301,11 +301,11 @@ def test_asynchronous_sampling_gives_the_tokens_of_synchronous_sampling(tmp_path
         runner.cache.check()
         return [(r.tokens, r.finish_reason) for r in results], scheduler.stats
 
-    for num_blocks in (64, 9):  # plenty of pages; so few that requests are preempted and recomputed
+    for num_blocks in (64, 7):  # plenty of pages; so few that requests are preempted and recomputed
         late, late_stats = run(True, num_blocks)
         at_once, _ = run(False, num_blocks)
         assert late == at_once, f"{num_blocks} pages"
-        if num_blocks == 9:
+        if num_blocks == 7:
             assert late_stats["preemptions"] >= 1
     assert at_once[1] == (greedy[:4], "stop")  # the end-of-sequence id is not emitted
     assert at_once[2][1] == "length" and len(at_once[2][0]) == 1
@@ -375,6 +375,33 @@ def test_trace_run_program(tmp_path, dtype):
         row = rows[at.get(number, 0)]
         at[number] = at.get(number, 0) + 1
         ru.assert_close(row[None], expected[rid][position][None], dtype, f"step {number} {rid}@{position}")
+
+
+def test_make_trace_feeds_trace_run_and_a_request_left_live_is_no_error(tmp_path):
+    """`python -m mini_infer_amd make-trace` prints what `bin/trace_run` reads; a trace that never
+    ends its last request still ends with exit code 0 (the program gives the pages back itself
+    and then finds the pool whole)."""
+    cfg, block, weights, folder = _folder(tmp_path, "A", 54)
+    made = subprocess.run(
+        [sys.executable, "-m", "mini_infer_amd", "make-trace", "--family", "mixed", "--lengths", "37,12,20",
+         "--vocab-size", str(cfg["vocab_size"]), "--seed", "3", "--tail", "6"],
+        capture_output=True, text=True, timeout=60, cwd=ROOT)
+    assert made.returncode == 0, made.stderr[-2000:]
+    lines = [json.loads(line) for line in made.stdout.splitlines()]
+    assert sum(len(e["tokens"]) for line in lines for e in line["entries"]) == 37 + 12 + 20
+    lines[-1]["end"] = []  # the last request is never ended
+    out_dir = tmp_path / "out"
+    done = subprocess.run(
+        [os.path.join(ROOT, "bin", "trace_run"), "--model", str(folder), "--dtype", "float32", "--out", str(out_dir),
+         "--max-tokens", "192", "--block-size", str(block)],
+        input="\n".join(json.dumps(line) for line in lines) + "\n", capture_output=True, text=True, timeout=110)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert done.stdout.split("\n")[:-1] == [f"done {n}" for n in range(len(lines))]
+    # the logits of the first step's first entry are the plain model's
+    first = lines[0]["entries"][0]
+    rows = np.fromfile(out_dir / "0.f32", dtype="<f4").reshape(-1, cfg["vocab_size"])
+    expected = pl.llama_logits(cfg, weights, np.array(first["tokens"]))
+    ru.assert_close(rows[: len(first["tokens"])], expected, "float32", "make-trace step 0")
 
 
 # -- long decoding, first tokens -----------------------------------------------------------

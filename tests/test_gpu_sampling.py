@@ -111,3 +111,69 @@ def test_bad_arguments():
         SamplingParams(top_p=1.5)
     with pytest.raises(ValueError, match="one params"):
         sample_tokens(torch.zeros(2, 4, device=DEV), [SamplingParams()], [0], [0])
+
+
+def test_sampling_from_state_slots_is_sampling_with_the_same_settings_and_advances_the_draw():
+    """Rows whose settings, seed and draw index are read from the requests' state slots give the
+    tokens of the same settings handed over as arrays, draw after draw, with nothing sent
+    from the host between the draws; slots not sampled are left alone."""
+    from mini_infer_amd.cache import StateSlots
+    from mini_infer_amd.sampling import sample_from_slots
+
+    slots = StateSlots(6, {}, DEV)
+    settings = [_params(temperature=0.8), _params(), _params(temperature=1.3, top_k=5),
+                _params(temperature=0.6, top_p=0.8), _params(temperature=1.0, top_k=50, top_p=0.5)]
+    seeds = [11, 12, 2**63 + 5, 14, 15]
+    owned = [slots.allocate(f"r{i}") for i in range(6)]  # 5, 4, ... or any order: ids are what counts
+    for slot, p, seed in zip(owned, settings, seeds):
+        slots.set_sampling(slot, temperature=p.temperature, top_k=p.top_k, top_p=p.top_p, seed=seed, draw=0)
+    order = [3, 0, 4, 1, 2]  # rows of the batch in another order than the slots
+    row_slots = torch.tensor([owned[i] for i in order], dtype=torch.int32, device=DEV)
+    for draw in range(4):
+        logits = torch.randn(5, 3000, generator=torch.Generator().manual_seed(10 + draw)).to(DEV)
+        expected = _sample(logits, [settings[i] for i in order], [seeds[i] for i in order], [draw] * 5)
+        assert sample_from_slots(logits, row_slots, slots.table).tolist() == expected
+    table = slots.table.cpu()
+    assert [int(table[owned[i], 3]) for i in range(5)] == [4] * 5 and int(table[owned[5], 3]) == 0
+    # one row alone, later: it goes on from its own draw index, whatever the others did
+    logits = torch.randn(1, 3000, generator=torch.Generator().manual_seed(99)).to(DEV)
+    alone = sample_from_slots(logits, row_slots[:1], slots.table).tolist()
+    assert alone == _sample(logits, [settings[3]], [seeds[3]], [4])
+    with pytest.raises(ValueError):
+        sample_from_slots(logits, row_slots, slots.table)
+
+
+def test_positions_and_draws_in_the_slot_table_follow_the_engine(tmp_path):
+    """After steps of every kind (portions, recorded single-token steps, a request left out of a
+    step) the device's slot table holds each request's length, as the host's copy does; a
+    failed step leaves it as it was."""
+    import tiny
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.exceptions import OutOfMemoryError
+
+    cfg, block = tiny.CONFIGS["A"]
+    folder = tiny.write_model_dir(tmp_path / "slots", cfg, tiny.make_weights(cfg, 70))
+    runner = ModelRunner.from_pretrained(folder, dtype="bfloat16", num_blocks=12, block_size=block, max_concurrent=3)
+    states = runner.cache.states
+
+    def check():
+        table = states.table.cpu().numpy()
+        for rid in runner.cache.live_requests():
+            slot = runner.cache.state_slot(rid)
+            assert table[slot, 0] == runner.cache.length(rid) == states.position(slot), rid
+
+    runner.step([StepEntry("a", tiny.random_tokens(cfg, 9, 1), [8]), StepEntry("b", tiny.random_tokens(cfg, 5, 2), [])])
+    check()
+    for step in range(6):  # recorded single-token steps of two requests, then of one
+        entries = [StepEntry("a", [step + 1], [0])] + ([StepEntry("b", [step + 2], [0])] if step < 4 else [])
+        runner.step(entries)
+        assert runner.last_row_slots.tolist() == [runner.cache.state_slot(e.request_id) for e in entries]
+        check()
+    assert runner.decode_graphs.replays == 6
+    with pytest.raises(OutOfMemoryError):
+        runner.step([StepEntry("a", [1] * 40, [])])
+    check()
+    runner.free_request("b")
+    runner.step([StepEntry("c", tiny.random_tokens(cfg, 7, 3), [6]), StepEntry("a", [3], [0])])
+    assert runner.cache.state_slot("c") is not None
+    check()

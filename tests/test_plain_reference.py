@@ -59,6 +59,44 @@ def test_llama3_bands_of_other_tables(head_dim, theta, factor, orig, kept, blend
     assert np.array_equal(is_div, wavelen > orig / 1.0)
 
 
+def test_llama3_hand_computed_table():
+    """The eight frequencies of head_dim 16, theta 1e4, factor 8, low 1, high 4, original
+    length 64, worked out by hand from the reference's formula text (models/blocks/rope.py:200-225),
+    with a calculator, not by running any implementation:
+
+      j  inv_freq = 1e4^(-j/8)  wavelen = 2*pi/inv_freq   band (L/high = 16, L/low = 64)
+      0  1                      6.2832                     < 16: kept            -> 1
+      1  10^-0.5 = 0.3162278    19.8692                    blend, smooth = (64/19.86918 - 1)/3 = 0.7403565
+                                 -> (1 - 0.7403565) * 0.3162278/8 + 0.7403565 * 0.3162278 = 0.2443846
+      2  0.1                    62.8319                    blend, smooth = (64/62.8319 - 1)/3 = 0.0061972
+                                 -> 0.9938028 * 0.0125 + 0.0061972 * 0.1 = 0.01304226
+      3  10^-1.5 = 0.03162278   198.692                    > 64: divided         -> 0.003952847
+      4  0.01                                                                     -> 0.00125
+      5..7                                                                        -> inv_freq / 8
+
+    A blend with `low` and `high` swapped, `1 - smooth` on the wrong term, or the band
+    edges taken on frequencies instead of wavelengths changes entries 1 and 2.
+    """
+    got = pl.inv_freq_llama3(pl.inv_freq_default(16, 10000.0), 8.0, 1.0, 4.0, 64)
+    by_hand = [1.0, 0.2443846, 0.01304226, 0.003952847, 0.00125, 10**-2.5 / 8, 1e-3 / 8, 10**-3.5 / 8]
+    assert np.allclose(got, by_hand, rtol=2e-6, atol=0)
+    # the same from the engine's own table builder
+    from mini_infer_amd.parts.position import default_inv_freq, llama3_inv_freq
+
+    ours = llama3_inv_freq(default_inv_freq(16, 10000.0), 8.0, 1.0, 4.0, 64).numpy()
+    assert np.allclose(ours, by_hand, rtol=2e-6, atol=0)
+
+
+def test_llama3_hand_computed_entry_of_the_released_table():
+    """Llama 3.1's own numbers (head_dim 128, theta 5e5, factor 8, low 1, high 4, L 8192), entry 32:
+    inv_freq = 5e5^(-0.5) = 0.001414214, wavelen = 4442.88 (between 2048 and 8192: blended),
+    smooth = (8192/4442.883 - 1)/3 = 0.2812826,
+    -> 0.7187174 * 0.001414214/8 + 0.2812826 * 0.001414214 = 0.0005248462."""
+    got = pl.inv_freq_llama3(pl.inv_freq_default(128, 500000.0), 8.0, 1.0, 4.0, 8192)
+    assert math.isclose(got[32], 0.0005248462, rel_tol=3e-6)
+    assert math.isclose(got[0], 1.0) and math.isclose(got[63], 500000.0 ** (-126 / 128) / 8, rel_tol=1e-6)
+
+
 def test_llama3_factor_one_is_identity():
     base = pl.inv_freq_default(64, 500000.0)
     assert np.allclose(pl.inv_freq_llama3(base, 1.0, 1.0, 4.0, 64), base, rtol=1e-6)

@@ -370,3 +370,63 @@ def test_a_step_that_raises_leaves_lengths_pages_and_admissions_as_they_were():
     runner.free_request("old")
     runner.free_request("new")
     assert runner.num_free_blocks() == 8
+
+
+def test_an_oversubscribed_load_is_admitted_in_waves_without_preemption():
+    """Sixteen long prompts for a pool that holds eight: admission counts the pages that the
+    requests already admitted will still take, so the rest waits instead of being admitted,
+    preempted and recomputed."""
+    runner = FakeRunner(num_blocks=4096, block_size=4, max_concurrent=16)
+    sched = make(runner, max_concurrent=16, chunk_size=512, max_num_batched_tokens=2048)
+    prompts = [prompt(2000, 100 + i) for i in range(16)]
+    handles = [sched.submit(Request(p, SamplingParams(), max_tokens=12)) for p in prompts]
+    most_live = 0
+    while sched.step():
+        most_live = max(most_live, len(runner.cache.live_requests()))
+    assert sched.stats["preemptions"] == 0 and sched.stats["rejected"] == 0
+    assert most_live == 8  # 500 pages of prompt + 3 of decoding each (8 of headroom asked for)
+    assert sched.stats["tokens_run"] == sum(len(p) + 11 for p in prompts)  # nothing was fed twice
+    for handle, p in zip(handles, prompts):
+        assert handle.wait().tokens == expected_tokens(p, 12)
+    assert runner.num_free_blocks() == runner.num_blocks
+
+
+def test_draw_index_lives_in_the_state_slot_survives_preemption_and_starts_at_zero_in_a_reused_slot():
+    """What the sampler is told comes from the request's state slot.  A preempted request is
+    given another slot when it returns and goes on with the draw index it had reached; a slot
+    that a finished request leaves starts at draw 0 for the next one."""
+    draws_by_seed: dict[int, list[int]] = {}
+    slot_rows = []
+
+    def sampler(logits, params, seeds, draws):
+        for seed, draw in zip(seeds, draws):
+            draws_by_seed.setdefault(seed, []).append(draw)
+        return logits.argmax(dim=-1).tolist()
+
+    prompts = [prompt(8, 20), prompt(8, 21), prompt(8, 22)]
+    runner = FakeRunner(num_blocks=9, block_size=4, max_concurrent=3)
+    sched = make(runner, sampler=sampler, decode_headroom_blocks=0, max_concurrent=3)
+    requests = [Request(p, SamplingParams(temperature=0.5, top_k=7, top_p=0.9, seed=1000 + i), max_tokens=12)
+                for i, p in enumerate(prompts)]
+    handles = [sched.submit(r) for r in requests]
+    sched.step()
+    states = runner.cache.states
+    for i in range(3):  # settings and seed are in the slot's row, the position follows the cache
+        slot = runner.cache.state_slot(i)
+        slot_rows.append(states.host[slot].copy())
+        assert states.seed(slot) == 1000 + i and states.position(slot) == runner.cache.length(i) == 8
+        assert states.host[slot, 5] == 7 and states.draws(slot) == 1
+        assert np.array([0.5, 0.9], dtype=np.float32).view(np.int32).tolist() == [states.host[slot, 4], states.host[slot, 6]]
+    while sched.step():
+        pass
+    assert sched.stats["preemptions"] >= 1
+    for i, (p, handle) in enumerate(zip(prompts, handles)):
+        assert handle.wait().tokens == expected_tokens(p, 12)
+        assert draws_by_seed[1000 + i] == list(range(12))  # no draw index used twice or skipped
+    # every slot is free again; the next request finds draw 0 and its own settings, not the last owner's
+    assert states.num_free == 3
+    sched.submit(Request(prompt(5, 1), SamplingParams(seed=77), max_tokens=1))
+    sched._admit_waiting()
+    slot = runner.cache.state_slot(3)
+    assert states.draws(slot) == 0 and states.seed(slot) == 77 and states.position(slot) == 0
+    assert states.host[slot, 5] == 0 and states.host[slot, 4] == 0
