@@ -88,17 +88,24 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
       const int page = bt[key / page_size];
       row_idx = (page * kv_heads + kvh) * page_size + key % page_size;
       const T* k_row = k_pages + (int64_t)row_idx * head_dim;
+      // four running sums per score (dims d, d+1, d+2, d+3 of every group of four), added
+      // at the end: shorter chains of roundings than one sum over the whole head
+      float s4[GT][4];
 #pragma unroll
-      for (int g = 0; g < GT; ++g) s[g] = 0.f;
+      for (int g = 0; g < GT; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s4[g][e] = 0.f;
       for (int d = 0; d < head_dim; d += KV) {
         const Pack<T, KV> kk = *reinterpret_cast<const Pack<T, KV>*>(k_row + d);
 #pragma unroll
         for (int e = 0; e < KV; ++e) {
           const float kf = to_f32(kk.v[e]);
 #pragma unroll
-          for (int g = 0; g < GT; ++g) s[g] += q_lds[g * head_dim + d + e] * kf;
+          for (int g = 0; g < GT; ++g) s4[g][e % 4] = fmaf(q_lds[g * head_dim + d + e], kf, s4[g][e % 4]);
         }
       }
+#pragma unroll
+      for (int g = 0; g < GT; ++g) s[g] = (s4[g][0] + s4[g][1]) + (s4[g][2] + s4[g][3]);
       const float distance = (float)(key - pos);
 #pragma unroll
       for (int g = 0; g < GT; ++g) s[g] += slope[g] * distance;

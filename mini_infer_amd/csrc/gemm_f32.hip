@@ -2,6 +2,8 @@
 // Plain FMA, no reduced-precision matrix mode.  Each output element is summed by
 // one thread in a fixed order (16-deep slices, slice by slice), so a row's result
 // does not depend on how many other rows are in the batch or on where its tile lies.
+// The slices' sums are added up with compensation (Kahan), so the rounding error of a
+// long row (K in the thousands) stays at a few units in the last place whatever K is.
 //
 // 64x64 output tile per 256-thread block, 16-deep K slices staged in LDS, 4x4
 // outputs per thread.  Any M, N, K; rows of A and W may have strides.
@@ -27,11 +29,11 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
   const int l_row = tid / 4;
   const int l_k = (tid % 4) * 4;
 
-  float acc[4][4];
+  float acc[4][4], lost[4][4];  // running sums and what their roundings have dropped so far
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = lost[i][j] = 0.f;
 
   for (int k0 = 0; k0 < k; k0 += BK) {
     {
@@ -49,8 +51,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
         w_s[l_k + i][l_row] = (r < n && k0 + l_k + i < k) ? src[i] : 0.f;
     }
     __syncthreads();
-    // two-level sum: each 16-deep slice is summed on its own, then added to the total,
-    // which keeps the rounding error of long rows (K in the thousands) small
+    // two-level sum: each 16-deep slice is summed on its own, then added to the total
     float part[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -71,7 +72,12 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] += part[i][j];
+      for (int j = 0; j < 4; ++j) {
+        const float y = part[i][j] - lost[i][j];
+        const float t = acc[i][j] + y;
+        lost[i][j] = (t - acc[i][j]) - y;
+        acc[i][j] = t;
+      }
     __syncthreads();
   }
 

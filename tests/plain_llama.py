@@ -7,6 +7,14 @@ softmax accumulate in float64 (`ACC`); the rotation angles follow the
 reference's float32 arithmetic so both sides see the same table.
 
 Weights are a dict of NumPy arrays under the checkpoint's tensor names.
+
+`store` (optional, on the whole-model function and the parts it calls): a function
+applied to every tensor that an engine computing in a narrower type would store in that
+type (the output of each norm, projection, rotation, attention, activation and the
+logits), with all arithmetic between still exact.  With `store=bf16_round` the model
+shows how far bfloat16 storage alone moves the logits of a given input, which is the
+yardstick the bfloat16 tests measure the engine's error with.  The residual stream is
+not rounded (the engine keeps it in float32).
 """
 
 from __future__ import annotations
@@ -26,10 +34,16 @@ ACC = np.float64
 def inv_freq_default(head_dim: int, theta: float) -> np.ndarray:
     """`1 / theta^(2j/D)`, j = 0..D/2-1, in float32.
 
-    models/blocks/rope.py:343-346 (`1.0 / base ** (arange(0, D, 2) / D)`).
+    models/blocks/rope.py:343-346 (`1.0 / base ** (arange(0, D, 2, dtype=float32) / D)`).
+    The table is a float32 constant of the model, like a weight: an entry that differs in
+    its last bit turns every key 2,000 positions away by another 1e-4 radians.  The
+    reference makes it with torch's float32 power, whose last bits are not NumPy's (13 of
+    the 64 entries differ for head size 128, theta 5e5), so this one line uses torch too.
     """
-    exponent = np.arange(0, head_dim, 2, dtype=np.float32) / np.float32(head_dim)
-    return (np.float32(1.0) / np.power(np.float32(theta), exponent)).astype(np.float32)
+    import torch
+
+    exponent = torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim
+    return (1.0 / (theta**exponent)).numpy().astype(np.float32)
 
 
 def inv_freq_llama3(
@@ -43,22 +57,22 @@ def inv_freq_llama3(
 
     models/blocks/rope.py:200-225: wavelengths above L/low are divided by
     `factor`, those below L/high are kept, the band between is blended with
-    `smooth = (L/wavelen - low) / (high - low)`.
+    `smooth = (L/wavelen - low) / (high - low)`.  Evaluated with torch's float32
+    operations like the table itself (a Python number divided by a float32 tensor is
+    rounded twice there, which moves last bits of the blended entries).
     """
-    inv_freq = inv_freq.astype(np.float32)
+    import torch
+
+    table = torch.from_numpy(np.ascontiguousarray(inv_freq, dtype=np.float32))
     old_len = original_max_position_embeddings
     low_wavelen = old_len / low_freq_factor
     high_wavelen = old_len / high_freq_factor
-    wavelen = (np.float32(2 * math.pi) / inv_freq).astype(np.float32)
-    scaled = np.where(wavelen > low_wavelen, inv_freq / np.float32(factor), inv_freq).astype(
-        np.float32
-    )
-    smooth = (np.float32(old_len) / wavelen - np.float32(low_freq_factor)) / np.float32(
-        high_freq_factor - low_freq_factor
-    )
-    smoothed = ((1 - smooth) * scaled / np.float32(factor) + smooth * scaled).astype(np.float32)
+    wavelen = 2 * math.pi / table
+    scaled = torch.where(wavelen > low_wavelen, table / factor, table)
+    smooth = (old_len / wavelen - low_freq_factor) / (high_freq_factor - low_freq_factor)
+    smoothed = (1 - smooth) * scaled / factor + smooth * scaled
     medium = ~(wavelen < high_wavelen) & ~(wavelen > low_wavelen)
-    return np.where(medium, smoothed, scaled).astype(np.float32)
+    return torch.where(medium, smoothed, scaled).numpy().astype(np.float32)
 
 
 def rope_tables(positions: np.ndarray, inv_freq: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
@@ -106,15 +120,26 @@ def silu(x: np.ndarray) -> np.ndarray:
     return x / (1.0 + np.exp(-x))
 
 
-def swiglu(x: np.ndarray, w_gate: np.ndarray, w_up: np.ndarray, w_down: np.ndarray) -> np.ndarray:
+def _keep(x: np.ndarray) -> np.ndarray:
+    return x
+
+
+def bf16_round(x: np.ndarray) -> np.ndarray:
+    """Values rounded to the nearest bfloat16 (ties to even), as float64."""
+    bits = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    rounded = (bits + np.uint32(0x7FFF) + ((bits >> np.uint32(16)) & np.uint32(1))) & np.uint32(0xFFFF0000)
+    return rounded.view(np.float32).astype(ACC)
+
+
+def swiglu(x: np.ndarray, w_gate: np.ndarray, w_up: np.ndarray, w_down: np.ndarray, store=_keep) -> np.ndarray:
     """`down(silu(gate(x)) * up(x))`, weights in [out, in] layout, no biases.
 
     models/blocks/swiglu.py:44-46, models/blocks/activations.py:36-45.
     """
     x = x.astype(ACC)
-    gate = x @ w_gate.astype(ACC).T
-    up = x @ w_up.astype(ACC).T
-    return (silu(gate) * up) @ w_down.astype(ACC).T
+    gate = store(x @ w_gate.astype(ACC).T)
+    up = store(x @ w_up.astype(ACC).T)
+    return store(store(silu(gate) * up) @ w_down.astype(ACC).T)
 
 
 def embedding(table: np.ndarray, ids: np.ndarray) -> np.ndarray:
@@ -176,6 +201,7 @@ def attention_layer(
     head_dim: int,
     window: int | None = None,
     kv_override: tuple[np.ndarray, np.ndarray] | None = None,
+    store=_keep,
 ) -> tuple[np.ndarray, tuple[np.ndarray, np.ndarray]]:
     """Project, rotate q and k, attend with scale 1/sqrt(D), project out.
 
@@ -185,16 +211,16 @@ def attention_layer(
     """
     t = x.shape[0]
     x = x.astype(ACC)
-    q = (x @ w_q.astype(ACC).T).reshape(t, num_heads, head_dim)
-    q = apply_rope(q, cos, sin)
+    q = store(x @ w_q.astype(ACC).T).reshape(t, num_heads, head_dim)
+    q = store(apply_rope(q, cos, sin))
     if kv_override is None:
-        k = (x @ w_k.astype(ACC).T).reshape(t, num_kv_heads, head_dim)
-        v = (x @ w_v.astype(ACC).T).reshape(t, num_kv_heads, head_dim)
-        k = apply_rope(k, cos, sin)
+        k = store(x @ w_k.astype(ACC).T).reshape(t, num_kv_heads, head_dim)
+        v = store(x @ w_v.astype(ACC).T).reshape(t, num_kv_heads, head_dim)
+        k = store(apply_rope(k, cos, sin))
     else:
         k, v = kv_override
-    out = causal_attention(q, k, v, 1.0 / math.sqrt(head_dim), window)
-    return out.reshape(t, num_heads * head_dim) @ w_o.astype(ACC).T, (k, v)
+    out = store(causal_attention(q, k, v, 1.0 / math.sqrt(head_dim), window))
+    return store(out.reshape(t, num_heads * head_dim) @ w_o.astype(ACC).T), (k, v)
 
 
 # ----------------------------------------------------------------------------
@@ -234,8 +260,10 @@ def llama_logits(
     first_position: int = 0,
     order: list[tuple[int, int | None]] | None = None,
     window: int | None | list[int | None] = None,
+    rows=None,
+    store=_keep,
 ) -> np.ndarray:
-    """Logits [T, V] of one whole sequence, float64.
+    """Logits [T, V] of one whole sequence, float64 (with `rows`: of those positions only).
 
     models/llama/llama.py:149-172 and models/blocks/transformer_block.py:95-153:
     embed; per layer `r += attn(norm(r))`, `r += mlp(norm(r))`; final norm; head
@@ -261,7 +289,7 @@ def llama_logits(
     windows = window if isinstance(window, list) else [window] * len(order)
     for call, (layer, reads) in enumerate(order):
         p = f"model.layers.{layer}."
-        h = rms_norm(r, weights[p + "input_layernorm.weight"], eps)
+        h = store(rms_norm(r, weights[p + "input_layernorm.weight"], eps))
         a, kv = attention_layer(
             h,
             weights[p + "self_attn.q_proj.weight"],
@@ -275,23 +303,27 @@ def llama_logits(
             head_dim,
             windows[call],
             kv_override=None if reads is None else kept[reads],
+            store=store,
         )
         kept.append(kv)
         r = r + a
-        h = rms_norm(r, weights[p + "post_attention_layernorm.weight"], eps)
+        h = store(rms_norm(r, weights[p + "post_attention_layernorm.weight"], eps))
         r = r + swiglu(
             h,
             weights[p + "mlp.gate_proj.weight"],
             weights[p + "mlp.up_proj.weight"],
             weights[p + "mlp.down_proj.weight"],
+            store=store,
         )
-    h = rms_norm(r, weights["model.norm.weight"], eps)
+    if rows is not None:
+        r = r[np.asarray(rows, dtype=np.int64)]
+    h = store(rms_norm(r, weights["model.norm.weight"], eps))
     head = (
         weights["model.embed_tokens.weight"]
         if cfg.get("tie_word_embeddings", False)
         else weights["lm_head.weight"]
     )
-    return h @ head.astype(ACC).T
+    return store(h @ head.astype(ACC).T)
 
 
 # ----------------------------------------------------------------------------

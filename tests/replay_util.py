@@ -13,14 +13,64 @@ from mini_infer_amd.engine.trace import (  # noqa: F401  (the schedule families 
 )
 
 FP32_TOL = 1e-4  # max-abs on logits, float32 engine against the float64 plain model
-BF16_REL_TOL = 0.04  # max-abs error allowed as a fraction of the largest |logit|
+# bfloat16 against a yardstick: the plain model with every stored tensor rounded to bfloat16
+# and all arithmetic exact shows how far bfloat16 storage alone moves the logits of this very
+# input.  The engine (which adds float32 summation and, on the matrix cores, probabilities in
+# bfloat16) may err at most twice as far at its worst logit and one and a half times as far at
+# the 99th percentile.  Measured: 0.9-1.6 times at the worst logit, 1.0-1.2 times at the 99th
+# percentile, on all tiny configurations under all schedules.
+BF16_MAX_FACTOR = 2.0
+BF16_P99_FACTOR = 1.5
+BF16_REL_TOL = 0.04  # for parts defined in tests, which have no yardstick: share of the largest |logit|
 
 
-def assert_close(got: np.ndarray, expected: np.ndarray, dtype: str, what: str = "") -> None:
-    assert got.shape == expected.shape, f"{what}: shape {got.shape} != {expected.shape}"
-    err = np.abs(got.astype(np.float64) - expected)
+class Oracle:
+    """Logits of the plain model for one request: `exact`, and `rounded` (bfloat16 storage, exact
+    arithmetic).  Indexing gives the rows asked for; the yardstick's statistics stay those of
+    the whole request, so that a comparison of few rows is not at the mercy of those rows."""
+
+    def __init__(self, exact: np.ndarray, rounded: np.ndarray, yard: tuple[float, float] | None = None) -> None:
+        self.exact, self.rounded = exact, rounded
+        if yard is None:
+            moved = np.abs(rounded - exact)
+            yard = (float(moved.max()), float(np.percentile(moved, 99)))
+        self.yard_max, self.yard_p99 = yard
+
+    @property
+    def shape(self):
+        return self.exact.shape
+
+    def __getitem__(self, rows) -> "Oracle":
+        return Oracle(self.exact[rows], self.rounded[rows], (self.yard_max, self.yard_p99))
+
+
+def oracle(cfg: dict, weights: dict, tokens, **kwargs) -> Oracle:
+    """Exact and bfloat16-storage logits of the plain NumPy model for one request."""
+    import plain_llama
+
+    ids = np.asarray(tokens)
+    return Oracle(
+        plain_llama.llama_logits(cfg, weights, ids, **kwargs),
+        plain_llama.llama_logits(cfg, weights, ids, store=plain_llama.bf16_round, **kwargs),
+    )
+
+
+def assert_close(got: np.ndarray, expected, dtype: str, what: str = "") -> None:
+    """`expected`: an `Oracle`, or an array (then bfloat16 falls back to a share of the largest logit)."""
+    yardstick = expected if isinstance(expected, Oracle) else None
+    exact = expected.exact if yardstick is not None else expected
+    assert got.shape == exact.shape, f"{what}: shape {got.shape} != {exact.shape}"
+    err = np.abs(got.astype(np.float64) - exact)
     worst = np.unravel_index(np.argmax(err), err.shape)
-    limit = FP32_TOL if dtype == "float32" else BF16_REL_TOL * max(1.0, float(np.abs(expected).max()))
+    if dtype == "float32":
+        limit = FP32_TOL
+    elif yardstick is not None:
+        limit = BF16_MAX_FACTOR * yardstick.yard_max
+        if err.size >= 2000:
+            p99, p99_limit = float(np.percentile(err, 99)), BF16_P99_FACTOR * yardstick.yard_p99
+            assert p99 < p99_limit, f"{what} [{dtype}]: 99th percentile of the error {p99:.3e} (limit {p99_limit:.3e})"
+    else:
+        limit = BF16_REL_TOL * max(1.0, float(np.abs(exact).max()))
     assert err.max() < limit, (
         f"{what} [{dtype}]: max error {err.max():.3e} at row {worst[0]} (limit {limit:.3e}); "
         f"first row over the limit: {int(np.argmax(err.max(axis=1) >= limit))}"

@@ -1,27 +1,34 @@
-"""One layer at the widths of Llama 3.1 8B (hidden 4096, 32/8 heads of 128, feed-forward
-14336, llama3 rope) against the plain model: the sums over 4,096 and 14,336 terms, the
-matrix-core attention at head size 128 and the weight-streaming GEMM shapes of the real
-model, which the tiny configurations do not reach.  The vocabulary is cut to 32,077 to
-keep the test short."""
+"""Two layers at the widths of Llama 3.1 8B (hidden 4096, 32/8 heads of 128, feed-forward
+14336, llama3 rope, the whole vocabulary of 128,256) against the plain model, where the
+benchmark runs: sums over 4,096 and 14,336 terms, the matrix-core attention at head size
+128, the weight-streaming products of the real shapes, contexts past 2,048 tokens, batches
+of 8 and of 40 single tokens through the recorded decode step.  The tiny configurations
+reach none of these.
+
+The plain side is `plain_llama_torch` (the NumPy model's twin in torch float64, pinned to
+it on the tiny configurations) run on the GPU: NumPy would take minutes here.
+"""
 
 import numpy as np
 import pytest
+import torch
 
-import plain_llama
+import plain_llama_torch as plt
 import replay_util as ru
 import tiny
 
 pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
 
 WIDE = {
     "architectures": ["LlamaForCausalLM"],
-    "num_hidden_layers": 1,
+    "num_hidden_layers": 2,
     "hidden_size": 4096,
     "num_attention_heads": 32,
     "num_key_value_heads": 8,
     "head_dim": 128,
     "intermediate_size": 14336,
-    "vocab_size": 32077,
+    "vocab_size": 128256,
     "rope_theta": 500000.0,
     "rope_scaling": {
         "rope_type": "llama3",
@@ -36,20 +43,54 @@ WIDE = {
 }
 
 
+def _make_weights(cfg, seed):
+    """`tiny.make_weights`' distributions (linear maps N(0, 1/fan_in) with q and k doubled,
+    embedding N(0, 1), norm weights U(0.5, 1.5), all bfloat16-exact), drawn on the GPU: a
+    billion values take NumPy too long."""
+    generator = torch.Generator(device=DEV).manual_seed(seed)
+    out = {}
+    for name, shape in sorted(tiny.tensor_shapes(cfg).items()):
+        if name.endswith("layernorm.weight") or name == "model.norm.weight":
+            values = torch.rand(shape, generator=generator, device=DEV) + 0.5
+        elif name == "model.embed_tokens.weight":
+            values = torch.randn(shape, generator=generator, device=DEV)
+        else:
+            values = torch.randn(shape, generator=generator, device=DEV) / shape[1] ** 0.5
+            if "q_proj" in name or "k_proj" in name:
+                values = values * 2.0
+        out[name] = values.to(torch.bfloat16)
+    return out
+
+
 @pytest.fixture(scope="module")
 def wide(tmp_path_factory):
-    weights = tiny.make_weights(WIDE, seed=8)
-    folder = tiny.write_model_dir(tmp_path_factory.mktemp("wide"), WIDE, weights)
-    requests = {"p": tiny.random_tokens(WIDE, 45, seed=1), "q": tiny.random_tokens(WIDE, 23, seed=2)}
-    expected = {rid: plain_llama.llama_logits(WIDE, weights, np.array(t)) for rid, t in requests.items()}
-    return folder, requests, expected
+    from safetensors.torch import save_file
+    import json
+
+    weights = _make_weights(WIDE, seed=8)
+    folder = tmp_path_factory.mktemp("wide")
+    (folder / "config.json").write_text(json.dumps(WIDE))
+    save_file({k: v.cpu() for k, v in weights.items()}, str(folder / "model.safetensors"))
+    plain_weights = {k: v.double() for k, v in weights.items()}  # on the GPU, for the plain model
+
+    def oracle(tokens, rows=None):
+        return ru.Oracle(
+            plt.llama_logits(WIDE, plain_weights, tokens, rows=rows, device=DEV),
+            plt.llama_logits(WIDE, plain_weights, tokens, rows=rows, device=DEV, store=plt.bf16_round),
+        )
+
+    yield folder, oracle
+    plain_weights.clear()
+    torch.cuda.empty_cache()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_real_widths_under_three_schedules(wide, dtype):
     from mini_infer_amd.engine import ModelRunner
 
-    folder, requests, expected = wide
+    folder, oracle = wide
+    requests = {"p": tiny.random_tokens(WIDE, 45, seed=1), "q": tiny.random_tokens(WIDE, 23, seed=2)}
+    expected = {rid: oracle(t) for rid, t in requests.items()}
     runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=8, block_size=16)
     schedules = {
         "whole": ru.schedule_whole(requests),
@@ -86,17 +127,79 @@ def test_single_tokens_over_a_longer_context_at_real_widths(wide, monkeypatch):
 
     monkeypatch.setattr(ops, "linear_from_attention", count_from_attention)
     monkeypatch.setattr(kernels, "linear_partial_sums", count_partial_sums)
-    folder, _, _ = wide
+    folder, oracle = wide
     tokens = tiny.random_tokens(WIDE, 600, seed=5)
-    expected = plain_llama.llama_logits(WIDE, tiny.make_weights(WIDE, seed=8), np.array(tokens))  # the fixture's weights
+    expected = oracle(tokens, rows=list(range(582, 600)))
     runner = ModelRunner.from_pretrained(folder, dtype="bfloat16", num_blocks=40, block_size=16)
     got = [runner.step([StepEntry("r", tokens[:583], [582])]).cpu().numpy()]
     got.append(runner.step([StepEntry("r", tokens[583:590], list(range(7)))]).cpu().numpy())
     for at in range(590, 600):
         got.append(runner.step([StepEntry("r", tokens[at : at + 1], [0])]).cpu().numpy())
-    seen = expected.copy()
-    seen[582:600] = np.concatenate(got)
-    ru.assert_close(seen, expected, "bfloat16", "8B widths, 600 tokens")
+    ru.assert_close(np.concatenate(got), expected, "bfloat16", "8B widths, 600 tokens")
     assert calls["from_attention"] >= 1 and calls["partial_sums"] >= 1  # (a replayed step calls nothing)
+    assert runner.decode_graphs.replays == 10
     runner.free_request("r")
     assert runner.num_free_blocks() == 40
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_eight_requests_past_two_thousand_tokens_decoded_in_recorded_steps(wide, dtype):
+    """The benchmark's regime: 8 requests with contexts of about 2,100 tokens, decoded together
+    for 4 steps (in bfloat16 the batch-of-8 graph, replayed: 8 rows through the fused
+    projection + rotation + cache write, the matrix-core attention over 130 pages each, the
+    down product left in partial sums).  The last prompt position and every decoded position
+    of each request is compared."""
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+
+    folder, oracle = wide
+    lengths = [2075, 2110, 2048, 2099, 2064, 2081, 2107, 2090]
+    decode = 4
+    requests = {f"c{i}": tiny.random_tokens(WIDE, n + decode, seed=60 + i) for i, n in enumerate(lengths)}
+    pages = sum(-(-(n + decode) // 16) for n in lengths)
+    runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=pages, block_size=16, max_concurrent=8)
+    got = {rid: [] for rid in requests}
+    for (rid, tokens), n in zip(requests.items(), lengths):
+        got[rid].append(runner.step([StepEntry(rid, tokens[:n], [n - 1])]).cpu().numpy())
+    for k in range(decode):
+        entries = [StepEntry(rid, [requests[rid][n + k]], [0]) for rid, n in zip(requests, lengths)]
+        logits = runner.step(entries).cpu().numpy()
+        for row, rid in enumerate(requests):
+            got[rid].append(logits[row : row + 1])
+    if dtype == "bfloat16":
+        assert runner.decode_graphs.replays == decode and list(runner.decode_graphs.graphs) == [(8, 256)]
+    for (rid, tokens), n in zip(requests.items(), lengths):
+        expected = oracle(tokens, rows=list(range(n - 1, n + decode)))
+        ru.assert_close(np.concatenate(got[rid]), expected, dtype, f"8B widths, batch 8, {rid} ({n} tokens)")
+    assert runner.num_free_blocks() == 0
+    for rid in requests:
+        runner.free_request(rid)
+    runner.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_forty_single_tokens_in_one_step(wide, dtype):
+    """40 requests with contexts of 17 to 290 tokens each bring one token to the same step (in
+    bfloat16 the batch-of-64 graph with 24 padding rows: the vendor library's products for
+    q|k|v and gate|up recorded in the graph, o and down left in partial sums, decode attention
+    with rows that write nowhere).  Twice, so that the second step is a replay."""
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+
+    folder, oracle = wide
+    lengths = [17 + (7 * i) % 274 for i in range(40)]
+    requests = {f"s{i}": tiny.random_tokens(WIDE, n + 2, seed=100 + i) for i, n in enumerate(lengths)}
+    runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=40 * 19, block_size=16, max_concurrent=40)
+    ids = list(requests)
+    for first in range(0, 40, 8):  # the prompts, eight requests a step
+        runner.step([StepEntry(rid, requests[rid][: lengths[ids.index(rid)]], []) for rid in ids[first : first + 8]])
+    got = []
+    for k in range(2):
+        entries = [StepEntry(rid, [requests[rid][n + k]], [0]) for rid, n in zip(ids, lengths)]
+        got.append(runner.step(entries).cpu().numpy())
+    if dtype == "bfloat16":
+        assert runner.decode_graphs.replays == 2 and list(runner.decode_graphs.graphs) == [(64, 32)]
+    for row, (rid, n) in enumerate(zip(ids, lengths)):
+        expected = oracle(requests[rid], rows=[n, n + 1])
+        ru.assert_close(np.stack([got[0][row], got[1][row]]), expected, dtype, f"8B widths, 40 rows, {rid} ({n} tokens)")
+    for rid in ids:
+        runner.free_request(rid)
+    runner.cache.check()

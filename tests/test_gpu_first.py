@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-import plain_llama
+import replay_util as ru
 import tiny
 
 pytestmark = pytest.mark.gpu
@@ -19,13 +19,11 @@ def test_whole_prompt_logits(tmp_path, name, dtype):
     weights = tiny.make_weights(cfg, seed=ord(name))
     folder = tiny.write_model_dir(tmp_path / name, cfg, weights)
     tokens = tiny.random_tokens(cfg, 75, seed=7)
-    expected = plain_llama.llama_logits(cfg, weights, np.array(tokens))
+    expected = ru.oracle(cfg, weights, tokens)
 
     runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=64, block_size=block)
     got = runner.step([StepEntry("r", tokens, list(range(len(tokens))))]).cpu().numpy()
-    err = np.abs(got - expected).max()
-    print(f"{name} {dtype}: max |logit| {np.abs(expected).max():.3f}, max err {err:.3e}")
-    if dtype == "float32":
-        assert err < 1e-4
-    else:
-        assert err < 0.08 * max(1.0, np.abs(expected).max())
+    err = np.abs(got - expected.exact).max()
+    print(f"{name} {dtype}: max |logit| {np.abs(expected.exact).max():.3f}, max err {err:.3e}, "
+          f"bfloat16 storage alone {expected.yard_max:.3e}")
+    ru.assert_close(got, expected, dtype, f"{name} whole prompt")

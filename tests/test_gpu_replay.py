@@ -10,7 +10,6 @@ the plain whole-sequence model.
 import numpy as np
 import pytest
 
-import plain_llama
 import replay_util as ru
 import tiny
 
@@ -26,7 +25,7 @@ def case(request, tmp_path_factory):
     weights = tiny.make_weights(cfg, seed=100 + ord(name))
     folder = tiny.write_model_dir(tmp_path_factory.mktemp(f"model{name}"), cfg, weights)
     requests = {f"r{i}": tiny.random_tokens(cfg, n, seed=i) for i, n in enumerate(LENGTHS)}
-    expected = {rid: plain_llama.llama_logits(cfg, weights, np.array(t)) for rid, t in requests.items()}
+    expected = {rid: ru.oracle(cfg, weights, t) for rid, t in requests.items()}
     return name, cfg, block, folder, requests, expected
 
 

@@ -108,9 +108,9 @@ def test_engine_tables_equal_plain_tables():
     for head_dim, theta in ((16, 10000.0), (32, 500000.0), (128, 500000.0), (48, 20000.0)):
         ours = default_inv_freq(head_dim, theta).numpy()
         plain = pl.inv_freq_default(head_dim, theta)
-        assert np.allclose(ours, plain, rtol=2e-7, atol=0)
+        assert np.array_equal(ours, plain)  # bit for bit: one last bit is 1e-4 radians at position 2,000
         ours3 = llama3_inv_freq(torch.from_numpy(plain), 8.0, 1.0, 4.0, 64).numpy()
-        assert np.allclose(ours3, pl.inv_freq_llama3(plain, 8.0, 1.0, 4.0, 64), rtol=5e-7, atol=0)  # blend: a few ulp
+        assert np.array_equal(ours3, pl.inv_freq_llama3(plain, 8.0, 1.0, 4.0, 64))
 
 
 # -- rotation -----------------------------------------------------------------------
@@ -302,6 +302,33 @@ def test_order_list_and_cache_reading():
     looped = pl.llama_logits(cfg, weights, tokens, order=[(0, None), (1, None), (0, None)])
     shared = pl.llama_logits(cfg, weights, tokens, order=[(0, None), (1, 0)])
     assert not np.allclose(looped, base) and not np.allclose(shared, base)
+
+
+def test_torch_twin_of_the_plain_model_equals_it():
+    """`plain_llama_torch` (the same formulas in torch float64, for inputs too large for NumPy) is
+    pinned to the NumPy implementation on all tiny configurations, with and without rounding
+    of the stored tensors, whole and at chosen rows."""
+    import plain_llama_torch as plt
+
+    for name in "ABC":
+        cfg, _ = tiny.CONFIGS[name]
+        weights = tiny.make_weights(cfg, 40 + ord(name))
+        tokens = tiny.random_tokens(cfg, 70, 5)
+        exact = pl.llama_logits(cfg, weights, np.array(tokens))
+        assert np.abs(plt.llama_logits(cfg, weights, tokens) - exact).max() < 1e-9
+        assert np.abs(plt.llama_logits(cfg, weights, tokens, rows=[0, 41, 69]) - exact[[0, 41, 69]]).max() < 1e-9
+        rounded = pl.llama_logits(cfg, weights, np.array(tokens), store=pl.bf16_round)
+        twin = plt.llama_logits(cfg, weights, tokens, store=plt.bf16_round)
+        # a value that sits on a rounding boundary may fall to either side in the two libraries
+        assert np.mean(np.abs(twin - rounded) > 1e-9) < 0.02
+        assert 0 < np.abs(rounded - exact).max() < 0.05 * np.abs(exact).max()
+
+
+def test_bf16_round_is_round_to_nearest_even():
+    x = np.array([1.0, 1.00390625, 1.01171875, -3.0e-40, 65280.0, 1.0 + 2.0**-9], dtype=np.float64)
+    assert np.array_equal(pl.bf16_round(x), torch.from_numpy(x).float().bfloat16().double().numpy())
+    assert pl.bf16_round(np.array([1.00390625]))[0] == 1.0  # a tie goes to the even neighbour
+    assert pl.bf16_round(np.array([1.01171875]))[0] == 1.015625
 
 
 # -- sampling ---------------------------------------------------------------------
