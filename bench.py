@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--serving] [--reference-workload]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--sizes 8b|3b|70b]
+                    [--max-context N] [--serving] [--reference-workload]
 
 Default workload: the layer sizes of Llama 3.1 8B with random bfloat16 weights
 made on the device, a batch of 8 requests with 2,048-token uniform-random prompts,
@@ -222,6 +223,65 @@ def measure_reference_workload(dtype: str) -> dict:
     }
 
 
+def measure_attention(tokens: int, batch: int, repeats: int, sizes: dict) -> dict:
+    """The attention kernel alone at the head sizes of `sizes`, on random keys, values and
+    queries in shuffled pages (the workload of the hardware-counter runs under `profiles/`):
+    with `batch` == 0 one whole prompt of `tokens` tokens (prefill shape, causal), else one
+    token of each of `batch` requests over `tokens` keys (decode shape)."""
+    import math
+
+    import torch
+
+    from mini_infer_amd import ops
+
+    device = "cuda:0"
+    q_heads, kv_heads, head_dim = sizes["num_attention_heads"], sizes["num_key_value_heads"], sizes["head_dim"]
+    requests = max(1, batch)
+    pages_each = -(-tokens // BLOCK_SIZE)
+    pages = requests * pages_each
+    keys = (torch.randn(pages, kv_heads, BLOCK_SIZE, head_dim, device=device) * 0.5).bfloat16()
+    values = (torch.randn(pages, kv_heads, head_dim, BLOCK_SIZE, device=device) * 0.5).bfloat16()  # transposed pages
+    table = torch.randperm(pages, device=device).int().view(requests, pages_each).contiguous()
+    if batch == 0:
+        rows, cu = tokens, [0, tokens]
+        positions = torch.arange(tokens, dtype=torch.int32, device=device)
+        token_request = torch.zeros(tokens, dtype=torch.int32, device=device)
+        flops = 4.0 * head_dim * q_heads * tokens * (tokens + 1) / 2
+        moved = 2.0 * tokens * kv_heads * head_dim * 2
+    else:
+        rows, cu = batch, list(range(batch + 1))
+        positions = torch.full((batch,), tokens - 1, dtype=torch.int32, device=device)
+        token_request = torch.arange(batch, dtype=torch.int32, device=device)
+        flops = 4.0 * head_dim * q_heads * tokens * batch
+        moved = 2.0 * tokens * kv_heads * head_dim * 2 * batch
+    queries = torch.randn(rows, q_heads * head_dim, device=device).bfloat16()
+    cu_device = torch.tensor(cu, dtype=torch.int32, device=device)
+
+    def call() -> None:
+        ops.paged_attention(
+            queries, keys, values, table, token_request, positions, cu_device, cu, q_heads=q_heads,
+            kv_heads=kv_heads, head_dim=head_dim, scale=1 / math.sqrt(head_dim), window=None,
+            max_seq_len=tokens, v_transposed=True,
+        )
+
+    call()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(repeats):
+        call()
+    end.record()
+    torch.cuda.synchronize()
+    seconds = start.elapsed_time(end) / 1e3 / repeats
+    return {
+        "kernel": "paged attention, " + ("one prompt (prefill shape)" if batch == 0 else f"{batch} single tokens (decode shape)"),
+        "tokens": tokens, "q_heads": q_heads, "kv_heads": kv_heads, "head_dim": head_dim,
+        "us": round(seconds * 1e6, 2), "tflops": round(flops / seconds / 1e12, 1),
+        "frac_of_bf16_peak": round(flops / seconds / PEAK_FLOPS["bf16"], 4),
+        "kv_gb_s": round(moved / seconds / 1e9, 1),
+    }
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -232,6 +292,8 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (both numbers are reported)")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--sizes", choices=sorted(SIZES), default="8b", help="layer sizes of the model (default: Llama 3.1 8B)")
+    parser.add_argument("--max-context", type=int, default=2 * PROMPT_LEN,
+                        help="total positions a request may reach (default 4,096; 8,192 for the 70B workload)")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument(
@@ -243,12 +305,24 @@ def main() -> int:
         help="also run the workload the reference publishes numbers for (1,024-token prompts, 128 tokens, "
         "1 request and 16 at once; adds a 'reference_workload' entry)",
     )
+    parser.add_argument(
+        "--attention", type=int, default=None, metavar="TOKENS",
+        help="time the attention kernel alone instead: one prompt of TOKENS tokens, or with --attention-batch B one "
+        "token of each of B requests over TOKENS keys; prints one JSON line and exits",
+    )
+    parser.add_argument("--attention-batch", type=int, default=0)
+    parser.add_argument("--attention-repeats", type=int, default=20)
     args = parser.parse_args()
+    if args.attention is not None:
+        print(json.dumps(measure_attention(args.attention, args.attention_batch, args.attention_repeats, SIZES[args.sizes][1])), flush=True)
+        return 0
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
-    if args.steps <= 0 or args.warmup < 0 or args.steps + args.warmup > PROMPT_LEN:
-        print(f"bench.py: --warmup + --steps must be at most {PROMPT_LEN} (decoding runs from 2,048 to at most 4,096)")
+    room = args.max_context - PROMPT_LEN
+    if args.steps <= 0 or args.warmup < 0 or args.steps + args.warmup > room:
+        print(f"bench.py: --warmup + --steps must be at most {room} (decoding runs from {PROMPT_LEN} to at most "
+              f"{args.max_context} positions; see --max-context)")
         return 2
 
     import numpy as np
@@ -266,6 +340,8 @@ def main() -> int:
     context_end = PROMPT_LEN + args.warmup + args.steps
     pages_per_request = -(-(context_end + 1) // BLOCK_SIZE)
     num_blocks = max(batches) * pages_per_request + 8
+    print(f"bench.py: {model_name} layer sizes, {cfg['num_hidden_layers']} layers: making random weights on the device",
+          file=sys.stderr, flush=True)
     runner = ModelRunner.from_random(
         cfg,
         seed=0,
@@ -274,6 +350,7 @@ def main() -> int:
         block_size=BLOCK_SIZE,
         max_concurrent=max(batches),
     )
+    print("bench.py: weights are on the device", file=sys.stderr, flush=True)
     rng = np.random.default_rng(0)
 
     def sample(logits) -> torch.Tensor:
@@ -331,6 +408,9 @@ def main() -> int:
             on_device = one_step(on_device, last, draw)
             if k > 0:
                 generated += len(read_ids(draw - 1))
+            if k % 1024 == 1023:  # a long run shows that it is alive (a line on stderr every thousand steps)
+                print(f"bench.py: batch {batch}: {k + 1} of {args.steps} steps, "
+                      f"{(time.perf_counter() - started) / (k + 1) * 1e3:.3f} ms a step so far", file=sys.stderr, flush=True)
         generated += len(read_ids(args.warmup + args.steps - 1))
         sync()
         assert generated == batch * args.steps
