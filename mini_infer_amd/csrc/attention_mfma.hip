@@ -224,15 +224,26 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     for (int s = 0; s < KSTEPS; ++s) q_reg[rg][s] = *reinterpret_cast<const bf16x8_t*>(q_row + s * 32);
   }
 
-  f32x4_t o_acc[RG][DBLOCKS];
-  float m_run[RG], l_run[RG];  // running maximum (log2 units) and sum of exp2(score - max)
+  // Where the sum of a row's probabilities is kept.  Prefill shape (SHARED): in one more
+  // block of the value product, o_acc[rg][DBLOCKS], whose value rows are all ones: the matrix
+  // pipe adds up the probabilities (as rounded to bfloat16, the very numbers the values are
+  // weighted with), every lane finds its row's sum in all four values it holds of that
+  // block, and the vector pipe is spared an addition per score and a reduction per block.
+  // Decode shape: in l_run, added up by the vector pipe (which idles there anyway).
+  constexpr bool SUM_ON_MATRIX_PIPE = SHARED;
+  constexpr int ACC_BLOCKS = DBLOCKS + (SUM_ON_MATRIX_PIPE ? 1 : 0);
+  f32x4_t o_acc[RG][ACC_BLOCKS];
+  float m_run[RG], l_run[RG];  // reference point of the exponentials (log2 units); sum of exp2(score - reference)
 #pragma unroll
   for (int rg = 0; rg < RG; ++rg) {
 #pragma unroll
-    for (int db = 0; db < DBLOCKS; ++db) o_acc[rg][db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int db = 0; db < ACC_BLOCKS; ++db) o_acc[rg][db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     m_run[rg] = -INFINITY;
     l_run[rg] = 0.f;
   }
+  bf16x8_t ones;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ones[i] = (bf16_t)1.0f;
 
   // One 32-key block: the K operands of its two 16-key halves and where its V^T operands
   // start.  A half never straddles a page; K rows of a (page, head) chunk are
@@ -346,27 +357,46 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
           }
         }
       }
-      mx = quad_max(mx) * scale_log2;
-      // The reference point of the exponentials follows the running maximum lazily: it
-      // moves only when the maximum grows by more than RESCALE_SLACK (in log2 units), so
-      // probabilities stay below 2^RESCALE_SLACK and the accumulator is rarely rescaled.
-      const float m_new = (mx > m_run[rg] + RESCALE_SLACK) ? mx : m_run[rg];
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen nothing yet
-      // A row's first visible block moves the reference from -inf; its sum and accumulator
-      // are still zero, so nothing is to be rescaled (alpha 1, not exp2(-inf)).
-      // arguments are bounded above: the hardware exp2 is exact enough, tiny results flush to 0
-      alpha[rg] = (m_run[rg] == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[rg] - m_safe);
-      float sum = 0.f;
+      if constexpr (SUM_ON_MATRIX_PIPE) {
+        mx *= scale_log2;
+        // The reference point of the exponentials follows the running maximum lazily: it
+        // moves only when the maximum grows by more than RESCALE_SLACK (in log2 units), so
+        // probabilities stay below 2^RESCALE_SLACK and the accumulator is rarely rescaled.
+        // Each lane looks at its own 8 scores first; only if some lane of the wave finds
+        // one that far above the reference do the 4 lanes of a row agree on a maximum.
+        alpha[rg] = 1.f;
+        if (__ballot(mx > m_run[rg] + RESCALE_SLACK) != 0ull) {
+          mx = quad_max(mx);
+          const float m_new = (mx > m_run[rg] + RESCALE_SLACK) ? mx : m_run[rg];
+          // A row's first visible block moves the reference from -inf; its sums are still
+          // zero, so nothing is to be rescaled (alpha 1, not exp2(-inf)).
+          alpha[rg] = (m_run[rg] == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[rg] - m_new);
+          m_run[rg] = m_new;
+          moved = moved || (__ballot(alpha[rg] != 1.f) != 0ull);
+        }
+        const float m_safe = (m_run[rg] == -INFINITY) ? 0.f : m_run[rg];  // a row that has seen nothing yet
+        // arguments are bounded above: the hardware exp2 is exact enough, tiny results flush to 0
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], scale_log2, -m_safe));
-        sum += p;
-        p_reg[rg][i] = (bf16_t)p;
+        for (int i = 0; i < 8; ++i)
+          p_reg[rg][i] = (bf16_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], scale_log2, -m_safe));
+      } else {
+        mx = quad_max(mx) * scale_log2;
+        // (the same lazy reference point; here every block agrees on the row's maximum)
+        const float m_new = (mx > m_run[rg] + RESCALE_SLACK) ? mx : m_run[rg];
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen nothing yet
+        alpha[rg] = (m_run[rg] == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[rg] - m_safe);
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], scale_log2, -m_safe));
+          sum += p;
+          p_reg[rg][i] = (bf16_t)p;
+        }
+        sum = quad_sum(sum);
+        l_run[rg] = l_run[rg] * alpha[rg] + sum;
+        m_run[rg] = m_new;
+        moved = moved || (__ballot(alpha[rg] != 1.f) != 0ull);
       }
-      sum = quad_sum(sum);
-      l_run[rg] = l_run[rg] * alpha[rg] + sum;
-      m_run[rg] = m_new;
-      moved = moved || (__ballot(alpha[rg] != 1.f) != 0ull);
     }
     return moved;
   };
@@ -375,17 +405,20 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg)
 #pragma unroll
-      for (int db = 0; db < DBLOCKS; ++db)
+      for (int db = 0; db < ACC_BLOCKS; ++db)
 #pragma unroll
         for (int r = 0; r < 4; ++r) o_acc[rg][db][r] *= alpha[rg];
   };
   // ---- O^T += V^T . P^T ------------------------------------------------------------------
   auto block_values = [&](const bf16x8_t* v_op, const bf16x8_t (&p_reg)[RG]) {
 #pragma unroll
-    for (int rg = 0; rg < RG; ++rg)
+    for (int rg = 0; rg < RG; ++rg) {
 #pragma unroll
       for (int db = 0; db < DBLOCKS; ++db)
         o_acc[rg][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op[db], p_reg[rg], o_acc[rg][db], 0, 0, 0);
+      if constexpr (SUM_ON_MATRIX_PIPE)
+        o_acc[rg][DBLOCKS] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, p_reg[rg], o_acc[rg][DBLOCKS], 0, 0, 0);
+    }
   };
   auto compute_block = [&](int kb, KVBlock& blk) {
     bf16x8_t v_late[DBLOCKS];
@@ -421,32 +454,52 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][D * VROW];
     const int tid = threadIdx.x;
     bf16x8_t k_stage[K_PER], v_stage[V_PER];
+    // Which half of the tile (16 keys of one page) and which 16 bytes of it a thread fetches
+    // never changes: the offsets inside the half are made once, and the half is the same
+    // for all lanes of a wave (a half's chunks are a multiple of 64), so the address of
+    // a load is a scalar base plus a fixed lane offset and costs no vector arithmetic.
+    // (Offsets from the kernel's own pointer arguments, not pointers picked from an array:
+    // those lose their address space, become flat loads, and flat loads are counted with
+    // the LDS reads, so that every wait for an operand read would wait for them too.)
+    static_assert((16 * CPR) % 64 == 0 && (2 * D) % 64 == 0, "a half's chunks fill whole waves");
+    int k_half[K_PER], v_half[V_PER];
+    unsigned k_lane_off[K_PER], v_lane_off_tile[V_PER];
+#pragma unroll
+    for (int j = 0; j < K_PER; ++j) {
+      const int id = tid + j * THREADS;
+      k_half[j] = __builtin_amdgcn_readfirstlane(id / (16 * CPR));
+      k_lane_off[j] = (unsigned)(id % (16 * CPR)) * 8u;  // a half's 16 key rows are contiguous
+    }
+#pragma unroll
+    for (int j = 0; j < V_PER; ++j) {
+      const int id = tid + j * THREADS;
+      v_half[j] = __builtin_amdgcn_readfirstlane(id / (2 * D));
+      const int dim = (id % (2 * D)) / 2, part = id % 2;
+      v_lane_off_tile[j] = (unsigned)(dim * page_size + part * 8);
+    }
     auto request_tile = [&](int kb, const PageIds& ids) {
-      const bf16_t* k_base[2];
-      const bf16_t* v_base[2];
+      int64_t k_off[2], v_off[2];  // elements from the start of the key and value pages
 #pragma unroll
       for (int hlf = 0; hlf < 2; ++hlf) {
         const int key0 = kb + 16 * hlf;
         const int page = max(ids.page[hlf], 0);
         const int64_t chunk_off = (int64_t)page * page_stride + head_off;
         const int slot0 = key0 - page_index(key0) * page_size;
-        k_base[hlf] = k_pages + chunk_off + (int64_t)slot0 * D;
-        v_base[hlf] = vt_pages + chunk_off + slot0;
+        k_off[hlf] = chunk_off + (int64_t)slot0 * D;
+        v_off[hlf] = chunk_off + slot0;
       }
 #pragma unroll
       for (int j = 0; j < K_PER; ++j) {
-        const int id = tid + j * THREADS;
-        if (K_CHUNKS % THREADS == 0 || id < K_CHUNKS) {
-          const int key = id / CPR, part = id % CPR;
-          k_stage[j] = *reinterpret_cast<const bf16x8_t*>(k_base[key / 16] + (key % 16) * D + part * 8);
+        if (K_CHUNKS % THREADS == 0 || tid + j * THREADS < K_CHUNKS) {
+          const bf16_t* base = k_pages + (k_half[j] ? k_off[1] : k_off[0]);
+          k_stage[j] = *reinterpret_cast<const bf16x8_t*>(base + k_lane_off[j]);
         }
       }
 #pragma unroll
       for (int j = 0; j < V_PER; ++j) {
-        const int id = tid + j * THREADS;
-        if (V_CHUNKS % THREADS == 0 || id < V_CHUNKS) {
-          const int hlf = id / (2 * D), dim = (id % (2 * D)) / 2, part = id % 2;
-          v_stage[j] = *reinterpret_cast<const bf16x8_t*>(v_base[hlf] + dim * page_size + part * 8);
+        if (V_CHUNKS % THREADS == 0 || tid + j * THREADS < V_CHUNKS) {
+          const bf16_t* base = vt_pages + (v_half[j] ? v_off[1] : v_off[0]);
+          v_stage[j] = *reinterpret_cast<const bf16x8_t*>(base + v_lane_off_tile[j]);
         }
       }
     };
@@ -610,6 +663,12 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
 #pragma unroll
   for (int rg = 0; rg < RG; ++rg) {
     if (!row_valid[rg]) continue;
+    if constexpr (SUM_ON_MATRIX_PIPE) {
+      // the four values are equal; 4x/4 is exact, and reading all four leaves no dead
+      // lane in a register tuple that lives across the key loop
+      const f32x4_t s4 = o_acc[rg][ACC_BLOCKS - 1];
+      l_run[rg] = 0.25f * ((s4[0] + s4[1]) + (s4[2] + s4[3]));
+    }
     if (num_splits == 1) {
       const float inv = 1.f / l_run[rg];
       bf16_t* o = out + (int64_t)token[rg] * out_row_stride + (int64_t)head[rg] * D + quad * 4;
