@@ -37,6 +37,8 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 
 #define RESCALE_SLACK 8.0f
 #define LOG2E 1.4426950408889634f
@@ -244,6 +246,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   bf16x8_t ones;
 #pragma unroll
   for (int i = 0; i < 8; ++i) ones[i] = (bf16_t)1.0f;
+  asm volatile("" : "+v"(ones));  // registers of its own for the whole kernel, not a constant made anew in every turn
 
   // One 32-key block: the K operands of its two 16-key halves and where its V^T operands
   // start.  A half never straddles a page; K rows of a (page, head) chunk are
@@ -329,8 +332,22 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   // the factor the old accumulator must be multiplied with in alpha; returns whether any
   // row of the wave needs that multiplication (alpha != 1 somewhere).
   auto block_softmax = [&](int kb, f32x4_t (&s_acc)[RG][2], bf16x8_t (&p_reg)[RG], float (&alpha)[RG]) -> bool {
-    // a block every row of this wave sees whole needs no mask (most blocks of a long prompt)
+    // a block every row of this wave sees whole needs no mask (most blocks of a long prompt);
+    // elsewhere hidden scores become -inf where they lie, before anything reads them (one
+    // branch for all row groups, and no second copy of the scores for the two ways to merge in)
     const bool interior = kb >= wave_lo_max && kb + 31 <= wave_pos_min && kb >= k_begin && kb + 32 <= k_end;
+    if (!interior) {
+#pragma unroll
+      for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+        for (int hlf = 0; hlf < 2; ++hlf)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int key = kb + 16 * hlf + 4 * quad + r;
+            const bool visible = key >= lo_row[rg] && key <= pos[rg] && key >= k_begin && key < k_end;
+            s_acc[rg][hlf][r] = visible ? s_acc[rg][hlf][r] : -INFINITY;
+          }
+    }
     bool moved = false;
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) {
@@ -338,24 +355,10 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
       // score inside the exponential's argument, as one multiply-add
       float sc[8];
       float mx = -INFINITY;
-      if (interior) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          sc[i] = s_acc[rg][i / 4][i % 4];
-          mx = fmaxf(mx, sc[i]);
-        }
-      } else {
-#pragma unroll
-        for (int hlf = 0; hlf < 2; ++hlf) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int key = kb + 16 * hlf + 4 * quad + r;
-            const bool visible = key >= lo_row[rg] && key <= pos[rg] && key >= k_begin && key < k_end;
-            const float v = visible ? s_acc[rg][hlf][r] : -INFINITY;
-            sc[hlf * 4 + r] = v;
-            mx = fmaxf(mx, v);
-          }
-        }
+      for (int i = 0; i < 8; ++i) {
+        sc[i] = s_acc[rg][i / 4][i % 4];
+        mx = fmaxf(mx, sc[i]);
       }
       if constexpr (SUM_ON_MATRIX_PIPE) {
         mx *= scale_log2;
@@ -377,8 +380,13 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
         const float m_safe = (m_run[rg] == -INFINITY) ? 0.f : m_run[rg];  // a row that has seen nothing yet
         // arguments are bounded above: the hardware exp2 is exact enough, tiny results flush to 0
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          p_reg[rg][i] = (bf16_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], scale_log2, -m_safe));
+        for (int i = 0; i < 8; i += 2) {  // (pairs: one conversion instruction for two)
+          const f32x2_t e = {__builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], scale_log2, -m_safe)),
+                             __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i + 1], scale_log2, -m_safe))};
+          const bf16x2_t b = __builtin_convertvector(e, bf16x2_t);
+          p_reg[rg][i] = b[0];
+          p_reg[rg][i + 1] = b[1];
+        }
       } else {
         mx = quad_max(mx) * scale_log2;
         // (the same lazy reference point; here every block agrees on the row's maximum)
