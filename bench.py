@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--sizes 8b|3b|70b]
                     [--max-context N] [--serving] [--reference-workload]
+                    [--long-context 8192,32768,131072] [--attention TOKENS]
 
 Default workload: the layer sizes of Llama 3.1 8B with random bfloat16 weights
 made on the device, a batch of 8 requests with 2,048-token uniform-random prompts,
@@ -282,6 +283,95 @@ def measure_attention(tokens: int, batch: int, repeats: int, sizes: dict) -> dic
     }
 
 
+LONG_DECODE_STEPS = 32
+LONG_WARMUP_STEPS = 8
+LONG_PORTION = 8192
+
+
+def measure_long_context(contexts: list[int], batch: int, dtype: str, sizes: str, layers: int | None) -> dict:
+    """Prefill and decode at long contexts: for each context length C, requests with prompts of
+    C - 40 tokens are prefilled in portions of 8,192 tokens (the first one is timed: tokens a
+    second over the whole prompt, share of the matrix peak) and then decoded 8 untimed and 32
+    timed steps, ending at C positions, once alone and once `batch` together."""
+    import numpy as np
+    import torch
+
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.sampling import sample_from_slots
+
+    model_name, full = SIZES[sizes]
+    cfg = dict(full)
+    cfg["num_hidden_layers"] = layers if layers is not None else full["num_hidden_layers"]
+    elem = 2 if dtype == "bfloat16" else 4
+    peak = PEAK_FLOPS["bf16" if dtype == "bfloat16" else "fp32"]
+    longest = max(contexts)
+    if longest > cfg["max_position_embeddings"]:
+        raise SystemExit(f"bench.py: context {longest} is beyond max_position_embeddings {cfg['max_position_embeddings']}")
+    runner = ModelRunner.from_random(
+        cfg, seed=0, dtype=dtype, num_blocks=batch * (-(-longest // BLOCK_SIZE)) + 8, block_size=BLOCK_SIZE, max_concurrent=batch
+    )
+    print(f"bench.py: {model_name} layer sizes, {cfg['num_hidden_layers']} layers, weights are on the device", file=sys.stderr, flush=True)
+    rng = np.random.default_rng(0)
+    # untimed: the first call of every kernel and library routine at this portion size
+    runner.step([StepEntry("warm", rng.integers(0, cfg["vocab_size"], size=LONG_PORTION).tolist(), [])])
+    runner.free_request("warm")
+    rows = []
+    for context in contexts:
+        prompt_len = context - LONG_WARMUP_STEPS - LONG_DECODE_STEPS
+        prefill_seconds = None
+        for live in sorted({1, batch}):
+            ids = [f"c{context}_{live}_{i}" for i in range(live)]
+            last = []
+            for rid in ids:
+                prompt = rng.integers(0, cfg["vocab_size"], size=prompt_len).tolist()
+                torch.cuda.synchronize()
+                started = time.perf_counter()
+                for at in range(0, prompt_len, LONG_PORTION):
+                    portion = prompt[at : at + LONG_PORTION]
+                    final = at + LONG_PORTION >= prompt_len
+                    logits = runner.step([StepEntry(rid, portion, [len(portion) - 1] if final else [])])
+                torch.cuda.synchronize()
+                seconds = time.perf_counter() - started
+                prefill_seconds = seconds if prefill_seconds is None else min(prefill_seconds, seconds)
+                last.append(int(sample_from_slots(logits, runner.last_row_slots, runner.cache.states.table).tolist()[0]))
+                print(f"bench.py: context {context}: prompt of {rid} in {seconds:.2f} s", file=sys.stderr, flush=True)
+            on_device = None
+            for k in range(LONG_WARMUP_STEPS + LONG_DECODE_STEPS):
+                if k == LONG_WARMUP_STEPS:
+                    torch.cuda.synchronize()
+                    started = time.perf_counter()
+                if on_device is None:
+                    entries = [StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, last)]
+                else:
+                    entries = [StepEntry(rid, [0], [0], device_row=row) for row, rid in enumerate(ids)]
+                logits = runner.step(entries, device_tokens=on_device)
+                on_device = sample_from_slots(logits, runner.last_row_slots, runner.cache.states.table)
+            torch.cuda.synchronize()
+            step = (time.perf_counter() - started) / LONG_DECODE_STEPS
+            mean_context = context - LONG_DECODE_STEPS / 2
+            step_bytes = weight_bytes(cfg, elem) + live * mean_context * kv_bytes_per_token(cfg, elem)
+            rows.append({
+                "context": context,
+                "batch": live,
+                "decode_tok_s": round(live / step, 2),
+                "ms_per_step": round(step * 1e3, 3),
+                "hbm_frac": round(step_bytes / step / 1e9 / PEAK_HBM_GBS, 4),
+                "prefill_tok_s": round(prompt_len / prefill_seconds, 1),
+                "prefill_s": round(prefill_seconds, 3),
+                "prefill_frac": round(prefill_flops(cfg, prompt_len) / prefill_seconds / peak, 4),
+            })
+            print(f"bench.py: {rows[-1]}", file=sys.stderr, flush=True)
+            for rid in ids:
+                runner.free_request(rid)
+    return {
+        "metric": f"long contexts, {model_name} layer sizes, prompts prefilled in portions of {LONG_PORTION}, {LONG_DECODE_STEPS} decode steps timed",
+        "dtype": "bf16" if dtype == "bfloat16" else "fp32",
+        "layers": cfg["num_hidden_layers"],
+        "layers_full_model": full["num_hidden_layers"],
+        "rows": rows,
+    }
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -310,6 +400,11 @@ def main() -> int:
         help="time the attention kernel alone instead: one prompt of TOKENS tokens, or with --attention-batch B one "
         "token of each of B requests over TOKENS keys; prints one JSON line and exits",
     )
+    parser.add_argument(
+        "--long-context", default=None, metavar="C1,C2,...",
+        help="instead of the default run: for each context length C, prompts of C-40 tokens prefilled in portions "
+        "of 8,192 and decoded to C positions, at batch 1 and at --batch; prints one JSON line and exits",
+    )
     parser.add_argument("--attention-batch", type=int, default=0)
     parser.add_argument("--attention-repeats", type=int, default=20)
     args = parser.parse_args()
@@ -319,6 +414,10 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.long_context is not None:
+        contexts = [int(c) for c in args.long_context.split(",")]
+        print(json.dumps(measure_long_context(contexts, args.batch, args.dtype, args.sizes, args.layers)), flush=True)
+        return 0
     room = args.max_context - PROMPT_LEN
     if args.steps <= 0 or args.warmup < 0 or args.steps + args.warmup > room:
         print(f"bench.py: --warmup + --steps must be at most {room} (decoding runs from {PROMPT_LEN} to at most "

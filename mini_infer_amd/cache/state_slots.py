@@ -12,8 +12,11 @@ admits and frees a request as a whole.  A slot is
     from there and advances the draw index itself, the first kernel of a step
     writes the positions.  The host copy is what the scheduler plans with; both
     are advanced by the same events, so they agree whenever the device is idle;
-  * one row in each state tensor a mixer asked for, `[max_requests, *shape]` per
-    layer call, zeroed when the slot is handed out (Llama asks for none).
+  * one row in each state tensor a mixer asked for, `[max_requests + 1, *shape]` per
+    layer call, zeroed when the slot is handed out (Llama asks for none).  The last
+    row belongs to no request: the padding rows of a recorded decode step carry slot
+    -1, which indexes it, so a mixer that reads and writes `state[slots]` with device
+    tensors alone needs no special case for them and can be recorded.
 """
 
 from __future__ import annotations
@@ -63,7 +66,7 @@ class StateSlots:
         if allocate_storage:
             self.table = torch.zeros((max_requests, SLOT_WORDS), dtype=torch.int32, device=device)
             for call, need in needs.items():
-                self.tensors[call] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
+                self.tensors[call] = torch.zeros((max_requests + 1, *need.shape), dtype=need.dtype, device=device)
 
     @property
     def num_free(self) -> int:

@@ -109,13 +109,22 @@ class DecodeGraph:
         assert at == self.total
 
     def capture(self) -> None:
-        """Run once outside a graph (library handles, workspaces), then record."""
+        """Run once outside a graph (library handles, workspaces), then record.
+
+        The run outside the graph must leave no trace, since the replay that follows does the
+        step's work again: keys and values land in the same places both times, and per-request
+        state is kept out of it by giving every row slot -1 (the state tensors' spare row)
+        for that run.
+        """
         model, caches = self.runner.model, self.runner._layer_caches
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             self.ctx.shared.clear()
+            slots = self.ctx.state_slots.clone()
+            self.ctx.state_slots.fill_(-1)
             model.forward(self.ctx, caches)
+            self.ctx.state_slots.copy_(slots)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.ctx.shared.clear()

@@ -150,7 +150,7 @@ def test_groups_are_formed_by_needs_and_calls_without_cache_have_none():
     caches = m.layer_caches()
     assert caches[0].k_pages.shape == (8, 2, 4, 16) and caches[2].k_pages.shape == (8, 1, 4, 32)
     assert caches[1].group is None and caches[1].k_pages is None
-    assert caches[3].state.shape == (2, 3) and caches[4].state.shape == (2, 2, 2) and caches[4].group is None
+    assert caches[3].state.shape == (3, 3) and caches[4].state.shape == (3, 2, 2) and caches[4].group is None
     assert caches[0].k_pages.data_ptr() != caches[3].k_pages.data_ptr()
 
 

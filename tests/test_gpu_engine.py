@@ -819,7 +819,7 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path, dtype):
         expected = {rid: plain(t) for rid, t in requests.items()}
         runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=24, block_size=4, max_concurrent=4)
         caches = runner.cache.layer_caches()
-        assert caches[1].state.shape == (4, hidden) and caches[1].k_pages is None and caches[0].state is None
+        assert caches[1].state.shape == (4 + 1, hidden) and caches[1].k_pages is None and caches[0].state is None
         got = ru.run_schedule(runner, requests, ru.schedule_mixed(requests, seed=4, tail=5))
         for rid in requests:
             ru.assert_close(got[rid], expected[rid], dtype, f"toy {rid}")
@@ -828,6 +828,123 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path, dtype):
     finally:
         ARCHITECTURES.unregister("ToyStateTestLM")
         MIXERS.unregister("decaying_sum")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_state_mixer_on_device_tensors_alone_is_recorded_and_replayed(tmp_path, dtype):
+    """The decaying sum once more, written with device tensors alone (no loop over the step's
+    requests on the host) and declared `graph_safe`: its single-token steps are recorded and
+    replayed like Llama's.  Three requests decode together in the bucket of four, so one row of
+    every replay is padding with slot -1 and must touch no request's state; the run that
+    precedes a recording must not advance the state either."""
+    import copy
+    import dataclasses
+
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.models.spec import LayerSpec
+    from mini_infer_amd.parts import CacheNeeds, Mixer, ParamSpec, StateNeeds
+    from mini_infer_amd.registry import ARCHITECTURES, MIXERS
+
+    hidden = tiny.TINY_A["hidden_size"]
+    decay = 0.75
+
+    class DecayingSumOnDevice(Mixer):
+        graph_safe = True
+
+        def param_specs(self, prefix):
+            return {prefix + "mix.weight": ParamSpec((hidden, hidden))}
+
+        def load_params(self, prefix, get):
+            self.weight = get(prefix + "mix.weight")
+
+        def cache_needs(self, page_size):
+            return CacheNeeds(state=StateNeeds((hidden,), torch.float32))
+
+        def forward(self, x, ctx, cache, writes_cache=True):
+            request = ctx.token_request.long()  # [T]
+            slots = ctx.state_slots.long()  # [B]; -1 (the spare row) for padding rows
+            at = torch.arange(x.shape[0], device=x.device)
+            starts = ctx.cu_seqlens_q.long()
+            distance = at[:, None] - at[None, :]
+            earlier_of_same_request = (request[:, None] == request[None, :]) & (distance >= 0)
+            weights = torch.where(earlier_of_same_request, decay ** distance.clamp(min=0).float(), 0.0)
+            carried = (decay ** (at - starts[request] + 1).float())[:, None] * cache.state[slots[request]]
+            states = weights @ x.float() + carried  # the state after each token
+            cache.state[slots] = states[starts[1:] - 1]
+            return (states @ self.weight.float().T).to(x.dtype)
+
+    MIXERS.register("decaying_sum_on_device", lambda desc, dtype_, device, shared=None: DecayingSumOnDevice(dtype_, device))
+
+    def with_toy(spec):
+        layers = list(spec.layers)
+        block = copy.deepcopy(layers[1].block)
+        block["mixer"] = {"kind": "decaying_sum_on_device"}
+        layers[1] = LayerSpec(layers[1].prefix, block)
+        return dataclasses.replace(spec, layers=layers)
+
+    _register_variant("ToyDeviceStateTestLM", with_toy)
+    try:
+        cfg = dict(tiny.TINY_A, architectures=["ToyDeviceStateTestLM"])
+        weights = tiny.make_weights(cfg, 63)
+        for n in "qkvo":
+            del weights[f"model.layers.1.self_attn.{n}_proj.weight"]
+        rng = np.random.default_rng(5)
+        weights["model.layers.1.self_attn.mix.weight"] = tiny.bf16_round(rng.standard_normal((hidden, hidden)) / 16)
+        folder = tiny.write_model_dir(tmp_path / "toy", cfg, weights)
+
+        def plain(tokens):
+            """Layer 0 as Llama's, layer 1 with the decaying sum (a loop over the tokens) in place of attention."""
+            eps = cfg["rms_norm_eps"]
+            r = pl.embedding(weights["model.embed_tokens.weight"], np.array(tokens))
+            cos, sin = pl.rope_tables(np.arange(len(tokens)), pl.config_inv_freq(cfg))
+            p = "model.layers.0."
+            a, _ = pl.attention_layer(
+                pl.rms_norm(r, weights[p + "input_layernorm.weight"], eps),
+                *(weights[p + f"self_attn.{n}_proj.weight"] for n in "qkvo"), cos, sin, 4, 2, 16)
+            r = r + a
+            r = r + pl.swiglu(pl.rms_norm(r, weights[p + "post_attention_layernorm.weight"], eps),
+                              *(weights[p + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            p = "model.layers.1."
+            h = pl.rms_norm(r, weights[p + "input_layernorm.weight"], eps)
+            if dtype == "bfloat16":
+                h = tiny.bf16_round(h).astype(np.float64)
+            state, mixed = np.zeros(hidden), []
+            for row in h:
+                state = decay * state + row
+                mixed.append(weights[p + "self_attn.mix.weight"].astype(np.float64) @ state)
+            r = r + np.array(mixed)
+            r = r + pl.swiglu(pl.rms_norm(r, weights[p + "post_attention_layernorm.weight"], eps),
+                              *(weights[p + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            return pl.rms_norm(r, weights["model.norm.weight"], eps) @ weights["model.embed_tokens.weight"].astype(np.float64).T
+
+        prompts, decoded = (13, 6, 9), 7
+        requests = {f"d{i}": tiny.random_tokens(cfg, n + decoded, seed=20 + i) for i, n in enumerate(prompts)}
+        expected = {rid: plain(t) for rid, t in requests.items()}
+        runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=24, block_size=4, max_concurrent=4)
+        assert runner.model.graph_safe and runner.decode_graphs is not None
+        got = {rid: [] for rid in requests}
+        # prompts: the first alone and in two portions, the other two together
+        runner.step([StepEntry("d0", requests["d0"][:5], [])])
+        got["d0"].append(runner.step([StepEntry("d0", requests["d0"][5:13], list(range(8)))]).cpu().numpy())
+        both = runner.step([StepEntry("d1", requests["d1"][:6], [5]), StepEntry("d2", requests["d2"][:9], [8])]).cpu().numpy()
+        got["d1"].append(both[:1])
+        got["d2"].append(both[1:])
+        for k in range(decoded):
+            entries = [StepEntry(rid, [requests[rid][n + k]], [0]) for rid, n in zip(requests, prompts)]
+            logits = runner.step(entries).cpu().numpy()
+            for row, rid in enumerate(requests):
+                got[rid].append(logits[row : row + 1])
+        assert runner.decode_graphs.replays == decoded and list(runner.decode_graphs.graphs) == [(4, 16)]
+        ru.assert_close(np.concatenate(got["d0"]), expected["d0"][5:], dtype, "toy on device d0")
+        ru.assert_close(np.concatenate(got["d1"]), expected["d1"][5:], dtype, "toy on device d1")
+        ru.assert_close(np.concatenate(got["d2"]), expected["d2"][8:], dtype, "toy on device d2")
+        for rid in requests:
+            runner.free_request(rid)
+        runner.cache.check()
+        assert runner.cache.states.num_free == 4
+    finally:
+        ARCHITECTURES.unregister("ToyDeviceStateTestLM")
+        MIXERS.unregister("decaying_sum_on_device")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
