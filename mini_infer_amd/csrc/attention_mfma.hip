@@ -76,8 +76,8 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   // immediates); PS == 0: any multiple of 16, divided by multiplying with
   // page_magic = floor(2^32 / page_size) + 1 (exact for keys below 2^32 / page_size).
   const int page_size = PS ? PS : page_size_arg;
-  auto page_index = [&](int key) -> int {
-    return PS ? key / PS : (int)__umulhi((unsigned)key, page_magic);
+  auto page_index = [&](int key) -> int {  // (keys are never negative: unsigned division is a shift)
+    return PS ? (int)((unsigned)key / (unsigned)(PS ? PS : 1)) : (int)__umulhi((unsigned)key, page_magic);
   };
   constexpr int DBLOCKS = D / 16;  // 16-dim blocks of the output
 
@@ -216,6 +216,9 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   const int k_begin = tile_lo + split * chunk;
   const int k_end = min(k_begin + chunk, tile_hi);
   const int* bt = block_table + (int64_t)req * max_blocks;
+  // 32-key blocks starting in [interior_first, interior_last] are seen whole by every row of this wave
+  const int interior_first = max(wave_lo_max, k_begin);
+  const int interior_last = min(wave_pos_min - 31, k_end - 32);
 
   // ---- Q^T operands: this lane's rows, 8 consecutive dims per k-step --------------
   bf16x8_t q_reg[RG][KSTEPS];
@@ -236,12 +239,20 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   constexpr int ACC_BLOCKS = DBLOCKS + (SUM_ON_MATRIX_PIPE ? 1 : 0);
   f32x4_t o_acc[RG][ACC_BLOCKS];
   float m_run[RG], l_run[RG];  // reference point of the exponentials (log2 units); sum of exp2(score - reference)
+  // Two values that follow m_run and change only when it does, so that a block whose maximum
+  // stays below the reference spends nothing on them: the addend of the exponentials'
+  // arguments (-m_run, or 0 while the row has seen nothing), and the RAW score (before the
+  // scale) above which the reference has to move.
+  float neg_ref[RG], raw_limit[RG];
+  const float inv_scale_log2 = 1.f / scale_log2;
 #pragma unroll
   for (int rg = 0; rg < RG; ++rg) {
 #pragma unroll
     for (int db = 0; db < ACC_BLOCKS; ++db) o_acc[rg][db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     m_run[rg] = -INFINITY;
     l_run[rg] = 0.f;
+    neg_ref[rg] = 0.f;
+    raw_limit[rg] = -INFINITY;
   }
   bf16x8_t ones;
 #pragma unroll
@@ -270,7 +281,8 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
 #pragma unroll
     for (int hlf = 0; hlf < 2; ++hlf) {
       // (past the table only for keys past the request's end, which are masked)
-      ids.page[hlf] = bt[min(page_index(kb + 16 * hlf), max_blocks - 1)];
+      const unsigned entry = (unsigned)min(page_index(kb + 16 * hlf), max_blocks - 1);
+      ids.page[hlf] = *reinterpret_cast<const int*>(reinterpret_cast<const char*>(bt) + entry * 4u);
     }
     return ids;
   };
@@ -335,7 +347,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     // a block every row of this wave sees whole needs no mask (most blocks of a long prompt);
     // elsewhere hidden scores become -inf where they lie, before anything reads them (one
     // branch for all row groups, and no second copy of the scores for the two ways to merge in)
-    const bool interior = kb >= wave_lo_max && kb + 31 <= wave_pos_min && kb >= k_begin && kb + 32 <= k_end;
+    const bool interior = kb >= interior_first && kb <= interior_last;
     if (!interior) {
 #pragma unroll
       for (int rg = 0; rg < RG; ++rg)
@@ -361,28 +373,28 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
         mx = fmaxf(mx, sc[i]);
       }
       if constexpr (SUM_ON_MATRIX_PIPE) {
-        mx *= scale_log2;
         // The reference point of the exponentials follows the running maximum lazily: it
         // moves only when the maximum grows by more than RESCALE_SLACK (in log2 units), so
         // probabilities stay below 2^RESCALE_SLACK and the accumulator is rarely rescaled.
-        // Each lane looks at its own 8 scores first; only if some lane of the wave finds
+        // Each lane looks at its own 8 raw scores first; only if some lane of the wave finds
         // one that far above the reference do the 4 lanes of a row agree on a maximum.
         alpha[rg] = 1.f;
-        if (__ballot(mx > m_run[rg] + RESCALE_SLACK) != 0ull) {
-          mx = quad_max(mx);
+        if (__ballot(mx > raw_limit[rg]) != 0ull) {
+          mx = quad_max(mx) * scale_log2;
           const float m_new = (mx > m_run[rg] + RESCALE_SLACK) ? mx : m_run[rg];
           // A row's first visible block moves the reference from -inf; its sums are still
           // zero, so nothing is to be rescaled (alpha 1, not exp2(-inf)).
           alpha[rg] = (m_run[rg] == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[rg] - m_new);
           m_run[rg] = m_new;
+          neg_ref[rg] = (m_new == -INFINITY) ? 0.f : -m_new;  // (0: a row that has seen nothing yet)
+          raw_limit[rg] = (m_new + RESCALE_SLACK) * inv_scale_log2;
           moved = moved || (__ballot(alpha[rg] != 1.f) != 0ull);
         }
-        const float m_safe = (m_run[rg] == -INFINITY) ? 0.f : m_run[rg];  // a row that has seen nothing yet
         // arguments are bounded above: the hardware exp2 is exact enough, tiny results flush to 0
 #pragma unroll
         for (int i = 0; i < 8; i += 2) {  // (pairs: one conversion instruction for two)
-          const f32x2_t e = {__builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], scale_log2, -m_safe)),
-                             __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i + 1], scale_log2, -m_safe))};
+          const f32x2_t e = {__builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], scale_log2, neg_ref[rg])),
+                             __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i + 1], scale_log2, neg_ref[rg]))};
           const bf16x2_t b = __builtin_convertvector(e, bf16x2_t);
           p_reg[rg][i] = b[0];
           p_reg[rg][i + 1] = b[1];
@@ -463,51 +475,65 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     const int tid = threadIdx.x;
     bf16x8_t k_stage[K_PER], v_stage[V_PER];
     // Which half of the tile (16 keys of one page) and which 16 bytes of it a thread fetches
-    // never changes: the offsets inside the half are made once, and the half is the same
+    // never changes: the byte offsets inside the half are made once, and the half is the same
     // for all lanes of a wave (a half's chunks are a multiple of 64), so the address of
-    // a load is a scalar base plus a fixed lane offset and costs no vector arithmetic.
-    // (Offsets from the kernel's own pointer arguments, not pointers picked from an array:
-    // those lose their address space, become flat loads, and flat loads are counted with
-    // the LDS reads, so that every wait for an operand read would wait for them too.)
+    // a load is a 64-bit scalar base (pages + page * bytes per page + head + first slot) plus
+    // a fixed 32-bit lane offset: the form a global load takes as it is, with no vector
+    // arithmetic, and with a handful of scalar instructions per tile.
+    // (Bases are made from the kernel's own pointer arguments, not picked from an array of
+    // pointers: those lose their address space, become flat loads, and flat loads are
+    // counted with the LDS reads, so that every wait for an operand read would wait for them.)
     static_assert((16 * CPR) % 64 == 0 && (2 * D) % 64 == 0, "a half's chunks fill whole waves");
+    constexpr bool K_HALF_KNOWN = (16 * CPR) % THREADS == 0;  // then (tid + j * THREADS) / (16 * CPR) is j's alone
+    constexpr bool V_HALF_KNOWN = (2 * D) % THREADS == 0;
     int k_half[K_PER], v_half[V_PER];
-    unsigned k_lane_off[K_PER], v_lane_off_tile[V_PER];
+    unsigned k_lane_byte[K_PER], v_lane_byte[V_PER];
 #pragma unroll
     for (int j = 0; j < K_PER; ++j) {
       const int id = tid + j * THREADS;
-      k_half[j] = __builtin_amdgcn_readfirstlane(id / (16 * CPR));
-      k_lane_off[j] = (unsigned)(id % (16 * CPR)) * 8u;  // a half's 16 key rows are contiguous
+      k_half[j] = K_HALF_KNOWN ? (j * THREADS) / (16 * CPR) : __builtin_amdgcn_readfirstlane(id / (16 * CPR));
+      k_lane_byte[j] = (unsigned)(id % (16 * CPR)) * 16u;  // a half's 16 key rows are contiguous
     }
 #pragma unroll
     for (int j = 0; j < V_PER; ++j) {
       const int id = tid + j * THREADS;
-      v_half[j] = __builtin_amdgcn_readfirstlane(id / (2 * D));
+      v_half[j] = V_HALF_KNOWN ? (j * THREADS) / (2 * D) : __builtin_amdgcn_readfirstlane(id / (2 * D));
       const int dim = (id % (2 * D)) / 2, part = id % 2;
-      v_lane_off_tile[j] = (unsigned)(dim * page_size + part * 8);
+      v_lane_byte[j] = (unsigned)(dim * page_size + part * 8) * 2u;
     }
+    const unsigned page_bytes = (unsigned)page_stride * 2u;
+    const char* const k_head = reinterpret_cast<const char*>(k_pages + head_off);
+    const char* const v_head = reinterpret_cast<const char*>(vt_pages + head_off);
     auto request_tile = [&](int kb, const PageIds& ids) {
-      int64_t k_off[2], v_off[2];  // elements from the start of the key and value pages
+      uint64_t k_base[2], v_base[2];
 #pragma unroll
       for (int hlf = 0; hlf < 2; ++hlf) {
         const int key0 = kb + 16 * hlf;
-        const int page = max(ids.page[hlf], 0);
-        const int64_t chunk_off = (int64_t)page * page_stride + head_off;
-        const int slot0 = key0 - page_index(key0) * page_size;
-        k_off[hlf] = chunk_off + (int64_t)slot0 * D;
-        v_off[hlf] = chunk_off + slot0;
+        const unsigned page = (unsigned)max(ids.page[hlf], 0);
+        // (tiles start at multiples of 32 keys: with pages of 16 a half is a whole page)
+        const unsigned slot0 = PS == 16 ? 0u : (unsigned)(key0 - page_index(key0) * page_size);
+        const uint64_t chunk = (uint64_t)page * page_bytes;
+        k_base[hlf] = reinterpret_cast<uint64_t>(k_head) + chunk + slot0 * (unsigned)(D * 2);
+        v_base[hlf] = reinterpret_cast<uint64_t>(v_head) + chunk + slot0 * 2u;
+        // (kept in scalar registers as they are: otherwise the lane offset is added to the
+        // heads once and the page product is redone per load on the vector pipe, in 64 bits)
+        asm("" : "+s"(k_base[hlf]));
+        asm("" : "+s"(v_base[hlf]));
       }
+      using global_bytes = const __attribute__((address_space(1))) char;
+      using global_chunk = const __attribute__((address_space(1))) bf16x8_t;
 #pragma unroll
       for (int j = 0; j < K_PER; ++j) {
         if (K_CHUNKS % THREADS == 0 || tid + j * THREADS < K_CHUNKS) {
-          const bf16_t* base = k_pages + (k_half[j] ? k_off[1] : k_off[0]);
-          k_stage[j] = *reinterpret_cast<const bf16x8_t*>(base + k_lane_off[j]);
+          global_bytes* base = reinterpret_cast<global_bytes*>(k_half[j] ? k_base[1] : k_base[0]);
+          k_stage[j] = *reinterpret_cast<global_chunk*>(base + k_lane_byte[j]);
         }
       }
 #pragma unroll
       for (int j = 0; j < V_PER; ++j) {
         if (V_CHUNKS % THREADS == 0 || tid + j * THREADS < V_CHUNKS) {
-          const bf16_t* base = vt_pages + (v_half[j] ? v_off[1] : v_off[0]);
-          v_stage[j] = *reinterpret_cast<const bf16x8_t*>(base + v_lane_off_tile[j]);
+          global_bytes* base = reinterpret_cast<global_bytes*>(v_half[j] ? v_base[1] : v_base[0]);
+          v_stage[j] = *reinterpret_cast<global_chunk*>(base + v_lane_byte[j]);
         }
       }
     };
