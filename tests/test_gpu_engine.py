@@ -1406,6 +1406,132 @@ def _long_case():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_block_arrangement_and_toy_norm_in_one_layer_of_two(tmp_path, dtype):
+    """Layer 0 is Llama's; layer 1 is described with a block kind and a norm kind defined here:
+    ONE norm (centred, with a bias: mean and variance instead of the mean square) whose output
+    feeds the attention and the feed-forward side by side, their sum going to the residual.  The
+    model is built layer by layer from the descriptions, loaded by tensor name (the toy norm's
+    bias included), stepped in portions and as recorded single tokens: no framework file changes."""
+    import copy
+    import dataclasses
+
+    from mini_infer_amd.engine import ModelRunner
+    from mini_infer_amd.models.spec import LayerSpec
+    from mini_infer_amd.parts import Block, Norm, ParamSpec
+    from mini_infer_amd.registry import ARCHITECTURES, BLOCKS, FEED_FORWARDS, MIXERS, NORMS
+
+    hidden = tiny.TINY_A["hidden_size"]
+    toy_eps = 3e-4
+
+    class CentredNorm(Norm):
+        graph_safe = True
+
+        def param_specs(self, prefix):
+            return {prefix + "weight": ParamSpec((hidden,), init="norm_weight"), prefix + "bias": ParamSpec((hidden,))}
+
+        def load_params(self, prefix, get):
+            self.weight, self.bias = get(prefix + "weight").float(), get(prefix + "bias").float()
+
+        def forward(self, delta, residual, rows=None):
+            if delta is not None:
+                residual += delta.float()
+            centred = residual - residual.mean(dim=-1, keepdim=True)
+            variance = (centred * centred).mean(dim=-1, keepdim=True)
+            return (centred * torch.rsqrt(variance + toy_eps) * self.weight + self.bias).to(self.dtype)
+
+    class SideBySide(Block):
+        def __init__(self, norm, mixer, feed_forward, dtype_, device):
+            super().__init__(dtype_, device)
+            self.norm, self.mixer, self.feed_forward = norm, mixer, feed_forward
+
+        @property
+        def graph_safe(self):
+            return self.norm.graph_safe and self.mixer.graph_safe and self.feed_forward.graph_safe
+
+        def _children(self):
+            return (("input_layernorm.", self.norm), ("self_attn.", self.mixer), ("mlp.", self.feed_forward))
+
+        def param_specs(self, prefix):
+            specs = {}
+            for sub, part in self._children():
+                specs.update(part.param_specs(prefix + sub))
+            return specs
+
+        def load_params(self, prefix, get):
+            for sub, part in self._children():
+                part.load_params(prefix + sub, get)
+
+        def forward(self, delta, residual, ctx, cache, writes_cache=True):
+            h = self.norm.forward(delta, residual)
+            return self.mixer.forward(h, ctx, cache, writes_cache) + self.feed_forward.forward(h, ctx)
+
+    NORMS.register("centred_norm", lambda desc, dtype_, device, shared=None: CentredNorm(dtype_, device))
+    BLOCKS.register(
+        "side_by_side",
+        lambda desc, dtype_, device, shared=None: SideBySide(
+            NORMS.lookup(desc["norm"]["kind"])(desc["norm"], dtype_, device, shared),
+            MIXERS.lookup(desc["mixer"]["kind"])(desc["mixer"], dtype_, device, shared),
+            FEED_FORWARDS.lookup(desc["feed_forward"]["kind"])(desc["feed_forward"], dtype_, device, shared),
+            dtype_, device,
+        ),
+    )
+
+    def with_toy(spec):
+        layers = list(spec.layers)
+        block = copy.deepcopy(layers[1].block)
+        block["kind"] = "side_by_side"
+        block["norm"] = {"kind": "centred_norm"}
+        layers[1] = LayerSpec(layers[1].prefix, block)
+        return dataclasses.replace(spec, layers=layers)
+
+    _register_variant("ToyBlockTestLM", with_toy)
+    try:
+        cfg = dict(tiny.TINY_A, architectures=["ToyBlockTestLM"])
+        weights = tiny.make_weights(cfg, 64)
+        del weights["model.layers.1.post_attention_layernorm.weight"]
+        rng = np.random.default_rng(6)
+        weights["model.layers.1.input_layernorm.bias"] = tiny.bf16_round(rng.standard_normal(hidden) / 4)
+        folder = tiny.write_model_dir(tmp_path / "toy", cfg, weights)
+
+        def plain(tokens):
+            eps = cfg["rms_norm_eps"]
+            w = {k: v.astype(np.float64) for k, v in weights.items()}
+            r = pl.embedding(weights["model.embed_tokens.weight"], np.array(tokens))
+            cos, sin = pl.rope_tables(np.arange(len(tokens)), pl.config_inv_freq(cfg))
+            p = "model.layers.0."
+            a, _ = pl.attention_layer(pl.rms_norm(r, w[p + "input_layernorm.weight"], eps),
+                                      *(w[p + f"self_attn.{n}_proj.weight"] for n in "qkvo"), cos, sin, 4, 2, 16)
+            r = r + a
+            r = r + pl.swiglu(pl.rms_norm(r, w[p + "post_attention_layernorm.weight"], eps),
+                              *(w[p + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            p = "model.layers.1."
+            centred = r - r.mean(axis=-1, keepdims=True)
+            h = centred / np.sqrt((centred * centred).mean(axis=-1, keepdims=True) + toy_eps)
+            h = h * w[p + "input_layernorm.weight"] + w[p + "input_layernorm.bias"]
+            if dtype == "bfloat16":
+                h = tiny.bf16_round(h).astype(np.float64)
+            a, _ = pl.attention_layer(h, *(w[p + f"self_attn.{n}_proj.weight"] for n in "qkvo"), cos, sin, 4, 2, 16)
+            r = r + a + pl.swiglu(h, *(w[p + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+            return pl.rms_norm(r, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T
+
+        requests = {f"s{i}": tiny.random_tokens(cfg, n, seed=40 + i) for i, n in enumerate((26, 11, 19))}
+        expected = {rid: plain(t) for rid, t in requests.items()}
+        runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=24, block_size=4, max_concurrent=3)
+        assert type(runner.model.blocks[1]).__name__ == "SideBySide" and type(runner.model.blocks[0]).__name__ == "PreNormBlock"
+        assert runner.model.graph_safe and runner.decode_graphs is not None
+        got = ru.run_schedule(runner, requests, ru.schedule_mixed(requests, seed=8, max_live=3, tail=6))
+        for rid in requests:
+            ru.assert_close(got[rid], expected[rid], dtype, f"toy block {rid}")
+        assert runner.decode_graphs.replays > 0
+        runner.cache.check()
+        assert runner.num_free_blocks() == 24
+    finally:
+        ARCHITECTURES.unregister("ToyBlockTestLM")
+        BLOCKS.unregister("side_by_side")
+        NORMS.unregister("centred_norm")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_context_past_eight_thousand_keys(tmp_path, dtype):
     """8,288 tokens in portions of 2,048, then 12 tokens one by one, where single tokens'
     keys are cut into the many ranges of long contexts.  (In float32 a page read from the
