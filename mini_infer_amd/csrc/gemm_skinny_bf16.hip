@@ -39,14 +39,26 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 //              head's first half and their partners, rotates them, and writes queries
 //              to c[m, q_heads*head_dim] and keys and values straight into their cache
 //              slots.
+//   EPI_ADDNORM  the product is a layer's contribution to the residual stream and the next
+//              thing to happen is an RMS norm: residual += bf16(product) (float32, stored), and
+//              c = bf16(residual * norm_weight), the norm's output but for the row's factor
+//              rsqrt(mean(residual^2) + eps).  That factor needs the whole row, which no block
+//              has: every block leaves the sum of squares of its features per row in
+//              sumsq[block][row], and the product that consumes c (PRO_SCALED) adds them up
+//              and multiplies its own sums with the factor, which commutes with the product.
+//              The norm's launch between two products is saved.
 // In every case the sums are rounded to bfloat16 before the activation or rotation,
 // exactly as when the product and the second step run as two kernels.
-enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2 };
+enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2, EPI_ADDNORM = 3 };
 // Where the activations come from: a matrix in memory, or (PRO_ATTN, few rows) the
 // uncombined key ranges of attn_mfma: each wave first combines its own columns of the
 // attention output (what attn_reduce would have written) into LDS, so the combining launch
 // between the attention and its output projection is saved at the smallest batches.
-enum { PRO_NONE = 0, PRO_ATTN = 1 };
+// PRO_SCALED: rows whose norm factor is still apart (what EPI_ADDNORM leaves): the sums are
+// multiplied with rsqrt(sum of the pieces' squares / width + eps) of their row before rounding.
+enum { PRO_NONE = 0, PRO_ATTN = 1, PRO_SCALED = 2 };
+#define SK_SCALE_PARTS 32  // threads per row that add up the pieces of a row's sum of squares
+#define SK_SCALE_PIECES 8  // pieces per such thread: 256 pieces at most
 #define SK_PRO_VALUES 4096  // activations a wave makes and holds: rows * (K / 8 waves) at most
 
 struct RopeArgs {  // EPI_ROPE only
@@ -61,6 +73,17 @@ struct RopeArgs {  // EPI_ROPE only
   const float* part_acc;
   const float* part_ml;
   int num_splits, attn_heads, attn_head_dim;
+  // EPI_ADDNORM: the float32 residual rows [m, n] the product is added to, the norm's weight [n],
+  // where the block's sums of squares go ([blocks][m])
+  float* residual;
+  int64_t ld_residual;
+  const bf16_t* norm_weight;
+  float* sumsq_out;
+  // PRO_SCALED: the pieces of the rows' sums of squares [pieces][m], the norm's eps and width
+  const float* sumsq_in;
+  int sumsq_pieces;
+  float norm_eps;
+  int norm_width;
 };
 
 template <int NT, int U, int EPI, int PRO = PRO_NONE>
@@ -69,6 +92,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     bf16_t* __restrict__ c, int64_t ldc, int m, int n, int k, int features_per_block, const RopeArgs rope) {
   constexpr bool GATED = EPI == EPI_GATED;
   constexpr bool ROPE = EPI == EPI_ROPE;
+  constexpr bool ADDNORM = EPI == EPI_ADDNORM;
+  constexpr bool SCALED = PRO == PRO_SCALED;
   static_assert(!ROPE || NT == 1, "the rotary epilogue takes one tile of dims and its partner tile");
   constexpr int WT = (GATED || ROPE) ? 2 * NT : NT;  // weight tiles per block
   __shared__ float red[SK_WAVES][WT][256];
@@ -168,6 +193,25 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   }
   const bf16_t* own = &a_own[PRO == PRO_ATTN ? wave : 0][(PRO == PRO_ATTN ? min(col, m - 1) * own_stride : 0) + quad * 8];
 
+  __shared__ float scale_part[SCALED ? SK_SCALE_PARTS : 1][16];
+  // EPI_ADDNORM: the residual values and norm weights of the thread's four outputs, asked for
+  // now, so that the last step does not begin with a trip to memory
+  f32x4_t res_old = {0.f, 0.f, 0.f, 0.f};
+  float norm_w4[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (ADDNORM) {
+    const int item = threadIdx.x;
+    const int token = (item % 64) % 16, feature = n0 + (item / 64) * 16 + ((item % 64) / 16) * 4;
+    if (item < NT * 64 && token < m) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (feature + r < n_end) {
+          res_old[r] = rope.residual[(int64_t)token * rope.ld_residual + feature + r];
+          norm_w4[r] = (float)rope.norm_weight[feature + r];
+        }
+      }
+    }
+  }
+
   f32x4_t acc[WT];
 #pragma unroll
   for (int t = 0; t < WT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
@@ -202,12 +246,31 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     }
   }
 
+  // PRO_SCALED: SK_SCALE_PARTS threads per row each add up every SK_SCALE_PARTS-th piece of the
+  // row's sum of squares, in a fixed order.  Asked for only now: held through the loop above
+  // they would cost the registers of a resident block per CU (measured: 16 % slower).
+  float scale_piece[SCALED ? SK_SCALE_PIECES : 1];
+  if constexpr (SCALED) {
+    const int row = threadIdx.x % 16, part = threadIdx.x / 16;
+#pragma unroll
+    for (int i = 0; i < SK_SCALE_PIECES; ++i) {
+      const int piece = part + i * SK_SCALE_PARTS;
+      scale_piece[i] = (row < m && piece < rope.sumsq_pieces) ? rope.sumsq_in[(int64_t)piece * m + row] : 0.f;
+    }
+  }
   // acc[t][r] = C^T[feature n0 + 16*(t % NT) + 4*quad + r][token col]; add the 8 waves in order
 #pragma unroll
   for (int t = 0; t < WT; ++t) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][t][(quad * 4 + r) * 16 + col] = acc[t][r];
   }
+  if constexpr (SCALED) {
+    float scale_mine = 0.f;
+#pragma unroll
+    for (int i = 0; i < SK_SCALE_PIECES; ++i) scale_mine += scale_piece[i];
+    scale_part[threadIdx.x / 16][threadIdx.x % 16] = scale_mine;
+  }
+  __shared__ float squares[ADDNORM ? NT * 4 : 1][16];  // EPI_ADDNORM: per (4 features, row) of the block
   __syncthreads();
   // 256*NT outputs, each a sum of 8 (two such when gated): a thread takes 4 consecutive
   // features of one token
@@ -228,12 +291,40 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) up[r] += red[wv][NT + nt][(fq * 4 + r) * 16 + token];
     }
+    if constexpr (SCALED) {
+      float total = 0.f;
+#pragma unroll
+      for (int part = 0; part < SK_SCALE_PARTS; ++part) total += scale_part[part][token];
+      const float inv = rsqrtf(total / (float)rope.norm_width + rope.norm_eps);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        sum[r] *= inv;
+        up[r] *= inv;
+      }
+    }
     if (GATED) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float g = (float)(bf16_t)sum[r];
         sum[r] = g / (1.f + expf(-g)) * (float)(bf16_t)up[r];
       }
+    }
+    if constexpr (ADDNORM) {
+      const int feature = n0 + nt * 16 + fq * 4;
+      float* res = rope.residual + (int64_t)token * rope.ld_residual + feature;
+      bf16_t* dst = c + (int64_t)token * ldc + feature;
+      float sq = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (feature + r < n_end) {  // (rows past n_end repeat the last feature: not counted twice)
+          const float x = res_old[r] + (float)(bf16_t)sum[r];
+          res[r] = x;
+          dst[r] = (bf16_t)(x * norm_w4[r]);
+          sq += x * x;
+        }
+      }
+      squares[nt * 4 + fq][token] = sq;
+      continue;
     }
     if (ROPE) {
       // this thread: four consecutive pairs (never across a head: half is a multiple of 4), one token
@@ -301,6 +392,15 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         if (feature + r < n_end) dst[r] = (bf16_t)sum[r];
+    }
+  }
+  if constexpr (ADDNORM) {
+    __syncthreads();
+    if (threadIdx.x < m) {
+      float total = 0.f;
+#pragma unroll
+      for (int i = 0; i < NT * 4; ++i) total += squares[i][threadIdx.x];
+      rope.sumsq_out[(int64_t)blockIdx.x * m + threadIdx.x] = total;
     }
   }
 }
@@ -405,6 +505,105 @@ extern "C" int mi_gemm_skinny_attn_bf16(const float* part_acc, const float* part
     default: gemm_skinny_bf16_kernel<4, 2, EPI_STORE, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args); break;
   }
   MI_CHECK_LAUNCH("gemm_skinny_attn_bf16");
+  return MI_OK;
+}
+
+// The product as a layer's contribution to the residual stream, with the following RMS norm but
+// for its row factor (EPI_ADDNORM): residual[m, n] += bf16(a . w^T); values[m, n] =
+// bf16(residual * norm_weight); sumsq[pieces][m] = each block's sums of squares, where
+// pieces = mi_gemm_skinny_addnorm_pieces(n).  With part_acc the activations are the
+// uncombined key ranges of attn_mfma (as in mi_gemm_skinny_attn_bf16; a, lda unused).
+extern "C" int mi_gemm_skinny_addnorm_pieces(int n) {
+  const int cus = compute_units();
+  if (cus <= 0 || n < 1) return 0;
+  return ceil_div(n, features_per_block_for(n, cus, 4));
+}
+
+extern "C" int mi_gemm_skinny_addnorm_bf16(const void* a, int64_t lda, const float* part_acc, const float* part_ml,
+                                           int num_splits, int heads, int head_dim, const void* w, int64_t ldw,
+                                           float* residual, int64_t ld_residual, const void* norm_weight,
+                                           void* values, int64_t ldv, float* sumsq, int m, int n, int k,
+                                           hipStream_t stream) {
+  const bool from_attention = part_acc != nullptr;
+  if (from_attention) {
+    MI_REQUIRE(part_ml && num_splits >= 1 && num_splits <= 64 && heads * head_dim == k,
+               "gemm_skinny_addnorm_bf16: needs the partial buffers of 1..64 key ranges over k = heads*head_dim; "
+               "got splits=%d heads=%d head_dim=%d k=%d", num_splits, heads, head_dim, k);
+    MI_REQUIRE(mi_gemm_skinny_attn_bf16_supported(m, heads, head_dim) && ldw % 8 == 0,
+               "gemm_skinny_addnorm_bf16: rows x (heads*head_dim / 8) must be at most %d, head_dim a multiple of 32; "
+               "got m=%d heads=%d head_dim=%d", SK_PRO_VALUES, m, heads, head_dim);
+  } else {
+    MI_REQUIRE(mi_gemm_skinny_bf16_supported(m, n, k, lda, ldw) && lda >= k,
+               "gemm_skinny_addnorm_bf16: takes 1 <= m <= 16, k a multiple of 32, rows aligned to 16 bytes; "
+               "got m=%d n=%d k=%d lda=%lld ldw=%lld", m, n, k, (long long)lda, (long long)ldw);
+  }
+  MI_REQUIRE(n >= 1 && ldw >= k && ldv >= n && ld_residual >= n, "gemm_skinny_addnorm_bf16: a row stride is shorter than its row");
+  MI_REQUIRE(residual && norm_weight && values && sumsq, "gemm_skinny_addnorm_bf16: needs residual, norm weight and both outputs");
+  RopeArgs args = {};
+  args.part_acc = part_acc;
+  args.part_ml = part_ml;
+  args.num_splits = num_splits;
+  args.attn_heads = heads;
+  args.attn_head_dim = head_dim;
+  args.residual = residual;
+  args.ld_residual = ld_residual;
+  args.norm_weight = (const bf16_t*)norm_weight;
+  args.sumsq_out = sumsq;
+  const bf16_t* wp = (const bf16_t*)w;
+  const bf16_t* ap = from_attention ? wp : (const bf16_t*)a;  // (never read when the activations are made in the kernel)
+  if (from_attention) lda = ldw;
+  bf16_t* cp = (bf16_t*)values;
+  const int cus = compute_units();
+  MI_REQUIRE(cus > 0, "gemm_skinny_addnorm_bf16: cannot read the device's compute unit count");
+  const int fpb = features_per_block_for(n, cus, 4);
+  const int blocks = ceil_div(n, fpb);
+  const int threads = 64 * SK_WAVES;
+#define SK_ADDNORM(NT_, U_)                                                                                        \
+  if (from_attention)                                                                                              \
+    gemm_skinny_bf16_kernel<NT_, U_, EPI_ADDNORM, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldv, m, n, k, fpb, args); \
+  else                                                                                                             \
+    gemm_skinny_bf16_kernel<NT_, U_, EPI_ADDNORM><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldv, m, n, k, fpb, args)
+  switch (ceil_div(fpb, 16)) {
+    case 1: SK_ADDNORM(1, 8); break;
+    case 2: SK_ADDNORM(2, 8); break;
+    case 3: SK_ADDNORM(3, 4); break;
+    default: SK_ADDNORM(4, 2); break;
+  }
+#undef SK_ADDNORM
+  MI_CHECK_LAUNCH("gemm_skinny_addnorm_bf16");
+  return MI_OK;
+}
+
+// The gated product on rows whose norm factor is still apart (PRO_SCALED): a = the values of
+// mi_gemm_skinny_addnorm_bf16, sumsq[pieces][m] its sums of squares; out[m, n] =
+// silu(f * a . gate^T) * (f * a . up^T) with f = rsqrt(sum of the row's pieces / k + eps).
+extern "C" int mi_gemm_skinny_swiglu_scaled_bf16(const void* a, int64_t lda, const float* sumsq, int pieces, float eps,
+                                                 const void* w, int64_t ldw, void* out, int64_t ldo, int m, int n,
+                                                 int k, hipStream_t stream) {
+  MI_REQUIRE(mi_gemm_skinny_bf16_supported(m, n, k, lda, ldw),
+             "gemm_skinny_swiglu_scaled_bf16: takes 1 <= m <= 16, k a multiple of 32, rows aligned to 16 bytes; "
+             "got m=%d n=%d k=%d lda=%lld ldw=%lld", m, n, k, (long long)lda, (long long)ldw);
+  MI_REQUIRE(lda >= k && ldw >= k && ldo >= n, "gemm_skinny_swiglu_scaled_bf16: a row stride is shorter than its row");
+  MI_REQUIRE(sumsq && pieces >= 1 && pieces <= SK_SCALE_PARTS * SK_SCALE_PIECES && eps >= 0.f,
+             "gemm_skinny_swiglu_scaled_bf16: needs the rows' sums of squares in 1..%d pieces, got %d",
+             SK_SCALE_PARTS * SK_SCALE_PIECES, pieces);
+  RopeArgs args = {};
+  args.sumsq_in = sumsq;
+  args.sumsq_pieces = pieces;
+  args.norm_eps = eps;
+  args.norm_width = k;
+  const int cus = compute_units();
+  MI_REQUIRE(cus > 0, "gemm_skinny_swiglu_scaled_bf16: cannot read the device's compute unit count");
+  const int fpb = features_per_block_for(n, cus, 2);
+  const int blocks = ceil_div(n, fpb);
+  const int threads = 64 * SK_WAVES;
+  if (fpb <= 16)
+    gemm_skinny_bf16_kernel<1, 4, EPI_GATED, PRO_SCALED><<<blocks, threads, 0, stream>>>(
+        (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)out, ldo, m, n, k, fpb, args);
+  else
+    gemm_skinny_bf16_kernel<2, 2, EPI_GATED, PRO_SCALED><<<blocks, threads, 0, stream>>>(
+        (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)out, ldo, m, n, k, fpb, args);
+  MI_CHECK_LAUNCH("gemm_skinny_swiglu_scaled_bf16");
   return MI_OK;
 }
 

@@ -542,17 +542,35 @@ def qkv_rope_write(
     return q_out
 
 
-def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+def linear_swiglu(x: "torch.Tensor | ScaledRows", gate_up_weight: torch.Tensor) -> torch.Tensor:
     """`silu(x @ gate.T) * (x @ up.T)` with `gate_up_weight` = [gate; up] stacked, [2I, K].
 
     bfloat16 with at most 16 rows runs as ONE hand-written kernel (the product with the
     activation in its last step); otherwise the product and `silu_mul` run in turn.
     Both ways round the two products to the element type before the activation, so a
-    token's result does not depend on which one ran.
+    token's result does not depend on which one ran.  `x` may be `ScaledRows`: the rows'
+    factors are then applied to the sums of the two products (the same kernel with one
+    more step), or to `x` first where that kernel does not take the shapes.
     """
     rows, width = gate_up_weight.shape
     if rows % 2:
         raise KernelShapeError(f"linear_swiglu: stacked weight has an odd number of rows ({rows})")
+    scaled = None
+    if isinstance(x, ScaledRows):
+        values = x.values
+        if (
+            values.dtype == torch.bfloat16
+            and gate_up_weight.dtype == torch.bfloat16
+            and values.shape[1] == width
+            and values.stride(1) == 1
+            and gate_up_weight.stride(1) == 1
+            and x.sumsq.is_contiguous()
+            and x.sumsq.shape[0] <= SCALED_ROWS_MAX_PIECES
+            and skinny_gemm_takes(values.shape[0], width, values.stride(0), gate_up_weight.stride(0))
+        ):
+            scaled, x = x, values
+        else:
+            x = x.finish()
     if (
         x.dtype == torch.bfloat16
         and gate_up_weight.dtype == torch.bfloat16
@@ -566,6 +584,15 @@ def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor
         m, n = x.shape[0], rows // 2
         out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
         lib = library.load()
+        if scaled is not None:
+            _need_cuda(scaled.sumsq)
+            library.check(
+                lib.mi_gemm_skinny_swiglu_scaled_bf16(
+                    _ptr(x), x.stride(0), _ptr(scaled.sumsq), scaled.sumsq.shape[0], scaled.eps,
+                    _ptr(gate_up_weight), gate_up_weight.stride(0), _ptr(out), out.stride(0), m, n, width, _stream(),
+                )
+            )
+            return out
         library.check(
             lib.mi_gemm_skinny_swiglu_bf16(
                 _ptr(x), x.stride(0), _ptr(gate_up_weight), gate_up_weight.stride(0), _ptr(out), out.stride(0),
@@ -649,6 +676,113 @@ def linear_from_attention(pieces: AttentionPieces, weight: torch.Tensor) -> torc
         )
     )
     return out
+
+
+PENDING_PRODUCT_MAX_ROWS = 16  # rows up to which a product is worth handing on unmade
+SCALED_ROWS_MAX_PIECES = 256  # pieces of a row's sum of squares the consuming kernel adds up
+
+
+@dataclasses.dataclass
+class PendingProduct:
+    """`x @ weight.T` that has not been made yet: a part's contribution to the residual stream,
+    handed to the norm that follows it so that one kernel can make the product, add it to the
+    residual and begin the norm (`linear_add_norm`).  `x` is a matrix, or an attention output
+    still lying in its key ranges.  Anything else calls `finish()`."""
+
+    x: torch.Tensor | AttentionPieces
+    weight: torch.Tensor
+
+    def finish(self) -> torch.Tensor:
+        if isinstance(self.x, AttentionPieces):
+            return linear_from_attention(self.x, self.weight)
+        return linear(self.x, self.weight)
+
+
+@dataclasses.dataclass
+class ScaledRows:
+    """The output of an RMS norm but for each row's factor: `values` [T, H] = residual * norm
+    weight (rounded to the element type), `sumsq` [pieces, T] float32 = sums of squares of
+    the residual rows over `pieces` ranges of H.  Row t is still to be multiplied with
+    rsqrt(sum(sumsq[:, t]) / H + eps); a product that consumes the rows does that to its own
+    sums instead (`linear_swiglu`), since the factor commutes with the product.  Anything
+    else calls `finish()`."""
+
+    values: torch.Tensor
+    sumsq: torch.Tensor
+    eps: float
+
+    def finish(self) -> torch.Tensor:
+        factor = torch.rsqrt(self.sumsq.sum(dim=0) / self.values.shape[1] + self.eps)
+        return (self.values.float() * factor[:, None]).to(self.values.dtype)
+
+
+def linear_add_norm_takes(pending: PendingProduct, residual: torch.Tensor, norm_weight: torch.Tensor) -> bool:
+    """Whether `linear_add_norm` runs as one kernel: bfloat16, at most 16 rows, K a multiple
+    of 32 (from key ranges: what `linear_from_attention` takes)."""
+    weight = pending.weight
+    if (
+        weight.dtype != torch.bfloat16
+        or norm_weight.dtype != torch.bfloat16
+        or weight.dim() != 2
+        or weight.stride(1) != 1
+        or residual.dtype != torch.float32
+        or not residual.is_cuda
+        or not residual.is_contiguous()
+        or tuple(norm_weight.shape) != (weight.shape[0],)
+    ):
+        return False
+    x = pending.x
+    if isinstance(x, AttentionPieces):
+        return (
+            x.dtype == torch.bfloat16
+            and x.heads * x.head_dim == weight.shape[1]
+            and tuple(residual.shape) == (x.tokens, weight.shape[0])
+            and weight.stride(0) % 8 == 0
+            and bool(library.load().mi_gemm_skinny_attn_bf16_supported(x.tokens, x.heads, x.head_dim))
+        )
+    return (
+        x.dtype == torch.bfloat16
+        and x.dim() == 2
+        and x.stride(1) == 1
+        and x.shape[1] == weight.shape[1]
+        and tuple(residual.shape) == (x.shape[0], weight.shape[0])
+        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), weight.stride(0))
+    )
+
+
+def linear_add_norm(pending: PendingProduct, residual: torch.Tensor, norm_weight: torch.Tensor, eps: float) -> ScaledRows:
+    """`residual += x @ weight.T` (rounded to bfloat16 first, added in float32, kept) and the
+    RMS norm of the sum but for the rows' factors, in one kernel (see `ScaledRows`)."""
+    if not linear_add_norm_takes(pending, residual, norm_weight):
+        raise KernelShapeError(
+            "linear_add_norm takes bfloat16, at most 16 rows, K a multiple of 32, a float32 residual [rows, N] "
+            f"and a norm weight [N]; got weight {tuple(pending.weight.shape)} {pending.weight.dtype}, "
+            f"residual {tuple(residual.shape)} {residual.dtype}"
+        )
+    weight, x = pending.weight, pending.x
+    _need_cuda(weight, residual, norm_weight)
+    _need_contiguous("norm weight", norm_weight)
+    rows, n = residual.shape
+    k = weight.shape[1]
+    lib = library.load()
+    pieces = lib.mi_gemm_skinny_addnorm_pieces(n)
+    if pieces <= 0:
+        raise KernelShapeError(f"linear_add_norm: no block count for {n} features")
+    values = torch.empty((rows, n), dtype=torch.bfloat16, device=residual.device)
+    sumsq = torch.empty((pieces, rows), dtype=torch.float32, device=residual.device)
+    if isinstance(x, AttentionPieces):
+        _need_cuda(x.part_acc, x.part_ml)
+        source = (None, 0, _ptr(x.part_acc), _ptr(x.part_ml), x.splits, x.heads, x.head_dim)
+    else:
+        _need_cuda(x)
+        source = (_ptr(x), x.stride(0), None, None, 0, 0, 0)
+    library.check(
+        lib.mi_gemm_skinny_addnorm_bf16(
+            *source, _ptr(weight), weight.stride(0), _ptr(residual), residual.stride(0), _ptr(norm_weight),
+            _ptr(values), values.stride(0), _ptr(sumsq), rows, n, k, _stream(),
+        )
+    )
+    return ScaledRows(values, sumsq, float(eps))
 
 
 def paged_attention(

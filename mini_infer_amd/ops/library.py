@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -52,6 +52,11 @@ _SIGNATURES: dict[str, list] = {
         _P, c_int64, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, _P, c_int64, _P, _P, c_int,
         c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, _P,
     ],
+    "mi_gemm_skinny_addnorm_pieces": [c_int],
+    "mi_gemm_skinny_addnorm_bf16": [
+        _P, c_int64, _P, _P, c_int, c_int, c_int, _P, c_int64, _P, c_int64, _P, _P, c_int64, _P, c_int, c_int, c_int, _P,
+    ],
+    "mi_gemm_skinny_swiglu_scaled_bf16": [_P, c_int64, _P, c_int, c_float, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_attn_mfma_tokens_per_tile": [c_int, c_int, c_int],
     "mi_attn_mfma_supported": [c_int, c_int],
     "mi_sample": [c_int, _P, c_int64, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P],

@@ -31,6 +31,7 @@ from mini_infer_amd.registry import POSITION_ENCODINGS, register_mixer
 
 class GQAttention(Mixer):
     graph_safe = True
+    can_defer_output = True
 
     def __init__(
         self,
@@ -126,9 +127,14 @@ class GQAttention(Mixer):
         return self._project(self._attend(qkv, ctx, cache))
 
     def _project(self, attended):
-        """The output projection of what `_attend` returned."""
+        """The output projection of what `_attend` returned; for few rows, where the block
+        asked for it, not made here but handed on to the norm that follows."""
+        assert self.out.weight is not None
+        if self.emit_pending_output and self.dtype == torch.bfloat16:
+            rows = attended.tokens if isinstance(attended, ops.AttentionPieces) else attended.shape[0]
+            if rows <= ops.PENDING_PRODUCT_MAX_ROWS:
+                return ops.PendingProduct(attended, self.out.weight)
         if isinstance(attended, ops.AttentionPieces):
-            assert self.out.weight is not None
             return ops.linear_from_attention(attended, self.out.weight)
         return self.out.forward(attended, partial_ok=self.emit_partial_sums)
 

@@ -168,9 +168,17 @@ class Norm(Part):
     `takes_partial_sums`: `delta` may also be an `ops.PartialSums` (a product whose sums
     over ranges of K are still apart); a model lets its mixers and feed-forwards emit
     those only if every one of its norms says it takes them.
+
+    `takes_pending_products`: `delta` may also be an `ops.PendingProduct` (a product not made
+    yet); and where the block has set `emit_scaled_rows` on the norm, because the part that
+    consumes its output says `takes_scaled_rows`, the norm may return `ops.ScaledRows`
+    (its output but for the rows' factors) instead of a tensor.  Both are a block's own
+    arrangement between its parts: a norm that knows neither is fine.
     """
 
     takes_partial_sums = False
+    takes_pending_products = False
+    emit_scaled_rows = False
 
     def forward(
         self,
@@ -218,9 +226,14 @@ class Mixer(Part):
     """Mixes tokens of one request: attention here, anything with a cache or a state.
 
     `emit_partial_sums` is set by the model, never by the part: when true, `forward` may
-    return an `ops.PartialSums` instead of a tensor (parts that ignore it are fine)."""
+    return an `ops.PartialSums` instead of a tensor (parts that ignore it are fine).
+    `emit_pending_output` is set by the block where the norm that follows says
+    `takes_pending_products` and the mixer `can_defer_output`: `forward` may then return an
+    `ops.PendingProduct` (its last product, not made yet) instead of a tensor."""
 
     emit_partial_sums = False
+    can_defer_output = False
+    emit_pending_output = False
 
     def cache_needs(self, page_size: int) -> CacheNeeds:
         """What the cache manager must keep for one call of this mixer, given its page size
@@ -234,9 +247,12 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """Acts on each token alone: dense or routed experts.  `emit_partial_sums`: as for `Mixer`."""
+    """Acts on each token alone: dense or routed experts.  `emit_partial_sums`: as for `Mixer`.
+    `takes_scaled_rows`: `x` may be an `ops.ScaledRows` (a norm's output but for the rows'
+    factors)."""
 
     emit_partial_sums = False
+    takes_scaled_rows = False
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError

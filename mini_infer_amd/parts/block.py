@@ -40,6 +40,12 @@ class PreNormBlock(Block):
         self.ffn_norm = ffn_norm
         self.feed_forward = feed_forward
         self.names = names  # part -> its prefix inside the layer, e.g. "self_attn."
+        # Where all three say they can, the mixer leaves its last product to the norm that
+        # follows, and that norm leaves the rows' factors to the feed-forward's first product:
+        # for few rows one launch between two weight-streaming products is saved.
+        if mixer.can_defer_output and ffn_norm.takes_pending_products and feed_forward.takes_scaled_rows:
+            mixer.emit_pending_output = True
+            ffn_norm.emit_scaled_rows = True
 
     @property
     def graph_safe(self) -> bool:  # type: ignore[override]

@@ -19,6 +19,7 @@ from mini_infer_amd.registry import register_feed_forward
 
 class SwiGLU(FeedForward):
     graph_safe = True
+    takes_scaled_rows = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, dtype: torch.dtype, device) -> None:
         super().__init__(dtype, device)
@@ -36,7 +37,7 @@ class SwiGLU(FeedForward):
         self.gate_up.load_params(prefix, get)
         self.down.load_params(prefix, get)
 
-    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+    def forward(self, x: "torch.Tensor | ops.ScaledRows", ctx: StepContext) -> torch.Tensor:
         assert self.gate_up.weight is not None, "SwiGLU used before its weights were loaded"
         return self.down.forward(ops.linear_swiglu(x, self.gate_up.weight), partial_ok=self.emit_partial_sums)
 

@@ -18,6 +18,7 @@ from mini_infer_amd.registry import register_norm
 class RMSNorm(Norm):
     graph_safe = True
     takes_partial_sums = True
+    takes_pending_products = True
 
     def __init__(self, hidden_size: int, eps: float, dtype: torch.dtype, device) -> None:
         super().__init__(dtype, device)
@@ -33,11 +34,17 @@ class RMSNorm(Norm):
 
     def forward(
         self,
-        delta: torch.Tensor | None,
+        delta: "torch.Tensor | ops.PartialSums | ops.PendingProduct | None",
         residual: torch.Tensor,
         rows: torch.Tensor | None = None,
-    ) -> torch.Tensor:
+    ) -> "torch.Tensor | ops.ScaledRows":
         assert self.weight is not None, "RMSNorm used before its weight was loaded"
+        if isinstance(delta, ops.PendingProduct):
+            # few rows: the product, the add and the norm but for the rows' factors are one
+            # kernel, if the part that follows takes the rows that way
+            if self.emit_scaled_rows and rows is None and ops.linear_add_norm_takes(delta, residual, self.weight):
+                return ops.linear_add_norm(delta, residual, self.weight, self.eps)
+            delta = delta.finish()
         return ops.add_rmsnorm(delta, residual, self.weight, self.eps, rows)
 
 

@@ -108,24 +108,25 @@ def test_real_widths_under_three_schedules(wide, dtype):
 def test_single_tokens_over_a_longer_context_at_real_widths(wide, monkeypatch):
     """One request of 600 tokens, the last 10 one by one in bfloat16 through the replayed decode
     step: at these widths and this context a single token's attention is left in its key ranges
-    and combined by the output projection, and the down product is summed up by the next norm
-    from 5 rows on (the 7-token portion)."""
+    and combined by the output projection (which also adds to the residual and begins the norm
+    that follows), and the down product is summed up by the next norm from 5 rows on (the
+    7-token portion)."""
     import mini_infer_amd.ops as ops
     from mini_infer_amd.engine import ModelRunner, StepEntry
     from mini_infer_amd.ops import kernels
 
     calls = {"from_attention": 0, "partial_sums": 0}
-    from_attention, partial_sums = ops.linear_from_attention, kernels.linear_partial_sums
+    add_norm, partial_sums = ops.linear_add_norm, kernels.linear_partial_sums
 
-    def count_from_attention(*args):
-        calls["from_attention"] += 1
-        return from_attention(*args)
+    def count_from_attention(pending, *args):
+        calls["from_attention"] += isinstance(pending.x, ops.AttentionPieces)
+        return add_norm(pending, *args)
 
     def count_partial_sums(*args):
         calls["partial_sums"] += 1
         return partial_sums(*args)
 
-    monkeypatch.setattr(ops, "linear_from_attention", count_from_attention)
+    monkeypatch.setattr(ops, "linear_add_norm", count_from_attention)
     monkeypatch.setattr(kernels, "linear_partial_sums", count_partial_sums)
     folder, oracle = wide
     tokens = tiny.random_tokens(WIDE, 600, seed=5)

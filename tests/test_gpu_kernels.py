@@ -612,6 +612,76 @@ def test_output_projection_from_uncombined_key_ranges(q_heads, kv_heads, head_di
     assert not ops.attention_pieces_pay(2, 32, 128) and not ops.attention_pieces_pay(1, 4, 48)
 
 
+@pytest.mark.parametrize(
+    "m,n,k,inter",
+    [(8, 4096, 4096, 14336), (1, 4096, 4096, 14336), (16, 96, 64, 160), (7, 160, 96, 301), (13, 4128, 160, 40), (3, 32, 32, 5)],
+)
+def test_product_add_and_norm_folded_into_two_products(m, n, k, inter):
+    """`linear_add_norm` (product, add into the residual, norm but for the rows' factors) followed
+    by `linear_swiglu` on its `ScaledRows`, against the four kernels they replace and against
+    float64: the residual is bit-equal (the same rounded product added in float32), the
+    activations agree as two bfloat16 roundings of the same numbers do."""
+    from mini_infer_amd import ops
+
+    x = _rand(m, k, dtype=torch.bfloat16, seed=51)
+    w = _rand(n, k, dtype=torch.bfloat16, seed=52, scale=0.1)
+    norm_w = (torch.rand(n, generator=torch.Generator().manual_seed(53)) + 0.5).bfloat16().to(DEV)
+    gate_up = _rand(2 * inter, n, dtype=torch.bfloat16, seed=54, scale=0.08)
+    residual0 = _rand(m, n, dtype=torch.float32, seed=55)
+    eps = 3e-5
+
+    apart_residual = residual0.clone()
+    normed = ops.add_rmsnorm(ops.linear(x, w), apart_residual, norm_w, eps)
+    apart = ops.linear_swiglu(normed, gate_up)
+
+    residual = residual0.clone()
+    rows = ops.linear_add_norm(ops.PendingProduct(x, w), residual, norm_w, eps)
+    assert isinstance(rows, ops.ScaledRows) and rows.values.shape == (m, n) and rows.sumsq.shape[1] == m
+    assert torch.equal(residual, apart_residual)
+    # the pieces add up to the rows' sums of squares, and finish() is the norm's output
+    exact_sumsq = (residual.double() ** 2).sum(dim=1)
+    assert ((rows.sumsq.double().sum(dim=0) - exact_sumsq).abs() <= 1e-5 * exact_sumsq).all()
+    exact_normed = residual.double() * torch.rsqrt(exact_sumsq / n + eps)[:, None] * norm_w.double()
+    assert (rows.finish().double() - exact_normed).abs().max() < 2.0 ** -6 * float(exact_normed.abs().max())
+    folded = ops.linear_swiglu(rows, gate_up)
+    assert folded.shape == (m, inter)
+
+    def activation(normed_rows):
+        both = (normed_rows @ gate_up.double().T).bfloat16().double()
+        return both[:, :inter] / (1 + torch.exp(-both[:, :inter])) * both[:, inter:]
+
+    exact = activation(exact_normed)
+    bound = 2.0 ** -5 * float(exact.abs().max()) + 1e-6
+    assert (folded.double() - exact).abs().max() < bound
+    assert (apart.double() - exact).abs().max() < bound  # (the yardstick: the four kernels are no closer)
+    # rows that meet something else than that product are finished first: the same function
+    assert ops.linear_swiglu(ops.ScaledRows(rows.values.float(), rows.sumsq, eps), gate_up.float()).shape == (m, inter)
+
+
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,lengths", [(32, 8, 128, [3000]), (6, 2, 64, [700]), (3, 1, 32, [517])])
+def test_product_add_and_norm_from_uncombined_key_ranges(q_heads, kv_heads, head_dim, lengths):
+    """The same fold with a single token's attention still in its key ranges: what
+    `linear_from_attention` then `add_rmsnorm` give, bit for bit in the residual."""
+    from mini_infer_amd import ops
+
+    case = _paged_case(torch.bfloat16, q_heads, kv_heads, head_dim, 16, lengths, [1] * len(lengths), seed=61,
+                       v_transposed=True)
+    pieces = ops.paged_attention(
+        case["q"], case["k_pages"], case["v_pages"], case["block_table"], case["token_request"], case["positions"],
+        case["cu"], case["host_cu"], q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=0.3, window=None,
+        max_seq_len=max(lengths), v_transposed=True, combine=False)
+    assert isinstance(pieces, ops.AttentionPieces)
+    k, n = q_heads * head_dim, 4096 if head_dim == 128 else 200
+    w = _rand(n, k, dtype=torch.bfloat16, seed=62, scale=0.1)
+    norm_w = (torch.rand(n, generator=torch.Generator().manual_seed(63)) + 0.5).bfloat16().to(DEV)
+    residual0 = _rand(len(lengths), n, dtype=torch.float32, seed=64)
+    apart_residual, residual = residual0.clone(), residual0.clone()
+    normed = ops.add_rmsnorm(ops.linear_from_attention(pieces, w), apart_residual, norm_w, 1e-5)
+    rows = ops.linear_add_norm(ops.PendingProduct(pieces, w), residual, norm_w, 1e-5)
+    assert torch.equal(residual, apart_residual)
+    assert (rows.finish().float() - normed.float()).abs().max() <= 2.0 ** -6 * float(normed.float().abs().max())
+
+
 def test_kernels_refuse_what_they_do_not_take():
     from mini_infer_amd import ops
     from mini_infer_amd.exceptions import KernelShapeError
