@@ -61,7 +61,8 @@ enum { PRO_NONE = 0, PRO_ATTN = 1, PRO_SCALED = 2 };
 #define SK_SCALE_PIECES 8  // pieces per such thread: 256 pieces at most
 #define SK_PRO_VALUES 4096  // activations a wave makes and holds: rows * (K / 8 waves) at most
 
-struct RopeArgs {  // EPI_ROPE only
+struct FoldArgs {  // what the folded neighbours of a product need
+  // EPI_ROPE:
   const float* cos_t;  // [m, head_dim/2]
   const float* sin_t;
   const int* slot_mapping;  // [m]: page * page_size + offset, negative: write nothing
@@ -89,7 +90,7 @@ struct RopeArgs {  // EPI_ROPE only
 template <int NT, int U, int EPI, int PRO = PRO_NONE>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t ldw,
-    bf16_t* __restrict__ c, int64_t ldc, int m, int n, int k, int features_per_block, const RopeArgs rope) {
+    bf16_t* __restrict__ c, int64_t ldc, int m, int n, int k, int features_per_block, const FoldArgs fold) {
   constexpr bool GATED = EPI == EPI_GATED;
   constexpr bool ROPE = EPI == EPI_ROPE;
   constexpr bool ADDNORM = EPI == EPI_ADDNORM;
@@ -108,8 +109,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   // partner half a head further on); pairs are numbered through all heads and a block
   // takes `features_per_block` (a multiple of 4, at most 16) consecutive ones, which may
   // lie in two heads: tile 0 holds the pairs' first dims, tile 1 their partners.
-  const int half = ROPE ? rope.head_dim / 2 : 0;
-  const int total_pairs = ROPE ? (rope.q_heads + 2 * rope.kv_heads) * half : 0;
+  const int half = ROPE ? fold.head_dim / 2 : 0;
+  const int total_pairs = ROPE ? (fold.q_heads + 2 * fold.kv_heads) * half : 0;
   const int pair0 = ROPE ? blockIdx.x * features_per_block : 0;
   const int pair_end = ROPE ? min(pair0 + features_per_block, total_pairs) : 0;
   const int n0 = blockIdx.x * features_per_block;
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     int row;
     if (ROPE) {
       const int pair = min(pair0 + col, pair_end - 1);
-      row = (pair / half) * rope.head_dim + pair % half + t * half;
+      row = (pair / half) * fold.head_dim + pair % half + t * half;
     } else {
       row = min(n0 + (t % NT) * 16 + col, n_end - 1) + (t / NT) * n;
     }
@@ -157,14 +158,14 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     // lane: the key ranges' accumulators weighted by exp(max - overall max), added in range
     // order, divided by the weighted sum of their sums (the arithmetic of attn_reduce_kernel)
     const int chunks = (s_end - s_begin) * 4;
-    const int head_dim = rope.attn_head_dim, splits = rope.num_splits;
+    const int head_dim = fold.attn_head_dim, splits = fold.num_splits;
     for (int idx = lane; idx < m * chunks; idx += MI_WAVE) {
       const int row = idx / chunks, chunk = idx % chunks;
       const int k0 = s_begin * 32 + chunk * 8;
       const int head = k0 / head_dim, dim = k0 % head_dim;
-      const int64_t base = ((int64_t)row * rope.attn_heads + head) * splits;
-      const float* ml = rope.part_ml + base * 2;
-      const float* pa = rope.part_acc + base * head_dim + dim;
+      const int64_t base = ((int64_t)row * fold.attn_heads + head) * splits;
+      const float* ml = fold.part_ml + base * 2;
+      const float* pa = fold.part_acc + base * head_dim + dim;
       // (requesting every range's values before the first use measured slower than this loop)
       float m_all = -INFINITY;
 #pragma unroll 8
@@ -205,8 +206,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         if (feature + r < n_end) {
-          res_old[r] = rope.residual[(int64_t)token * rope.ld_residual + feature + r];
-          norm_w4[r] = (float)rope.norm_weight[feature + r];
+          res_old[r] = fold.residual[(int64_t)token * fold.ld_residual + feature + r];
+          norm_w4[r] = (float)fold.norm_weight[feature + r];
         }
       }
     }
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
 #pragma unroll
     for (int i = 0; i < SK_SCALE_PIECES; ++i) {
       const int piece = part + i * SK_SCALE_PARTS;
-      scale_piece[i] = (row < m && piece < rope.sumsq_pieces) ? rope.sumsq_in[(int64_t)piece * m + row] : 0.f;
+      scale_piece[i] = (row < m && piece < fold.sumsq_pieces) ? fold.sumsq_in[(int64_t)piece * m + row] : 0.f;
     }
   }
   // acc[t][r] = C^T[feature n0 + 16*(t % NT) + 4*quad + r][token col]; add the 8 waves in order
@@ -295,7 +296,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
       float total = 0.f;
 #pragma unroll
       for (int part = 0; part < SK_SCALE_PARTS; ++part) total += scale_part[part][token];
-      const float inv = rsqrtf(total / (float)rope.norm_width + rope.norm_eps);
+      const float inv = rsqrtf(total / (float)fold.norm_width + fold.norm_eps);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         sum[r] *= inv;
@@ -311,7 +312,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     }
     if constexpr (ADDNORM) {
       const int feature = n0 + nt * 16 + fq * 4;
-      float* res = rope.residual + (int64_t)token * rope.ld_residual + feature;
+      float* res = fold.residual + (int64_t)token * fold.ld_residual + feature;
       bf16_t* dst = c + (int64_t)token * ldc + feature;
       float sq = 0.f;
 #pragma unroll
@@ -331,16 +332,16 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
       const int pair = pair0 + fq * 4;
       if (pair >= pair_end) continue;
       const int rope_head = pair / half, j = pair % half;
-      const int q_heads = rope.q_heads, kv_heads = rope.kv_heads, hd = rope.head_dim;
+      const int q_heads = fold.q_heads, kv_heads = fold.kv_heads, hd = fold.head_dim;
       float lo[4], hi[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         lo[r] = (float)(bf16_t)sum[r];
         hi[r] = (float)(bf16_t)up[r];
       }
-      if (rope_head < q_heads + kv_heads) {  // queries and keys are rotated (formula: models/blocks/rope.py:411-431)
-        const f32x4_t cs = *reinterpret_cast<const f32x4_t*>(rope.cos_t + (int64_t)token * half + j);
-        const f32x4_t sn = *reinterpret_cast<const f32x4_t*>(rope.sin_t + (int64_t)token * half + j);
+      if (rope_head < q_heads + kv_heads) {  // queries and keys are rotated (formula: models/blocks/fold.py:411-431)
+        const f32x4_t cs = *reinterpret_cast<const f32x4_t*>(fold.cos_t + (int64_t)token * half + j);
+        const f32x4_t sn = *reinterpret_cast<const f32x4_t*>(fold.sin_t + (int64_t)token * half + j);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float x0 = lo[r], x1 = hi[r];
@@ -359,22 +360,22 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
         *reinterpret_cast<bf16x4_t*>(dst) = lo_b;
         *reinterpret_cast<bf16x4_t*>(dst + half) = hi_b;
       } else {
-        const int slot = rope.slot_mapping[token];
+        const int slot = fold.slot_mapping[token];
         if (slot >= 0) {  // padding rows of a replayed step write nothing
-          const int page = slot / rope.page_size, off = slot % rope.page_size;
+          const int page = slot / fold.page_size, off = slot % fold.page_size;
           const bool is_key = rope_head < q_heads + kv_heads;
           const int h = rope_head - q_heads - (is_key ? 0 : kv_heads);
-          const int64_t chunk = ((int64_t)page * kv_heads + h) * rope.page_size * hd;
-          if (is_key || !rope.v_transposed) {
-            bf16_t* dst = (is_key ? rope.k_pages : rope.v_pages) + chunk + (int64_t)off * hd + j;
+          const int64_t chunk = ((int64_t)page * kv_heads + h) * fold.page_size * hd;
+          if (is_key || !fold.v_transposed) {
+            bf16_t* dst = (is_key ? fold.k_pages : fold.v_pages) + chunk + (int64_t)off * hd + j;
             *reinterpret_cast<bf16x4_t*>(dst) = lo_b;
             *reinterpret_cast<bf16x4_t*>(dst + half) = hi_b;
           } else {
-            bf16_t* dst = rope.v_pages + chunk + off;
+            bf16_t* dst = fold.v_pages + chunk + off;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              dst[(int64_t)(j + r) * rope.page_size] = lo_b[r];
-              dst[(int64_t)(half + j + r) * rope.page_size] = hi_b[r];
+              dst[(int64_t)(j + r) * fold.page_size] = lo_b[r];
+              dst[(int64_t)(half + j + r) * fold.page_size] = hi_b[r];
             }
           }
         }
@@ -400,7 +401,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
       float total = 0.f;
 #pragma unroll
       for (int i = 0; i < NT * 4; ++i) total += squares[i][threadIdx.x];
-      rope.sumsq_out[(int64_t)blockIdx.x * m + threadIdx.x] = total;
+      fold.sumsq_out[(int64_t)blockIdx.x * m + threadIdx.x] = total;
     }
   }
 }
@@ -444,17 +445,17 @@ extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, in
   const bf16_t* ap = (const bf16_t*)a;
   const bf16_t* wp = (const bf16_t*)w;
   bf16_t* cp = (bf16_t*)c;
-  const RopeArgs no_rope = {};
+  const FoldArgs nothing_folded = {};
   const int cus = compute_units();
   MI_REQUIRE(cus > 0, "gemm_skinny_bf16: cannot read the device's compute unit count");
   const int fpb = features_per_block_for(n, cus, 4);
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
   switch (ceil_div(fpb, 16)) {
-    case 1: gemm_skinny_bf16_kernel<1, 8, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, no_rope); break;
-    case 2: gemm_skinny_bf16_kernel<2, 8, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, no_rope); break;
-    case 3: gemm_skinny_bf16_kernel<3, 4, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, no_rope); break;
-    default: gemm_skinny_bf16_kernel<4, 2, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, no_rope); break;
+    case 1: gemm_skinny_bf16_kernel<1, 8, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); break;
+    case 2: gemm_skinny_bf16_kernel<2, 8, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); break;
+    case 3: gemm_skinny_bf16_kernel<3, 4, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); break;
+    default: gemm_skinny_bf16_kernel<4, 2, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); break;
   }
   MI_CHECK_LAUNCH("gemm_skinny_bf16");
   return MI_OK;
@@ -487,7 +488,7 @@ extern "C" int mi_gemm_skinny_attn_bf16(const float* part_acc, const float* part
   const int64_t lda = ldw;
   const bf16_t* wp = (const bf16_t*)w;
   bf16_t* cp = (bf16_t*)c;
-  RopeArgs args = {};
+  FoldArgs args = {};
   args.part_acc = part_acc;
   args.part_ml = part_ml;
   args.num_splits = num_splits;
@@ -539,7 +540,7 @@ extern "C" int mi_gemm_skinny_addnorm_bf16(const void* a, int64_t lda, const flo
   }
   MI_REQUIRE(n >= 1 && ldw >= k && ldv >= n && ld_residual >= n, "gemm_skinny_addnorm_bf16: a row stride is shorter than its row");
   MI_REQUIRE(residual && norm_weight && values && sumsq, "gemm_skinny_addnorm_bf16: needs residual, norm weight and both outputs");
-  RopeArgs args = {};
+  FoldArgs args = {};
   args.part_acc = part_acc;
   args.part_ml = part_ml;
   args.num_splits = num_splits;
@@ -587,7 +588,7 @@ extern "C" int mi_gemm_skinny_swiglu_scaled_bf16(const void* a, int64_t lda, con
   MI_REQUIRE(sumsq && pieces >= 1 && pieces <= SK_SCALE_PARTS * SK_SCALE_PIECES && eps >= 0.f,
              "gemm_skinny_swiglu_scaled_bf16: needs the rows' sums of squares in 1..%d pieces, got %d",
              SK_SCALE_PARTS * SK_SCALE_PIECES, pieces);
-  RopeArgs args = {};
+  FoldArgs args = {};
   args.sumsq_in = sumsq;
   args.sumsq_pieces = pieces;
   args.norm_eps = eps;
@@ -617,14 +618,14 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
   const bf16_t* ap = (const bf16_t*)a;
   const bf16_t* wp = (const bf16_t*)w;
   bf16_t* cp = (bf16_t*)out;
-  const RopeArgs no_rope = {};
+  const FoldArgs nothing_folded = {};
   const int cus = compute_units();
   MI_REQUIRE(cus > 0, "gemm_skinny_swiglu_bf16: cannot read the device's compute unit count");
   const int fpb = features_per_block_for(n, cus, 2);  // two output tiles = four weight tiles
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
-  if (fpb <= 16) gemm_skinny_bf16_kernel<1, 4, EPI_GATED><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, no_rope);
-  else gemm_skinny_bf16_kernel<2, 2, EPI_GATED><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, no_rope);
+  if (fpb <= 16) gemm_skinny_bf16_kernel<1, 4, EPI_GATED><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, nothing_folded);
+  else gemm_skinny_bf16_kernel<2, 2, EPI_GATED><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, nothing_folded);
   MI_CHECK_LAUNCH("gemm_skinny_swiglu_bf16");
   return MI_OK;
 }
@@ -651,17 +652,17 @@ extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* 
   MI_REQUIRE(cos_t && sin_t, "gemm_skinny_rope_bf16: needs the rotation tables");
   MI_REQUIRE(kv_heads == 0 || (slot_mapping && k_pages && v_pages && page_size > 0 && num_pages > 0),
              "gemm_skinny_rope_bf16: pages and slots are needed to write keys and values");
-  RopeArgs rope = {};
-  rope.cos_t = cos_t;
-  rope.sin_t = sin_t;
-  rope.slot_mapping = slot_mapping;
-  rope.k_pages = (bf16_t*)k_pages;
-  rope.v_pages = (bf16_t*)v_pages;
-  rope.q_heads = q_heads;
-  rope.kv_heads = kv_heads;
-  rope.head_dim = head_dim;
-  rope.page_size = page_size;
-  rope.v_transposed = v_transposed;
+  FoldArgs fold = {};
+  fold.cos_t = cos_t;
+  fold.sin_t = sin_t;
+  fold.slot_mapping = slot_mapping;
+  fold.k_pages = (bf16_t*)k_pages;
+  fold.v_pages = (bf16_t*)v_pages;
+  fold.q_heads = q_heads;
+  fold.kv_heads = kv_heads;
+  fold.head_dim = head_dim;
+  fold.page_size = page_size;
+  fold.v_transposed = v_transposed;
   // pairs per block: an even share over the CUs in whole rounds, as for the plain product
   const int cus = compute_units();
   MI_REQUIRE(cus > 0, "gemm_skinny_rope_bf16: cannot read the device's compute unit count");
@@ -671,7 +672,7 @@ extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* 
   if (pairs_per_block > 16) pairs_per_block = 16;
   const int blocks = ceil_div(total_pairs, pairs_per_block);
   gemm_skinny_bf16_kernel<1, 8, EPI_ROPE><<<blocks, 64 * SK_WAVES, 0, stream>>>(
-      (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, pairs_per_block, rope);
+      (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, pairs_per_block, fold);
   MI_CHECK_LAUNCH("gemm_skinny_rope_bf16");
   return MI_OK;
 }
