@@ -1531,6 +1531,121 @@ def test_toy_block_arrangement_and_toy_norm_in_one_layer_of_two(tmp_path, dtype)
         NORMS.unregister("centred_norm")
 
 
+def test_a_whole_architecture_with_config_keys_and_tensor_names_of_its_own(tmp_path):
+    """An architecture defined here from nothing but the framework's parts: config.json keys of
+    its own (read into a typed configuration of its own, which refuses what it does not know),
+    tensor names of its own, a feed-forward of another width in each layer, the layers run
+    twice over.  Registered under its name it gets a model folder with random weights from
+    the random-weights mode, is loaded by tensor name, steps and generates through `LLM` as
+    Llama does; the plain functions, fed the renamed tensors layer by layer, give the same
+    logits and the same greedy tokens.  No framework file changes."""
+    import dataclasses
+    import json
+
+    from safetensors.torch import load_file
+
+    from mini_infer_amd.engine import StepEntry
+    from mini_infer_amd.engine.llm import LLM
+    from mini_infer_amd.models.spec import Architecture, LayerCall, LayerSpec, ModelSpec
+    from mini_infer_amd.registry import ARCHITECTURES
+    from mini_infer_amd.weights import write_random_model
+
+    @dataclasses.dataclass(frozen=True)
+    class ToyConfig:
+        n_layer: int
+        d_model: int
+        n_head: int
+        n_kv_head: int
+        d_head: int
+        d_ff: tuple
+        n_vocab: int
+        norm_eps: float
+        rope_base: float
+        loops: int
+
+        @classmethod
+        def from_dict(cls, raw):
+            unknown = set(raw) - {f.name for f in dataclasses.fields(cls)} - {"architectures"}
+            if unknown:
+                raise ValueError(f"unknown keys in a TinyToyLM config: {sorted(unknown)}")
+            if len(raw["d_ff"]) != raw["n_layer"]:
+                raise ValueError("d_ff lists one width per layer")
+            return cls(**{k: (tuple(v) if k == "d_ff" else v) for k, v in raw.items() if k != "architectures"})
+
+    def toy_spec(cfg):
+        norm = {"kind": "rms_norm", "hidden_size": cfg.d_model, "eps": cfg.norm_eps}
+        layers = [
+            LayerSpec(prefix=f"blocks.{i}.", block={
+                "kind": "pre_norm",
+                "norm": norm,
+                "mixer": {"kind": "gqa_attention", "hidden_size": cfg.d_model, "num_heads": cfg.n_head,
+                          "num_kv_heads": cfg.n_kv_head, "head_dim": cfg.d_head,
+                          "position": {"kind": "rotary", "head_dim": cfg.d_head, "theta": cfg.rope_base}},
+                "feed_forward": {"kind": "swiglu", "hidden_size": cfg.d_model, "intermediate_size": cfg.d_ff[i]},
+                "names": {"mixer_norm": "ln1.", "mixer": "attn.", "ffn_norm": "ln2.", "feed_forward": "ff."},
+            })
+            for i in range(cfg.n_layer)
+        ]
+        return ModelSpec(
+            vocab_size=cfg.n_vocab, hidden_size=cfg.d_model, embedding_name="wte.weight", layers=layers,
+            order=[LayerCall(i) for _ in range(cfg.loops) for i in range(cfg.n_layer)],
+            final_norm=norm, final_norm_prefix="ln_f.", head_name="unused.weight", tie_word_embeddings=True,
+        )
+
+    raw = {"architectures": ["TinyToyLM"], "n_layer": 2, "d_model": 96, "n_head": 6, "n_kv_head": 3, "d_head": 16,
+           "d_ff": [80, 208], "n_vocab": 211, "norm_eps": 2e-5, "rope_base": 7000.0, "loops": 2}
+    ARCHITECTURES.register("TinyToyLM", Architecture("TinyToyLM", ToyConfig.from_dict, toy_spec))
+    try:
+        with pytest.raises(ValueError, match="unknown keys"):
+            ToyConfig.from_dict(dict(raw, hidden_size=5))
+        folder = write_random_model(raw, seed=11, out_dir=tmp_path / "toy_arch", std=0.25, norm_jitter=0.2)
+        assert json.loads((folder / "config.json").read_text()) == raw
+        weights = {k: v.double().numpy() for k, v in load_file(str(folder / "model.safetensors")).items()}
+        assert sorted(weights)[:3] == ["blocks.0.attn.k_proj.weight", "blocks.0.attn.o_proj.weight", "blocks.0.attn.q_proj.weight"]
+        assert "wte.weight" in weights and "ln_f.weight" in weights and len(weights) == 2 * 9 + 2
+        assert weights["blocks.0.ff.gate_proj.weight"].shape == (80, 96) and weights["blocks.1.ff.gate_proj.weight"].shape == (208, 96)
+
+        # the plain Llama model under Llama's names: the same formulas, the toy's tensors and order
+        renamed = {"model.embed_tokens.weight": weights["wte.weight"], "model.norm.weight": weights["ln_f.weight"]}
+        for i in range(2):
+            for ours, llamas in (("ln1.", "input_layernorm."), ("ln2.", "post_attention_layernorm."),
+                                 *((f"attn.{n}_proj.", f"self_attn.{n}_proj.") for n in "qkvo"),
+                                 *((f"ff.{n}_proj.", f"mlp.{n}_proj.") for n in ("gate", "up", "down"))):
+                renamed[f"model.layers.{i}.{llamas}weight"] = weights[f"blocks.{i}.{ours}weight"]
+        as_llama = {"num_hidden_layers": 2, "hidden_size": 96, "num_attention_heads": 6, "num_key_value_heads": 3,
+                    "head_dim": 16, "rms_norm_eps": 2e-5, "rope_theta": 7000.0, "tie_word_embeddings": True}
+        looped = [(0, None), (1, None), (0, None), (1, None)]
+
+        def plain(tokens):
+            return pl.llama_logits(as_llama, renamed, np.array(tokens), order=looped)
+
+        llm = LLM(folder, dtype="float32", num_blocks=48, block_size=4, max_num_batched_tokens=16, chunk_size=16)
+        assert len(llm.runner.cache.layer_caches()) == 4  # two layers, each called twice, each call with its own cache
+        rng = np.random.default_rng(12)
+        prompts = [[int(t) for t in rng.integers(0, 211, size=n)] for n in (9, 23, 1)]
+        for prompt, result in zip(prompts, llm.generate(prompts, max_tokens=6)):
+            tokens = list(prompt)
+            for _ in range(6):
+                tokens.append(pl.greedy(plain(tokens)[-1]))
+            assert result.tokens == tokens[len(prompt):]
+        # the step function on a whole prompt: the logits, not only their maxima
+        logits = llm.runner.step([StepEntry("whole", prompts[1], list(range(23)))]).cpu().numpy()
+        llm.runner.free_request("whole")
+        ru.assert_close(logits, plain(prompts[1]), "float32", "toy architecture, whole prompt")
+        assert llm.runner.num_free_blocks() == 48
+        # and in bfloat16, a portion and then single tokens (widths of 80 and 208: not every kernel's sizes)
+        from mini_infer_amd.engine import ModelRunner
+
+        runner = ModelRunner.from_pretrained(folder, dtype="bfloat16", num_blocks=8, block_size=4)
+        got = [runner.step([StepEntry("b", prompts[1][:17], list(range(17)))]).cpu().numpy()]
+        got += [runner.step([StepEntry("b", [t], [0])]).cpu().numpy() for t in prompts[1][17:]]
+        ru.assert_close(np.concatenate(got), ru.oracle(as_llama, renamed, prompts[1], order=looped), "bfloat16",
+                        "toy architecture, bfloat16")
+        assert runner.decode_graphs.replays == 6
+    finally:
+        ARCHITECTURES.unregister("TinyToyLM")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_context_past_eight_thousand_keys(tmp_path, dtype):
     """8,288 tokens in portions of 2,048, then 12 tokens one by one, where single tokens'
