@@ -397,7 +397,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   }
   if constexpr (ADDNORM) {
     __syncthreads();
-    if (threadIdx.x < m) {
+    if ((int)threadIdx.x < m) {
       float total = 0.f;
 #pragma unroll
       for (int i = 0; i < NT * 4; ++i) total += squares[i][threadIdx.x];
