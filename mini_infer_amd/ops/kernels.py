@@ -566,6 +566,7 @@ def linear_swiglu(x: "torch.Tensor | ScaledRows", gate_up_weight: torch.Tensor) 
             and gate_up_weight.stride(1) == 1
             and x.sumsq.is_contiguous()
             and x.sumsq.shape[0] <= SCALED_ROWS_MAX_PIECES
+            and values.shape[0] <= PENDING_PRODUCT_MAX_ROWS
             and skinny_gemm_takes(values.shape[0], width, values.stride(0), gate_up_weight.stride(0))
         ):
             scaled, x = x, values
@@ -732,6 +733,9 @@ def linear_add_norm_takes(pending: PendingProduct, residual: torch.Tensor, norm_
     ):
         return False
     x = pending.x
+    rows = x.tokens if isinstance(x, AttentionPieces) else x.shape[0]
+    if rows > PENDING_PRODUCT_MAX_ROWS:
+        return False
     if isinstance(x, AttentionPieces):
         return (
             x.dtype == torch.bfloat16
