@@ -430,3 +430,40 @@ def test_draw_index_lives_in_the_state_slot_survives_preemption_and_starts_at_ze
     slot = runner.cache.state_slot(3)
     assert states.draws(slot) == 0 and states.seed(slot) == 77 and states.position(slot) == 0
     assert states.host[slot, 5] == 0 and states.host[slot, 4] == 0
+
+
+@pytest.mark.parametrize("seed", range(120))
+def test_random_loads_give_every_request_the_tokens_it_would_get_alone(seed):
+    """Random loads on random small engines (pools from barely enough to plenty, budgets, portion
+    sizes, seats, headroom, an end-of-sequence token or none): whatever the scheduler decides
+    (portions, waves of admission, preemption and recomputation, cancelling what can never
+    fit), a request that ends by itself has exactly the tokens it would get alone, one that is
+    cancelled has a prefix of them, no step breaks the budget or the seats, and every page
+    and slot comes back."""
+    rng = np.random.default_rng(1000 + seed)
+    block_size = int(rng.choice([2, 4, 8]))
+    num_blocks = int(rng.integers(6, 60))
+    max_concurrent = int(rng.integers(1, 7))
+    budget = int(rng.integers(4, 40))
+    chunk = int(rng.integers(2, 40))
+    eos = int(rng.integers(0, VOCAB)) if rng.random() < 0.5 else None
+    runner = FakeRunner(num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent)
+    sched = make(runner, chunk_size=chunk, max_num_batched_tokens=budget, max_concurrent=max_concurrent,
+                 decode_headroom_blocks=int(rng.integers(0, 3)), eos_token_id=eos)
+    requests = [Request(prompt(int(rng.integers(1, 50)), seed * 100 + i),
+                        SamplingParams(ignore_eos=bool(rng.random() < 0.2)), max_tokens=int(rng.integers(0, 24)))
+                for i in range(int(rng.integers(1, 13)))]
+    results = sched.run_all(requests)
+    assert len(results) == len(requests)
+    for request, result in zip(requests, results):
+        alone = expected_tokens(request.prompt, request.max_tokens, None if request.sampling_params.ignore_eos else eos)
+        if result.finish_reason == "cancelled":
+            assert result.tokens == alone[: len(result.tokens)]
+        else:
+            assert result.tokens == alone
+            assert result.finish_reason == ("length" if len(alone) == request.max_tokens else "stop")
+    for step in runner.steps:
+        assert len(step) <= max_concurrent and sum(n for _, n, _ in step) <= budget
+        assert len({rid for rid, _, _ in step}) == len(step)  # a request is in a step once
+    runner.cache.check()
+    assert runner.num_free_blocks() == num_blocks and runner.cache.states.num_free == max_concurrent
