@@ -328,6 +328,33 @@ def test_tiny_b_workload_to_two_hundred_positions(tmp_path):
             assert abs(off) > 5 * math.sqrt(off_spread)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_loads_on_the_real_engine_generate_what_the_plain_model_generates(tmp_path, seed):
+    """Random loads (prompt lengths, token counts, pool from tight to roomy, budget, portion
+    size, seats) through `LLM` in float32 with the engine's own sampling on the device, ids
+    read a step late: every request that ends by itself has the plain model's greedy tokens,
+    a cancelled one a prefix of them, and the pool is whole afterwards."""
+    from mini_infer_amd.engine.llm import LLM
+
+    cfg, block, weights, folder = _folder(tmp_path, "A", 70 + seed)
+    rng = np.random.default_rng(500 + seed)
+    num_blocks = int(rng.integers(14, 60))
+    llm = LLM(folder, dtype="float32", num_blocks=num_blocks, block_size=block,
+              max_num_batched_tokens=int(rng.integers(8, 48)), chunk_size=int(rng.integers(4, 48)),
+              max_concurrent=int(rng.integers(1, 6)), decode_headroom_blocks=int(rng.integers(0, 3)))
+    prompts = [tiny.random_tokens(cfg, int(rng.integers(1, 40)), seed=seed * 50 + i) for i in range(int(rng.integers(2, 8)))]
+    new_tokens = int(rng.integers(1, 12))
+    results = llm.generate(prompts, max_tokens=new_tokens)
+    for prompt, result in zip(prompts, results):
+        expected = _plain_greedy(cfg, weights, prompt, new_tokens)
+        if result.finish_reason == "cancelled":
+            assert result.tokens == expected[: len(result.tokens)]
+        else:
+            assert result.tokens == expected and result.finish_reason == "length"
+    llm.runner.cache.check()
+    assert llm.runner.num_free_blocks() == num_blocks
+
+
 def test_preemption_on_the_real_engine_keeps_outputs(tmp_path):
     from mini_infer_amd.engine.llm import LLM
 
