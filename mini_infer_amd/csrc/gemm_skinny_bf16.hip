@@ -19,8 +19,34 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef int int32x4_t __attribute__((ext_vector_type(4)));
 
 #define SK_WAVES 8
+
+// How the weights are read (LINES).  The matrix-core operand wants, per k-step, 16 bytes of
+// each of 16 weight rows in every 16 lanes: four lanes a row, 64 bytes, half a cache line; the
+// other half is asked for by the next k-step's load.  Whole lines per load run faster, and
+// non-temporal loads (the weights are read once) faster again, but only on whole lines:
+// measured on MI355X for 28672 x 4096, 45.8 us as above, 47.5-50.1 us non-temporal on half
+// lines, 42.3-44.7 us non-temporal on whole lines.  So with LINES a load takes 8 rows x 128
+// bytes (two k-steps): lane (quad, col) reads row col % 8 of the tile's lower or upper 8 rows,
+// 16-byte chunk quad + 4 * (col / 8) of the line.  Of a pair of such loads (lower rows,
+// upper rows) the lanes col >= 8 of the first and col < 8 of the second change places, and
+// the pair is the operands of the two k-steps.
+// Needs: rows of the matrix on 128-byte boundaries, an even number of k-steps for every wave.
+__device__ __forceinline__ void lines_to_operands(bf16x8_t& lower_rows, bf16x8_t& upper_rows) {
+  int32x4_t lo = __builtin_bit_cast(int32x4_t, lower_rows), hi = __builtin_bit_cast(int32x4_t, upper_rows);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int lo_was = lo[e];
+    // row_shr:8, lanes 8-15 of every 16: lane c takes the upper rows' lane c - 8 (row c, first k-step)
+    lo[e] = __builtin_amdgcn_update_dpp(lo[e], hi[e], 0x118, 0xF, 0xC, false);
+    // row_shl:8, lanes 0-7: lane c takes the lower rows' lane c + 8 (row c, second k-step)
+    hi[e] = __builtin_amdgcn_update_dpp(hi[e], lo_was, 0x108, 0xF, 0x3, false);
+  }
+  lower_rows = __builtin_bit_cast(bf16x8_t, lo);  // operand of the pair's first k-step
+  upper_rows = __builtin_bit_cast(bf16x8_t, hi);  // operand of its second
+}
 
 // NT = 16-feature tiles of the OUTPUT per block (the activations a wave loads are used
 // for every weight tile of the block), U = k-steps whose loads are issued together
@@ -87,7 +113,7 @@ struct FoldArgs {  // what the folded neighbours of a product need
   int norm_width;
 };
 
-template <int NT, int U, int EPI, int PRO = PRO_NONE>
+template <int NT, int U, int EPI, int PRO = PRO_NONE, bool LINES = false>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t ldw,
     bf16_t* __restrict__ c, int64_t ldc, int m, int n, int k, int features_per_block, const FoldArgs fold) {
@@ -96,10 +122,13 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   constexpr bool ADDNORM = EPI == EPI_ADDNORM;
   constexpr bool SCALED = PRO == PRO_SCALED;
   static_assert(!ROPE || NT == 1, "the rotary epilogue takes one tile of dims and its partner tile");
+  static_assert(!LINES || (U % 2 == 0 && PRO != PRO_ATTN), "whole lines are read for pairs of k-steps");
   constexpr int WT = (GATED || ROPE) ? 2 * NT : NT;  // weight tiles per block
   __shared__ float red[SK_WAVES][WT][256];
 
-  const int wave = threadIdx.x / MI_WAVE;
+  // (with LINES made uniform for the compiler: the wave's range of K and with it the loop and
+  // the base address of every load are scalar)
+  const int wave = LINES ? __builtin_amdgcn_readfirstlane(threadIdx.x / MI_WAVE) : threadIdx.x / MI_WAVE;
   const int lane = threadIdx.x % MI_WAVE;
   const int col = lane % 16;
   const int quad = lane / 16;
@@ -123,18 +152,40 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
 
   // weights: lane reads feature n0 + 16*nt + col (and its twin n rows further down when
   // gated), 8 consecutive k
-  const bf16_t* wp[WT];
+  auto weight_row = [&](int t, int c) -> int {  // the matrix row behind row c of weight tile t
+    if (ROPE) {
+      const int pair = min(pair0 + c, pair_end - 1);
+      return (pair / half) * fold.head_dim + pair % half + t * half;
+    }
+    return min(n0 + (t % NT) * 16 + c, n_end - 1) + (t / NT) * n;
+  };
+  const bf16_t* wp[LINES ? 1 : WT];
+  // LINES: byte offsets of this lane's 16 bytes in the tile's lower and upper 8 rows
+  uint32_t line_lo[LINES ? WT : 1], line_hi[LINES ? WT : 1];
 #pragma unroll
   for (int t = 0; t < WT; ++t) {
-    int row;
-    if (ROPE) {
-      const int pair = min(pair0 + col, pair_end - 1);
-      row = (pair / half) * fold.head_dim + pair % half + t * half;
+    if constexpr (LINES) {
+      const uint32_t chunk = (uint32_t)(quad + 4 * (col / 8)) * 16u;
+      line_lo[t] = (uint32_t)weight_row(t, col % 8) * (uint32_t)(ldw * 2) + chunk;
+      line_hi[t] = (uint32_t)weight_row(t, 8 + col % 8) * (uint32_t)(ldw * 2) + chunk;
     } else {
-      row = min(n0 + (t % NT) * 16 + col, n_end - 1) + (t / NT) * n;
+      wp[t] = w + (int64_t)weight_row(t, col) * ldw + quad * 8;
     }
-    wp[t] = w + (int64_t)row * ldw + quad * 8;
   }
+  using global_bytes = const __attribute__((address_space(1))) char;
+  using global_chunk = const __attribute__((address_space(1))) bf16x8_t;
+  // the lane's operands of the k-steps first, first + 1 of weight tile t (LINES)
+  auto load_lines = [&](int t, int first, bf16x8_t& even_step, bf16x8_t& odd_step) {
+    uint64_t base_bits = reinterpret_cast<uint64_t>(w) + (uint64_t)(uint32_t)first * 64u;
+    asm("" : "+s"(base_bits));  // kept in scalar registers: the lanes add their 32-bit offsets
+    global_bytes* base = (global_bytes*)base_bits;
+    // (opaque to the compiler, or it widens the offsets to 64 bits once and for all and adds
+    // whole addresses in vector registers for every load)
+    uint32_t lo_at = line_lo[LINES ? t : 0], hi_at = line_hi[LINES ? t : 0];
+    asm("" : "+v"(lo_at), "+v"(hi_at));
+    even_step = __builtin_nontemporal_load((global_chunk*)(base + lo_at));
+    odd_step = __builtin_nontemporal_load((global_chunk*)(base + hi_at));
+  };
   // activations: lane reads token `col`; lanes past M re-read the last token (the same
   // cache lines as its own lane, so no extra traffic) and their columns are never stored
   const bf16_t* ap = a + (int64_t)min(col, m - 1) * lda + quad * 8;
@@ -150,7 +201,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
       for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int t = 0; t < WT; ++t)
-          w_first[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[t] + (int64_t)(s_begin + u) * 32);
+          w_first[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[LINES ? 0 : t] + (int64_t)(s_begin + u) * 32);
     }
   }
   if constexpr (PRO == PRO_ATTN) {
@@ -225,11 +276,21 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     for (int u = 0; u < U; ++u) {
 #pragma unroll
       for (int t = 0; t < WT; ++t) {
-        if (PRO == PRO_ATTN && first_ahead && s == s_begin) w_reg[u][t] = w_first[PRO == PRO_ATTN ? u : 0][t];
-        else w_reg[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[t] + (int64_t)(s + u) * 32);
+        if constexpr (LINES) {
+          if (u % 2 == 0) load_lines(t, s + u, w_reg[u][t], w_reg[u + 1][t]);
+        } else {
+          if (PRO == PRO_ATTN && first_ahead && s == s_begin) w_reg[u][t] = w_first[PRO == PRO_ATTN ? u : 0][t];
+          else w_reg[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[LINES ? 0 : t] + (int64_t)(s + u) * 32);
+        }
       }
       if constexpr (PRO == PRO_ATTN) a_reg[u] = *reinterpret_cast<const bf16x8_t*>(own + (s + u - s_begin) * 32);
       else a_reg[u] = *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)(s + u) * 32);
+    }
+    if constexpr (LINES) {
+#pragma unroll
+      for (int u = 0; u < U; u += 2)
+#pragma unroll
+        for (int t = 0; t < WT; ++t) lines_to_operands(w_reg[u][t], w_reg[u + 1][t]);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -237,12 +298,26 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
       for (int t = 0; t < WT; ++t)
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_reg[u][t], a_reg[u], acc[t], 0, 0, 0);
   }
-  for (; s < s_end; ++s) {  // fewer than U k-steps left
+  if constexpr (LINES) {
+    for (; s + 2 <= s_end; s += 2) {  // fewer than U k-steps left: pair by pair (their number is even)
+      const bf16x8_t a_even = *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)s * 32);
+      const bf16x8_t a_odd = *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)(s + 1) * 32);
+#pragma unroll
+      for (int t = 0; t < WT; ++t) {
+        bf16x8_t w_even, w_odd;
+        load_lines(t, s, w_even, w_odd);
+        lines_to_operands(w_even, w_odd);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_even, a_even, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_odd, a_odd, acc[t], 0, 0, 0);
+      }
+    }
+  }
+  for (; !LINES && s < s_end; ++s) {  // fewer than U k-steps left
     const bf16x8_t a_tail = PRO == PRO_ATTN ? *reinterpret_cast<const bf16x8_t*>(own + (s - s_begin) * 32)
                                             : *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)s * 32);
 #pragma unroll
     for (int t = 0; t < WT; ++t) {
-      const bf16x8_t w_tail = *reinterpret_cast<const bf16x8_t*>(wp[t] + (int64_t)s * 32);
+      const bf16x8_t w_tail = *reinterpret_cast<const bf16x8_t*>(wp[LINES ? 0 : t] + (int64_t)s * 32);
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_tail, a_tail, acc[t], 0, 0, 0);
     }
   }
@@ -436,6 +511,14 @@ static int features_per_block_for(int n, int cus, int max_tiles) {
   return fpb < 8 ? 8 : fpb;
 }
 
+// Whether a weight matrix of `rows` rows can be read in whole cache lines (LINES): its rows
+// begin on 128-byte boundaries, every wave gets an even number of k-steps, and byte offsets
+// into it fit 32 bits.
+static bool whole_lines(const void* w, int64_t ldw, int64_t rows, int k) {
+  return (uintptr_t)w % 128 == 0 && ldw % 64 == 0 && (k / 32) % (2 * SK_WAVES) == 0 &&
+         rows * ldw * 2 < ((int64_t)1 << 32);
+}
+
 extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* c,
                                    int64_t ldc, int m, int n, int k, hipStream_t stream) {
   MI_REQUIRE(mi_gemm_skinny_bf16_supported(m, n, k, lda, ldw),
@@ -451,12 +534,19 @@ extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, in
   const int fpb = features_per_block_for(n, cus, 4);
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
+  const bool lines = whole_lines(w, ldw, n, k);
+#define SK_PLAIN(NT_, U_)                                                                                          \
+  if (lines)                                                                                                       \
+    gemm_skinny_bf16_kernel<NT_, U_, EPI_STORE, PRO_NONE, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); \
+  else                                                                                                             \
+    gemm_skinny_bf16_kernel<NT_, U_, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded)
   switch (ceil_div(fpb, 16)) {
-    case 1: gemm_skinny_bf16_kernel<1, 8, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); break;
-    case 2: gemm_skinny_bf16_kernel<2, 8, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); break;
-    case 3: gemm_skinny_bf16_kernel<3, 4, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); break;
-    default: gemm_skinny_bf16_kernel<4, 2, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); break;
+    case 1: SK_PLAIN(1, 8); break;
+    case 2: SK_PLAIN(2, 8); break;
+    case 3: SK_PLAIN(3, 4); break;
+    default: SK_PLAIN(4, 2); break;
   }
+#undef SK_PLAIN
   MI_CHECK_LAUNCH("gemm_skinny_bf16");
   return MI_OK;
 }
@@ -559,9 +649,12 @@ extern "C" int mi_gemm_skinny_addnorm_bf16(const void* a, int64_t lda, const flo
   const int fpb = features_per_block_for(n, cus, 4);
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
+  const bool lines = whole_lines(w, ldw, n, k);
 #define SK_ADDNORM(NT_, U_)                                                                                        \
   if (from_attention)                                                                                              \
     gemm_skinny_bf16_kernel<NT_, U_, EPI_ADDNORM, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldv, m, n, k, fpb, args); \
+  else if (lines)                                                                                                  \
+    gemm_skinny_bf16_kernel<NT_, U_, EPI_ADDNORM, PRO_NONE, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldv, m, n, k, fpb, args); \
   else                                                                                                             \
     gemm_skinny_bf16_kernel<NT_, U_, EPI_ADDNORM><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldv, m, n, k, fpb, args)
   switch (ceil_div(fpb, 16)) {
@@ -598,12 +691,16 @@ extern "C" int mi_gemm_skinny_swiglu_scaled_bf16(const void* a, int64_t lda, con
   const int fpb = features_per_block_for(n, cus, 2);
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
-  if (fpb <= 16)
-    gemm_skinny_bf16_kernel<1, 4, EPI_GATED, PRO_SCALED><<<blocks, threads, 0, stream>>>(
-        (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)out, ldo, m, n, k, fpb, args);
-  else
-    gemm_skinny_bf16_kernel<2, 2, EPI_GATED, PRO_SCALED><<<blocks, threads, 0, stream>>>(
-        (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)out, ldo, m, n, k, fpb, args);
+  const bool lines = whole_lines(w, ldw, 2 * (int64_t)n, k);
+#define SK_SCALED(NT_, U_, LINES_)                                                          \
+  gemm_skinny_bf16_kernel<NT_, U_, EPI_GATED, PRO_SCALED, LINES_><<<blocks, threads, 0, stream>>>( \
+      (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)out, ldo, m, n, k, fpb, args)
+  if (fpb <= 16) {
+    if (lines) SK_SCALED(1, 4, true); else SK_SCALED(1, 4, false);
+  } else {
+    if (lines) SK_SCALED(2, 2, true); else SK_SCALED(2, 2, false);
+  }
+#undef SK_SCALED
   MI_CHECK_LAUNCH("gemm_skinny_swiglu_scaled_bf16");
   return MI_OK;
 }
@@ -624,8 +721,15 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
   const int fpb = features_per_block_for(n, cus, 2);  // two output tiles = four weight tiles
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
-  if (fpb <= 16) gemm_skinny_bf16_kernel<1, 4, EPI_GATED><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, nothing_folded);
-  else gemm_skinny_bf16_kernel<2, 2, EPI_GATED><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, nothing_folded);
+  const bool lines = whole_lines(w, ldw, 2 * (int64_t)n, k);
+#define SK_GATED(NT_, U_, LINES_) \
+  gemm_skinny_bf16_kernel<NT_, U_, EPI_GATED, PRO_NONE, LINES_><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, nothing_folded)
+  if (fpb <= 16) {
+    if (lines) SK_GATED(1, 4, true); else SK_GATED(1, 4, false);
+  } else {
+    if (lines) SK_GATED(2, 2, true); else SK_GATED(2, 2, false);
+  }
+#undef SK_GATED
   MI_CHECK_LAUNCH("gemm_skinny_swiglu_bf16");
   return MI_OK;
 }
@@ -671,8 +775,12 @@ extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* 
   int pairs_per_block = ceil_div(ceil_div(total_pairs, cus * rounds), 4) * 4;
   if (pairs_per_block > 16) pairs_per_block = 16;
   const int blocks = ceil_div(total_pairs, pairs_per_block);
-  gemm_skinny_bf16_kernel<1, 8, EPI_ROPE><<<blocks, 64 * SK_WAVES, 0, stream>>>(
-      (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, pairs_per_block, fold);
+  if (whole_lines(w, ldw, n, k))
+    gemm_skinny_bf16_kernel<1, 8, EPI_ROPE, PRO_NONE, true><<<blocks, 64 * SK_WAVES, 0, stream>>>(
+        (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, pairs_per_block, fold);
+  else
+    gemm_skinny_bf16_kernel<1, 8, EPI_ROPE><<<blocks, 64 * SK_WAVES, 0, stream>>>(
+        (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, pairs_per_block, fold);
   MI_CHECK_LAUNCH("gemm_skinny_rope_bf16");
   return MI_OK;
 }

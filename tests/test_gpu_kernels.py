@@ -23,6 +23,19 @@ def _rand(*shape, dtype=torch.float32, seed=0, scale=1.0):
     return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
 
 
+def _off_the_cache_lines(w):
+    """A contiguous copy of `w` that begins 16 bytes past a 128-byte boundary.  The weight-streaming
+    products read whole cache lines where the rows of the matrix begin on such boundaries (and K
+    gives every wave an even number of 32-element steps), half lines otherwise: both ways add
+    the same products in the same order, so their results are equal bit for bit."""
+    flat = torch.empty(w.numel() + 64, dtype=w.dtype, device=w.device)
+    shift = (-(flat.data_ptr() // w.element_size()) % 64 + 8) % 64
+    out = flat[shift : shift + w.numel()].view(w.shape)
+    assert out.data_ptr() % 128 == 16 and out.is_contiguous()
+    out.copy_(w)
+    return out
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hidden,vocab", [(4096, 1000), (100, 301), (90, 17)])
 def test_embed_gather(dtype, hidden, vocab):
@@ -106,7 +119,7 @@ def test_gemm_f32_is_true_float32(m, n, k):
 @pytest.mark.parametrize(
     "m,n,k",
     [(1, 4096, 4096), (8, 6144, 4096), (16, 96, 64), (7, 301, 96), (13, 130, 160), (16, 1000, 14336),
-     (5, 128256, 256), (3, 7, 32), (9, 28672, 4096), (2, 16400, 1056)],
+     (5, 128256, 256), (3, 7, 32), (9, 28672, 4096), (2, 16400, 1056), (4, 4096, 1536), (6, 640, 3072), (16, 2050, 512)],
 )
 def test_gemm_skinny_bf16(m, n, k):
     from mini_infer_amd import ops
@@ -123,6 +136,7 @@ def test_gemm_skinny_bf16(m, n, k):
     wide = _rand(m, k + 8, dtype=torch.bfloat16, seed=11)
     assert torch.equal(ops.gemm_skinny_bf16(wide[:, :k], w), ops.gemm_skinny_bf16(wide[:, :k].contiguous(), w))
     assert torch.equal(ops.linear(a, w), out)
+    assert torch.equal(ops.gemm_skinny_bf16(a, _off_the_cache_lines(w)), out)
 
 
 @pytest.mark.parametrize(
@@ -178,7 +192,8 @@ def test_linear_leaves_partial_sums_only_where_asked_and_where_it_pays():
 
 @pytest.mark.parametrize(
     "m,inter,k",
-    [(1, 14336, 4096), (8, 14336, 4096), (16, 160, 64), (7, 301, 96), (13, 4100, 160), (3, 5, 32), (9, 8192, 3072)],
+    [(1, 14336, 4096), (8, 14336, 4096), (16, 160, 64), (7, 301, 96), (13, 4100, 160), (3, 5, 32), (9, 8192, 3072),
+     (5, 520, 1536), (2, 24, 512)],
 )
 def test_linear_swiglu_is_the_product_followed_by_the_activation(m, inter, k):
     from mini_infer_amd import ops
@@ -189,6 +204,7 @@ def test_linear_swiglu_is_the_product_followed_by_the_activation(m, inter, k):
     assert fused.shape == (m, inter)
     # the two-kernel path: the product (rounded to bfloat16), then the activation
     assert torch.equal(fused, ops.silu_mul(ops.gemm_skinny_bf16(a, w)))
+    assert torch.equal(ops.linear_swiglu(a, _off_the_cache_lines(w)), fused)
     gate_up = (a.double() @ w.double().T).bfloat16().double()
     gate, up = gate_up[:, :inter], gate_up[:, inter:]
     expected = gate / (1 + torch.exp(-gate)) * up
@@ -206,7 +222,8 @@ def test_linear_swiglu_is_the_product_followed_by_the_activation(m, inter, k):
 @pytest.mark.parametrize("v_transposed", [False, True])
 @pytest.mark.parametrize(
     "m,hidden,q_heads,kv_heads,head_dim,page_size",
-    [(8, 4096, 32, 8, 128, 16), (1, 4096, 32, 8, 128, 16), (16, 96, 3, 1, 32, 16), (5, 160, 6, 2, 64, 32), (9, 64, 4, 4, 96, 48)],
+    [(8, 4096, 32, 8, 128, 16), (1, 4096, 32, 8, 128, 16), (16, 96, 3, 1, 32, 16), (5, 160, 6, 2, 64, 32), (9, 64, 4, 4, 96, 48),
+     (3, 1536, 6, 2, 64, 16)],
 )
 def test_qkv_rope_write_is_the_product_followed_by_rotation_and_cache_write(
     v_transposed, m, hidden, q_heads, kv_heads, head_dim, page_size
@@ -242,6 +259,10 @@ def test_qkv_rope_write_is_the_product_followed_by_rotation_and_cache_write(
     assert (queries.float() - qkv[:, : q_heads * head_dim].float()).abs().max() <= tol
     assert (k_one.float() - k_two.float()).abs().max() <= tol
     assert torch.equal(v_one, v_two)  # values are copied, not rotated
+    k_off, v_off = pages()
+    off_lines = ops.qkv_rope_write(x, _off_the_cache_lines(w), cos, sin, slots, k_off, v_off, q_heads=q_heads,
+                                   kv_heads=kv_heads, head_dim=head_dim, v_transposed=v_transposed)
+    assert torch.equal(off_lines, queries) and torch.equal(k_off, k_one) and torch.equal(v_off, v_one)
     # queries only (a layer that reads another layer's keys and values): pages stay untouched
     k_none, v_none = pages()
     only_q = ops.qkv_rope_write(x, w[: q_heads * head_dim], cos, sin, None, k_none, v_none, q_heads=q_heads,
@@ -614,7 +635,8 @@ def test_output_projection_from_uncombined_key_ranges(q_heads, kv_heads, head_di
 
 @pytest.mark.parametrize(
     "m,n,k,inter",
-    [(8, 4096, 4096, 14336), (1, 4096, 4096, 14336), (16, 96, 64, 160), (7, 160, 96, 301), (13, 4128, 160, 40), (3, 32, 32, 5)],
+    [(8, 4096, 4096, 14336), (1, 4096, 4096, 14336), (16, 96, 64, 160), (7, 160, 96, 301), (13, 4128, 160, 40), (3, 32, 32, 5),
+     (6, 1536, 1536, 520)],
 )
 def test_product_add_and_norm_folded_into_two_products(m, n, k, inter):
     """`linear_add_norm` (product, add into the residual, norm but for the rows' factors) followed
@@ -645,6 +667,11 @@ def test_product_add_and_norm_folded_into_two_products(m, n, k, inter):
     assert (rows.finish().double() - exact_normed).abs().max() < 2.0 ** -6 * float(exact_normed.abs().max())
     folded = ops.linear_swiglu(rows, gate_up)
     assert folded.shape == (m, inter)
+    residual_off = residual0.clone()
+    rows_off = ops.linear_add_norm(ops.PendingProduct(x, _off_the_cache_lines(w)), residual_off, norm_w, eps)
+    assert torch.equal(residual_off, residual) and torch.equal(rows_off.values, rows.values)
+    assert torch.equal(rows_off.sumsq, rows.sumsq)
+    assert torch.equal(ops.linear_swiglu(rows, _off_the_cache_lines(gate_up)), folded)
 
     def activation(normed_rows):
         both = (normed_rows @ gate_up.double().T).bfloat16().double()
