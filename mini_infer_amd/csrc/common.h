@@ -49,13 +49,59 @@ __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }
 
-// A load of data that a kernel reads once and nobody reads again soon (the weights of a
-// product with few rows, the keys and values of a decode step): marked non-temporal, so that
-// it does not push what is reused out of the caches.  Measured on MI355X, long reads run at
-// 7.0-7.1 TB/s with this mark against 6.1-6.3 TB/s without it.
-template <typename T>
-__device__ __forceinline__ T load_streamed(const T* p) {
-  return __builtin_nontemporal_load(p);
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef int int32x4_t __attribute__((ext_vector_type(4)));
+
+// How a weight-streaming product reads its weights ("LINES" in the kernels).  The matrix-core
+// operand wants, per k-step (32 elements), 16 bytes of each of 16 weight rows in every 16
+// lanes: four lanes a row, 64 bytes, half a cache line; the other half is asked for by the
+// next k-step's load.  Whole lines per load run faster, and non-temporal loads (the weights
+// are read once) faster again, but only on whole lines: measured on MI355X for 28672 x 4096,
+// 45.8 us on half lines, 47.5-50.1 us non-temporal on half lines, 42.3-44.7 us non-temporal
+// on whole lines; a long plain read reaches 6.1-6.3 TB/s, a non-temporal one 7.0-7.1 TB/s.
+// So a load takes 8 rows x 128 bytes (two k-steps): lane (quad, col) reads row col % 8 of
+// the tile's lower or upper 8 rows, 16-byte chunk quad + 4 * (col / 8) of the line.  Of a pair
+// of such loads (lower rows, upper rows) the lanes col >= 8 of the first and col < 8 of the
+// second change places, and the pair is the operands of the two k-steps.
+// Needs: rows of the matrix on 128-byte boundaries, k-steps taken in even-aligned pairs.
+__device__ __forceinline__ void lines_to_operands(bf16x8_t& lower_rows, bf16x8_t& upper_rows) {
+  int32x4_t lo = __builtin_bit_cast(int32x4_t, lower_rows), hi = __builtin_bit_cast(int32x4_t, upper_rows);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int lo_was = lo[e];
+    // row_shr:8, lanes 8-15 of every 16: lane c takes the upper rows' lane c - 8 (row c, first k-step)
+    lo[e] = __builtin_amdgcn_update_dpp(lo[e], hi[e], 0x118, 0xF, 0xC, false);
+    // row_shl:8, lanes 0-7: lane c takes the lower rows' lane c + 8 (row c, second k-step)
+    hi[e] = __builtin_amdgcn_update_dpp(hi[e], lo_was, 0x108, 0xF, 0x3, false);
+  }
+  lower_rows = __builtin_bit_cast(bf16x8_t, lo);  // operand of the pair's first k-step
+  upper_rows = __builtin_bit_cast(bf16x8_t, hi);  // operand of its second
+}
+
+// The 16-byte chunk of its row's line that a lane reads, as a byte offset.
+__device__ __forceinline__ uint32_t line_chunk_of_lane(int lane) {
+  return (uint32_t)(lane / 16 + 4 * ((lane % 16) / 8)) * 16u;
+}
+
+// The two loads of a pair of k-steps: base (uniform, kept in scalar registers) + the lane's offsets.
+template <bool STREAMED = true>
+__device__ __forceinline__ void load_line_pair(const void* matrix, int64_t first_kstep, uint32_t lower_at,
+                                               uint32_t upper_at, bf16x8_t& lower_rows, bf16x8_t& upper_rows) {
+  using global_bytes = const __attribute__((address_space(1))) char;
+  using global_chunk = const __attribute__((address_space(1))) bf16x8_t;
+  uint64_t base_bits = reinterpret_cast<uint64_t>(matrix) + (uint64_t)first_kstep * 64u;
+  asm("" : "+s"(base_bits));  // scalar: the lanes add their 32-bit offsets
+  global_bytes* base = (global_bytes*)base_bits;
+  // (opaque to the compiler, or it widens the offsets to 64 bits once and for all and adds
+  // whole addresses in vector registers for every load)
+  asm("" : "+v"(lower_at), "+v"(upper_at));
+  if constexpr (STREAMED) {
+    lower_rows = __builtin_nontemporal_load((global_chunk*)(base + lower_at));
+    upper_rows = __builtin_nontemporal_load((global_chunk*)(base + upper_at));
+  } else {
+    lower_rows = *(global_chunk*)(base + lower_at);
+    upper_rows = *(global_chunk*)(base + upper_at);
+  }
 }
 
 __device__ __forceinline__ float wave_max(float v) {

@@ -19,35 +19,11 @@
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
-typedef int int32x4_t __attribute__((ext_vector_type(4)));
 
 #define SK_WAVES 8
 
-// How the weights are read (LINES).  The matrix-core operand wants, per k-step, 16 bytes of
-// each of 16 weight rows in every 16 lanes: four lanes a row, 64 bytes, half a cache line; the
-// other half is asked for by the next k-step's load.  Whole lines per load run faster, and
-// non-temporal loads (the weights are read once) faster again, but only on whole lines:
-// measured on MI355X for 28672 x 4096, 45.8 us as above, 47.5-50.1 us non-temporal on half
-// lines, 42.3-44.7 us non-temporal on whole lines.  So with LINES a load takes 8 rows x 128
-// bytes (two k-steps): lane (quad, col) reads row col % 8 of the tile's lower or upper 8 rows,
-// 16-byte chunk quad + 4 * (col / 8) of the line.  Of a pair of such loads (lower rows,
-// upper rows) the lanes col >= 8 of the first and col < 8 of the second change places, and
-// the pair is the operands of the two k-steps.
-// Needs: rows of the matrix on 128-byte boundaries, an even number of k-steps for every wave.
-__device__ __forceinline__ void lines_to_operands(bf16x8_t& lower_rows, bf16x8_t& upper_rows) {
-  int32x4_t lo = __builtin_bit_cast(int32x4_t, lower_rows), hi = __builtin_bit_cast(int32x4_t, upper_rows);
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const int lo_was = lo[e];
-    // row_shr:8, lanes 8-15 of every 16: lane c takes the upper rows' lane c - 8 (row c, first k-step)
-    lo[e] = __builtin_amdgcn_update_dpp(lo[e], hi[e], 0x118, 0xF, 0xC, false);
-    // row_shl:8, lanes 0-7: lane c takes the lower rows' lane c + 8 (row c, second k-step)
-    hi[e] = __builtin_amdgcn_update_dpp(hi[e], lo_was, 0x108, 0xF, 0x3, false);
-  }
-  lower_rows = __builtin_bit_cast(bf16x8_t, lo);  // operand of the pair's first k-step
-  upper_rows = __builtin_bit_cast(bf16x8_t, hi);  // operand of its second
-}
-
+// LINES: the weights are read in whole cache lines (lines_to_operands in common.h), where
+// the matrix lies so that they can be.
 // NT = 16-feature tiles of the OUTPUT per block (the activations a wave loads are used
 // for every weight tile of the block), U = k-steps whose loads are issued together
 // before their products run.  Register use is kept low on purpose: many resident waves,
@@ -165,26 +141,16 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
 #pragma unroll
   for (int t = 0; t < WT; ++t) {
     if constexpr (LINES) {
-      const uint32_t chunk = (uint32_t)(quad + 4 * (col / 8)) * 16u;
+      const uint32_t chunk = line_chunk_of_lane(lane);
       line_lo[t] = (uint32_t)weight_row(t, col % 8) * (uint32_t)(ldw * 2) + chunk;
       line_hi[t] = (uint32_t)weight_row(t, 8 + col % 8) * (uint32_t)(ldw * 2) + chunk;
     } else {
       wp[t] = w + (int64_t)weight_row(t, col) * ldw + quad * 8;
     }
   }
-  using global_bytes = const __attribute__((address_space(1))) char;
-  using global_chunk = const __attribute__((address_space(1))) bf16x8_t;
   // the lane's operands of the k-steps first, first + 1 of weight tile t (LINES)
   auto load_lines = [&](int t, int first, bf16x8_t& even_step, bf16x8_t& odd_step) {
-    uint64_t base_bits = reinterpret_cast<uint64_t>(w) + (uint64_t)(uint32_t)first * 64u;
-    asm("" : "+s"(base_bits));  // kept in scalar registers: the lanes add their 32-bit offsets
-    global_bytes* base = (global_bytes*)base_bits;
-    // (opaque to the compiler, or it widens the offsets to 64 bits once and for all and adds
-    // whole addresses in vector registers for every load)
-    uint32_t lo_at = line_lo[LINES ? t : 0], hi_at = line_hi[LINES ? t : 0];
-    asm("" : "+v"(lo_at), "+v"(hi_at));
-    even_step = __builtin_nontemporal_load((global_chunk*)(base + lo_at));
-    odd_step = __builtin_nontemporal_load((global_chunk*)(base + hi_at));
+    load_line_pair(w, first, line_lo[LINES ? t : 0], line_hi[LINES ? t : 0], even_step, odd_step);
   };
   // activations: lane reads token `col`; lanes past M re-read the last token (the same
   // cache lines as its own lane, so no extra traffic) and their columns are never stored

@@ -142,7 +142,7 @@ def test_gemm_skinny_bf16(m, n, k):
 @pytest.mark.parametrize(
     "m,n,k",
     [(1, 4096, 14336), (8, 1000, 8192 + 32), (16, 4096, 4096), (17, 1003, 4096), (33, 136, 608), (64, 4096, 14336),
-     (47, 5, 32), (64, 260, 8192 - 224), (128, 4096, 4096), (101, 200, 1024 + 64)],
+     (47, 5, 32), (64, 260, 8192 - 224), (128, 4096, 4096), (101, 200, 1024 + 64), (24, 3072, 8192 + 64)],
 )
 def test_linear_in_partial_sums_then_norm_is_linear_then_norm(m, n, k):
     """A product left as sums over ranges of K, added up by the norm that follows it: the
@@ -162,6 +162,7 @@ def test_linear_in_partial_sums_then_norm_is_linear_then_norm(m, n, k):
     # strided activations: a slice of a wider buffer
     wide = _rand(m, k + 8, dtype=torch.bfloat16, seed=35)
     assert torch.equal(ops.linear_partial_sums(wide[:, :k], w).pieces, ops.linear_partial_sums(wide[:, :k].contiguous(), w).pieces)
+    assert torch.equal(ops.linear_partial_sums(a, _off_the_cache_lines(w)).pieces, partial.pieces)
     weight = _rand(n, dtype=torch.bfloat16, seed=33).abs() + 0.5
     for rows in (None, torch.tensor([m - 1, 0], dtype=torch.int32, device=DEV)):
         res_a, res_b = _rand(m, n, seed=34), _rand(m, n, seed=34)
