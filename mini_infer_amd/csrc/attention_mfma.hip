@@ -290,12 +290,20 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   const int head_off = kvh * page_size * D;
   const unsigned k_lane_off = (unsigned)(col * D + quad * 8);
   const unsigned v_lane_off = (unsigned)(col * page_size + 4 * quad);
+  // Decode shape with 16-slot pages and key rows of whole cache lines: keys and values are read
+  // once, so with non-temporal loads, and the keys in whole lines (lines_to_operands in
+  // common.h; the values' 16 rows of 32 bytes per load are whole lines as they are).
+  constexpr bool STREAM_KV = !SHARED && PS == 16 && D % 64 == 0;
+  const uint32_t k_line_lo = (uint32_t)((col % 8) * D * 2) + line_chunk_of_lane(lane);
+  const uint32_t k_line_hi = k_line_lo + 8u * D * 2u;
   auto load_values = [&](const bf16_t* const v_base[2], bf16x8_t* v) {
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db) {
       const unsigned off = v_lane_off + (unsigned)(db * 16) * (unsigned)page_size;
-      const bf16x4_t v0 = *reinterpret_cast<const bf16x4_t*>(v_base[0] + off);
-      const bf16x4_t v1 = *reinterpret_cast<const bf16x4_t*>(v_base[1] + off);
+      const bf16x4_t* from0 = reinterpret_cast<const bf16x4_t*>(v_base[0] + off);
+      const bf16x4_t* from1 = reinterpret_cast<const bf16x4_t*>(v_base[1] + off);
+      const bf16x4_t v0 = STREAM_KV ? __builtin_nontemporal_load(from0) : *from0;
+      const bf16x4_t v1 = STREAM_KV ? __builtin_nontemporal_load(from1) : *from1;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         v[db][i] = v0[i];
@@ -316,9 +324,15 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     }
 #pragma unroll
     for (int hlf = 0; hlf < 2; ++hlf) {
+      if constexpr (STREAM_KV) {
 #pragma unroll
-      for (int s = 0; s < KSTEPS; ++s)
-        blk.k[hlf][s] = *reinterpret_cast<const bf16x8_t*>(k_base[hlf] + (k_lane_off + s * 32));
+        for (int s = 0; s < KSTEPS; s += 2)
+          load_line_pair(k_base[hlf], s, k_line_lo, k_line_hi, blk.k[hlf][s], blk.k[hlf][s + 1]);
+      } else {
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+          blk.k[hlf][s] = *reinterpret_cast<const bf16x8_t*>(k_base[hlf] + (k_lane_off + s * 32));
+      }
     }
   };
 
@@ -443,6 +457,12 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   auto compute_block = [&](int kb, KVBlock& blk) {
     bf16x8_t v_late[DBLOCKS];
     load_values(blk.v_base, v_late);  // in flight during the scores and the softmax
+    if constexpr (STREAM_KV) {
+#pragma unroll
+      for (int hlf = 0; hlf < 2; ++hlf)
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s += 2) lines_to_operands(blk.k[hlf][s], blk.k[hlf][s + 1]);
+    }
     f32x4_t s_acc[RG][2];
     block_scores(blk, s_acc);
     bf16x8_t p_reg[RG];
@@ -786,6 +806,8 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
              head_dim, page_size);
   MI_REQUIRE(num_pages > 0 && max_blocks > 0, "attn_mfma: bad page counts num_pages=%d max_blocks=%d",
              num_pages, max_blocks);
+  MI_REQUIRE((uintptr_t)k_pages % 128 == 0 && (uintptr_t)vt_pages % 128 == 0,
+             "attn_mfma: the pages must begin on a 128-byte boundary (they are read in whole cache lines)");
   MI_REQUIRE(window >= 0, "attn_mfma: window=%d must be 0 (none) or positive", window);
   MI_REQUIRE(scale > 0.f, "attn_mfma: the score scale must be positive, got %g", (double)scale);
   MI_REQUIRE(num_splits >= 1 && num_splits <= 64, "attn_mfma: num_splits=%d must be 1..64", num_splits);
