@@ -294,7 +294,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   // once, so with non-temporal loads, and the keys in whole lines (lines_to_operands in
   // common.h; the values' 16 rows of 32 bytes per load are whole lines as they are).
   constexpr bool STREAM_KV = !SHARED && PS == 16 && D % 64 == 0;
-  const uint32_t k_line_lo = (uint32_t)((col % 8) * D * 2) + line_chunk_of_lane(lane);
+  const uint32_t k_line_lo = (uint32_t)(line_row_of_lane(lane) * D * 2) + line_chunk_of_lane(lane);
   const uint32_t k_line_hi = k_line_lo + 8u * D * 2u;
   auto load_values = [&](const bf16_t* const v_base[2], bf16x8_t* v) {
 #pragma unroll

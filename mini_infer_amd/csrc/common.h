@@ -56,32 +56,44 @@ typedef int int32x4_t __attribute__((ext_vector_type(4)));
 // operand wants, per k-step (32 elements), 16 bytes of each of 16 weight rows in every 16
 // lanes: four lanes a row, 64 bytes, half a cache line; the other half is asked for by the
 // next k-step's load.  Whole lines per load run faster, and non-temporal loads (the weights
-// are read once) faster again, but only on whole lines: measured on MI355X for 28672 x 4096,
-// 45.8 us on half lines, 47.5-50.1 us non-temporal on half lines, 42.3-44.7 us non-temporal
-// on whole lines; a long plain read reaches 6.1-6.3 TB/s, a non-temporal one 7.0-7.1 TB/s.
-// So a load takes 8 rows x 128 bytes (two k-steps): lane (quad, col) reads row col % 8 of
-// the tile's lower or upper 8 rows, 16-byte chunk quad + 4 * (col / 8) of the line.  Of a pair
-// of such loads (lower rows, upper rows) the lanes col >= 8 of the first and col < 8 of the
-// second change places, and the pair is the operands of the two k-steps.
+// are read once) faster again, but only on whole lines.  Measured on MI355X, microseconds for
+// 6144 x 4096 / 4096 x 14336 / 28672 x 4096 / 128256 x 4096 at 8 rows, weights not in any
+// cache: half lines 13.5 / 30.1 / 46.3 / 192; non-temporal on half lines slower (28672 x
+// 4096: 47.5-50.1 in a kernel that only reads); whole lines with every 16 lanes on 8 lines and
+// an exchange inside the 16 lanes 14.8 / 27.7 / 42.3 / 168; whole lines with every 8 lanes
+// on one line (this) 11.4 / 23.8 / 40.0 / 168.  A long plain read reaches 6.1-6.3 TB/s, a
+// non-temporal one 7.0-7.1 TB/s.
+// So a load takes 8 rows x 128 bytes (two k-steps): lane l reads 16-byte chunk l % 8 of the
+// line of row l / 8 of the tile's lower or upper 8 rows.  Of a pair of such loads (lower rows,
+// upper rows) the lanes with chunks 4-7 of the first and those with chunks 0-3 of the second
+// change places (inside every 16 lanes: two DPP moves), which sorts the chunks by k-step; then
+// every lane fetches its operand's 16 bytes from the lane that holds them (ds_bpermute, which
+// moves data between lanes through the LDS crossbar without touching LDS memory).
 // Needs: rows of the matrix on 128-byte boundaries, k-steps taken in even-aligned pairs.
 __device__ __forceinline__ void lines_to_operands(bf16x8_t& lower_rows, bf16x8_t& upper_rows) {
   int32x4_t lo = __builtin_bit_cast(int32x4_t, lower_rows), hi = __builtin_bit_cast(int32x4_t, upper_rows);
+  // operand lane (quad, col) wants row col, chunk quad of its k-step: after the exchange that
+  // is lane 8 * (col % 8) + 4 * (col / 8) + quad
+  const int lane = threadIdx.x % MI_WAVE, col = lane % 16, quad = lane / 16;
+  const int from = 4 * (8 * (col % 8) + 4 * (col / 8) + quad);
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int lo_was = lo[e];
-    // row_shr:8, lanes 8-15 of every 16: lane c takes the upper rows' lane c - 8 (row c, first k-step)
-    lo[e] = __builtin_amdgcn_update_dpp(lo[e], hi[e], 0x118, 0xF, 0xC, false);
-    // row_shl:8, lanes 0-7: lane c takes the lower rows' lane c + 8 (row c, second k-step)
-    hi[e] = __builtin_amdgcn_update_dpp(hi[e], lo_was, 0x108, 0xF, 0x3, false);
+    // row_shr:4 into lanes 4-7 and 12-15 of every 16: the upper rows' chunks 0-3 (first k-step)
+    lo[e] = __builtin_amdgcn_update_dpp(lo[e], hi[e], 0x114, 0xF, 0xA, false);
+    // row_shl:4 into lanes 0-3 and 8-11: the lower rows' chunks 4-7 (second k-step)
+    hi[e] = __builtin_amdgcn_update_dpp(hi[e], lo_was, 0x104, 0xF, 0x5, false);
+    lo[e] = __builtin_amdgcn_ds_bpermute(from, lo[e]);
+    hi[e] = __builtin_amdgcn_ds_bpermute(from, hi[e]);
   }
   lower_rows = __builtin_bit_cast(bf16x8_t, lo);  // operand of the pair's first k-step
   upper_rows = __builtin_bit_cast(bf16x8_t, hi);  // operand of its second
 }
 
-// The 16-byte chunk of its row's line that a lane reads, as a byte offset.
-__device__ __forceinline__ uint32_t line_chunk_of_lane(int lane) {
-  return (uint32_t)(lane / 16 + 4 * ((lane % 16) / 8)) * 16u;
-}
+// The row (0..7 of the lower or upper 8) whose line a lane reads, and its 16-byte chunk of
+// that line as a byte offset.
+__device__ __forceinline__ int line_row_of_lane(int lane) { return lane / 8; }
+__device__ __forceinline__ uint32_t line_chunk_of_lane(int lane) { return (uint32_t)(lane % 8) * 16u; }
 
 // The two loads of a pair of k-steps: base (uniform, kept in scalar registers) + the lane's offsets.
 template <bool STREAMED = true>

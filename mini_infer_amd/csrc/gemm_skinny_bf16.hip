@@ -98,7 +98,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   constexpr bool ADDNORM = EPI == EPI_ADDNORM;
   constexpr bool SCALED = PRO == PRO_SCALED;
   static_assert(!ROPE || NT == 1, "the rotary epilogue takes one tile of dims and its partner tile");
-  static_assert(!LINES || (U % 2 == 0 && PRO != PRO_ATTN), "whole lines are read for pairs of k-steps");
+  static_assert(!LINES || U % 2 == 0, "whole lines are read for pairs of k-steps");
   constexpr int WT = (GATED || ROPE) ? 2 * NT : NT;  // weight tiles per block
   __shared__ float red[SK_WAVES][WT][256];
 
@@ -142,8 +142,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   for (int t = 0; t < WT; ++t) {
     if constexpr (LINES) {
       const uint32_t chunk = line_chunk_of_lane(lane);
-      line_lo[t] = (uint32_t)weight_row(t, col % 8) * (uint32_t)(ldw * 2) + chunk;
-      line_hi[t] = (uint32_t)weight_row(t, 8 + col % 8) * (uint32_t)(ldw * 2) + chunk;
+      line_lo[t] = (uint32_t)weight_row(t, line_row_of_lane(lane)) * (uint32_t)(ldw * 2) + chunk;
+      line_hi[t] = (uint32_t)weight_row(t, 8 + line_row_of_lane(lane)) * (uint32_t)(ldw * 2) + chunk;
     } else {
       wp[t] = w + (int64_t)weight_row(t, col) * ldw + quad * 8;
     }
@@ -166,8 +166,13 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int t = 0; t < WT; ++t)
-          w_first[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[LINES ? 0 : t] + (int64_t)(s_begin + u) * 32);
+        for (int t = 0; t < WT; ++t) {
+          if constexpr (LINES) {
+            if (u % 2 == 0) load_lines(t, s_begin + u, w_first[u][t], w_first[u + 1][t]);
+          } else {
+            w_first[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[LINES ? 0 : t] + (int64_t)(s_begin + u) * 32);
+          }
+        }
     }
   }
   if constexpr (PRO == PRO_ATTN) {
@@ -243,7 +248,14 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
 #pragma unroll
       for (int t = 0; t < WT; ++t) {
         if constexpr (LINES) {
-          if (u % 2 == 0) load_lines(t, s + u, w_reg[u][t], w_reg[u + 1][t]);
+          if (u % 2 == 0) {
+            if (PRO == PRO_ATTN && first_ahead && s == s_begin) {
+              w_reg[u][t] = w_first[PRO == PRO_ATTN ? u : 0][t];
+              w_reg[u + 1][t] = w_first[PRO == PRO_ATTN ? u + 1 : 0][t];
+            } else {
+              load_lines(t, s + u, w_reg[u][t], w_reg[u + 1][t]);
+            }
+          }
         } else {
           if (PRO == PRO_ATTN && first_ahead && s == s_begin) w_reg[u][t] = w_first[PRO == PRO_ATTN ? u : 0][t];
           else w_reg[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[LINES ? 0 : t] + (int64_t)(s + u) * 32);
@@ -266,8 +278,10 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   }
   if constexpr (LINES) {
     for (; s + 2 <= s_end; s += 2) {  // fewer than U k-steps left: pair by pair (their number is even)
-      const bf16x8_t a_even = *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)s * 32);
-      const bf16x8_t a_odd = *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)(s + 1) * 32);
+      const bf16x8_t a_even = PRO == PRO_ATTN ? *reinterpret_cast<const bf16x8_t*>(own + (s - s_begin) * 32)
+                                              : *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)s * 32);
+      const bf16x8_t a_odd = PRO == PRO_ATTN ? *reinterpret_cast<const bf16x8_t*>(own + (s + 1 - s_begin) * 32)
+                                             : *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)(s + 1) * 32);
 #pragma unroll
       for (int t = 0; t < WT; ++t) {
         bf16x8_t w_even, w_odd;
@@ -555,12 +569,19 @@ extern "C" int mi_gemm_skinny_attn_bf16(const float* part_acc, const float* part
   const int fpb = features_per_block_for(n, cus, 4);
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
+  const bool lines = whole_lines(w, ldw, n, k);
+#define SK_ATTN(NT_, U_)                                                                                          \
+  if (lines)                                                                                                      \
+    gemm_skinny_bf16_kernel<NT_, U_, EPI_STORE, PRO_ATTN, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args); \
+  else                                                                                                            \
+    gemm_skinny_bf16_kernel<NT_, U_, EPI_STORE, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args)
   switch (ceil_div(fpb, 16)) {
-    case 1: gemm_skinny_bf16_kernel<1, 8, EPI_STORE, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args); break;
-    case 2: gemm_skinny_bf16_kernel<2, 8, EPI_STORE, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args); break;
-    case 3: gemm_skinny_bf16_kernel<3, 4, EPI_STORE, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args); break;
-    default: gemm_skinny_bf16_kernel<4, 2, EPI_STORE, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, args); break;
+    case 1: SK_ATTN(1, 8); break;
+    case 2: SK_ATTN(2, 8); break;
+    case 3: SK_ATTN(3, 4); break;
+    default: SK_ATTN(4, 2); break;
   }
+#undef SK_ATTN
   MI_CHECK_LAUNCH("gemm_skinny_attn_bf16");
   return MI_OK;
 }
@@ -617,7 +638,9 @@ extern "C" int mi_gemm_skinny_addnorm_bf16(const void* a, int64_t lda, const flo
   const int threads = 64 * SK_WAVES;
   const bool lines = whole_lines(w, ldw, n, k);
 #define SK_ADDNORM(NT_, U_)                                                                                        \
-  if (from_attention)                                                                                              \
+  if (from_attention && lines)                                                                                     \
+    gemm_skinny_bf16_kernel<NT_, U_, EPI_ADDNORM, PRO_ATTN, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldv, m, n, k, fpb, args); \
+  else if (from_attention)                                                                                         \
     gemm_skinny_bf16_kernel<NT_, U_, EPI_ADDNORM, PRO_ATTN><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldv, m, n, k, fpb, args); \
   else if (lines)                                                                                                  \
     gemm_skinny_bf16_kernel<NT_, U_, EPI_ADDNORM, PRO_NONE, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldv, m, n, k, fpb, args); \

@@ -376,28 +376,30 @@ PARTIAL_SUMS_MAX_ROWS = 128
 
 def partial_sums_pay(m: int, n: int, k: int) -> bool:
     """Whether a product of these sizes is left as sums over ranges of K when its caller
-    takes them (`linear(..., partial_ok=True)`).  Measured on MI355X, the product alone,
-    microseconds whole / in pieces at 8, 16, 32, 64 rows (whole = `gemm_skinny_bf16` up to
+    takes them (`linear(..., partial_ok=True)`).  Measured on MI355X, the product alone with
+    weights from memory, microseconds whole / in pieces (whole = `gemm_skinny_bf16` up to
     16 rows, the vendor library above):
 
-        4096 x 14336 (8B down)    30 / 24   37 / 25   34 / 25    39 / 28
-        8192 x 28672 (70B down)  101 / 86  120 / 86  101 / 89   144 / 100
-        3072 x 8192  (3B down)    15 / 18   18 / 18   17 / 20    23 / 22
-        4096 x 4096  (8B o)       10 / 10   11 / 10   13 / 11    15 / 13
-        3072 x 3072  (3B o)        8 / 8     9 / 8    11 / 9     16 / 11
-        8192 x 8192  (70B o)      29 / 36   33 / 36   31 / 38    34 / 40
+                                  8 rows    12 rows   16 rows   32 rows   64 rows
+        4096 x 14336 (8B down)    22 / 23   26 / 24   28 / 24   34 / 25   39 / 28
+        8192 x 28672 (70B down)   77 / 85   81 / 86   89 / 87  101 / 89  144 / 100
+        3072 x 8192  (3B down)    12 / 18   14 / 18   16 / 19   17 / 20   23 / 22
+        4096 x 4096  (8B o)        8 / 10    9 / 10   10 / 10   13 / 11   15 / 13
+        3072 x 3072  (3B o)        7 / 8     7 / 8     8 / 8    11 / 9    16 / 11
+        8192 x 8192  (70B o)      24 / 36   23 / 36   25 / 35   31 / 38   34 / 40
 
     and at 96 / 128 rows 63 / 75 against 36 / 39 (8B down), 22 / 24 against 16 / 18 (8B o),
     121 / 201 against 130 / 131 (70B down)
 
-    so: a long K from 5 rows on (with fewer rows the step as a whole ran 0.5 % slower this
-    way at 8B sizes), a small square-ish product from 12 rows on, nothing else.  Whole
-    steps at 8B sizes: batch 8 / 16 / 64 run 1.6 / 5 / 2.8 % faster."""
+    (the norm that adds the pieces up costs about a microsecond more than one that does not),
+    so: a long K from 11 rows on (15 with more than 4096 features), a small square-ish product
+    where the weight-streaming kernel ends (17 rows), nothing else.  Whole decode steps at 8B
+    sizes and 8 rows run 2.4 % faster with the down product whole, at 16 rows 2.6 % slower."""
     if not 5 <= m <= PARTIAL_SUMS_MAX_ROWS or n > 8192:
         return False
     if k >= 12288:
-        return True
-    return m >= 12 and n <= 4096 and 2048 <= k <= 4096
+        return m >= (11 if n <= 4096 else 15)
+    return m > SKINNY_MAX_ROWS and n <= 4096 and 2048 <= k <= 4096
 
 
 def linear_partial_sums(x: torch.Tensor, weight: torch.Tensor) -> PartialSums:

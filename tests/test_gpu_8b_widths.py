@@ -109,8 +109,8 @@ def test_single_tokens_over_a_longer_context_at_real_widths(wide, monkeypatch):
     """One request of 600 tokens, the last 10 one by one in bfloat16 through the replayed decode
     step: at these widths and this context a single token's attention is left in its key ranges
     and combined by the output projection (which also adds to the residual and begins the norm
-    that follows), and the down product is summed up by the next norm from 5 rows on (the
-    7-token portion)."""
+    that follows), and the down product is summed up by the next norm from 11 rows on (the
+    13-token portion)."""
     import mini_infer_amd.ops as ops
     from mini_infer_amd.engine import ModelRunner, StepEntry
     from mini_infer_amd.ops import kernels
@@ -130,10 +130,10 @@ def test_single_tokens_over_a_longer_context_at_real_widths(wide, monkeypatch):
     monkeypatch.setattr(kernels, "linear_partial_sums", count_partial_sums)
     folder, oracle = wide
     tokens = tiny.random_tokens(WIDE, 600, seed=5)
-    expected = oracle(tokens, rows=list(range(582, 600)))
+    expected = oracle(tokens, rows=list(range(576, 600)))
     runner = ModelRunner.from_pretrained(folder, dtype="bfloat16", num_blocks=40, block_size=16)
-    got = [runner.step([StepEntry("r", tokens[:583], [582])]).cpu().numpy()]
-    got.append(runner.step([StepEntry("r", tokens[583:590], list(range(7)))]).cpu().numpy())
+    got = [runner.step([StepEntry("r", tokens[:577], [576])]).cpu().numpy()]
+    got.append(runner.step([StepEntry("r", tokens[577:590], list(range(13)))]).cpu().numpy())
     for at in range(590, 600):
         got.append(runner.step([StepEntry("r", tokens[at : at + 1], [0])]).cpu().numpy())
     ru.assert_close(np.concatenate(got), expected, "bfloat16", "8B widths, 600 tokens")

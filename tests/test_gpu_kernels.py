@@ -175,10 +175,11 @@ def test_linear_leaves_partial_sums_only_where_asked_and_where_it_pays():
     from mini_infer_amd import ops
     from mini_infer_amd.exceptions import KernelShapeError
 
-    a, w = _rand(8, 12288, dtype=torch.bfloat16, seed=36), _rand(64, 12288, dtype=torch.bfloat16, seed=37, scale=0.05)
-    assert ops.partial_sums_pay(8, 64, 12288) and isinstance(ops.linear(a, w, partial_ok=True), ops.PartialSums)
+    a, w = _rand(12, 12288, dtype=torch.bfloat16, seed=36), _rand(64, 12288, dtype=torch.bfloat16, seed=37, scale=0.05)
+    assert ops.partial_sums_pay(12, 64, 12288) and isinstance(ops.linear(a, w, partial_ok=True), ops.PartialSums)
     assert isinstance(ops.linear(a, w), torch.Tensor)
-    assert not ops.partial_sums_pay(8, 64, 4096) and ops.partial_sums_pay(12, 64, 4096)
+    assert not ops.partial_sums_pay(8, 64, 12288) and not ops.partial_sums_pay(12, 8192, 12288) and ops.partial_sums_pay(15, 8192, 12288)
+    assert not ops.partial_sums_pay(16, 64, 4096) and ops.partial_sums_pay(17, 64, 4096)
     assert not ops.partial_sums_pay(4, 64, 12288) and not ops.partial_sums_pay(16, 3072, 8192)
     assert not ops.partial_sums_pay(129, 64, 12288) and not ops.partial_sums_pay(8, 28672, 12288)
     assert isinstance(ops.linear(a[:, :4096].contiguous(), w[:, :4096].contiguous(), partial_ok=True), torch.Tensor)
