@@ -23,7 +23,12 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define MID_KC 8  // k-steps of 32 per piece
 #define MID_AROW (MID_KC * 32 + 8)  // elements: rows 16 bytes apart in the banks, so 16 rows read side by side
 
-template <int MT>
+// LINES: the weights are read in whole cache lines (lines_to_operands in common.h), where the
+// matrix lies so that they can be.  Measured against half lines, microseconds at 16 / 64 / 128
+// rows: 4096 x 14336 23.4 / 28.0 / 41.5 against 23.7 / 28.3 / 39.6, 3072 x 8192 16.2 / 20.6 /
+// 31.6 against 18.5 / 22.3 / 30.7, 8192 x 28672 78 / 91 / 133 against 86 / 101 / 132: so up to
+// 64 rows.
+template <int MT, bool LINES>
 __global__ __launch_bounds__(64 * MID_WAVES) void gemm_mid_partial_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t ldw,
     float* __restrict__ part, int m, int n, int k, int pieces_per_range) {
@@ -34,7 +39,8 @@ __global__ __launch_bounds__(64 * MID_WAVES) void gemm_mid_partial_kernel(
   static_assert(A_IDS % THREADS == 0, "the activations' piece is shared out evenly");
   __shared__ __attribute__((aligned(16))) bf16_t a_lds[2][ROWS * MID_AROW];
 
-  const int wave = threadIdx.x / MI_WAVE;
+  // (with LINES made uniform for the compiler, so that the base address of the weight loads is scalar)
+  const int wave = LINES ? __builtin_amdgcn_readfirstlane(threadIdx.x / MI_WAVE) : threadIdx.x / MI_WAVE;
   const int lane = threadIdx.x % MI_WAVE;
   const int col = lane % 16, quad = lane / 16;
   const int n0 = blockIdx.x * (16 * MID_WAVES) + wave * 16;
@@ -45,6 +51,9 @@ __global__ __launch_bounds__(64 * MID_WAVES) void gemm_mid_partial_kernel(
 
   // weights: this lane reads feature n0 + col (past N: the last one, never stored), 8 consecutive k
   const bf16_t* wp = w + (int64_t)min(n0 + col, n - 1) * ldw + quad * 8;
+  // LINES: byte offsets of this lane's 16 bytes in the lower and upper 8 of the wave's rows
+  const uint32_t line_lo = (uint32_t)min(n0 + line_row_of_lane(lane), n - 1) * (uint32_t)(ldw * 2) + line_chunk_of_lane(lane);
+  const uint32_t line_hi = (uint32_t)min(n0 + 8 + line_row_of_lane(lane), n - 1) * (uint32_t)(ldw * 2) + line_chunk_of_lane(lane);
   // activations: chunk id -> (row, 16-byte part of the piece); rows past M repeat the last one
   const bf16_t* a_src[A_PER];
   int a_dst[A_PER];
@@ -70,8 +79,13 @@ __global__ __launch_bounds__(64 * MID_WAVES) void gemm_mid_partial_kernel(
     for (int j = 0; j < A_PER; ++j) *reinterpret_cast<bf16x8_t*>(&a_lds[buf][a_dst[j]]) = stage[j];
   };
   auto request_w = [&](int s0, bf16x8_t* regs) {
+    if constexpr (LINES) {  // (K holds an even number of k-steps and s0 is even)
 #pragma unroll
-    for (int u = 0; u < MID_KC; ++u) regs[u] = *reinterpret_cast<const bf16x8_t*>(wp + (int64_t)min(s0 + u, ksteps - 1) * 32);
+      for (int u = 0; u < MID_KC; u += 2) load_line_pair(w, min(s0 + u, ksteps - 2), line_lo, line_hi, regs[u], regs[u + 1]);
+    } else {
+#pragma unroll
+      for (int u = 0; u < MID_KC; ++u) regs[u] = *reinterpret_cast<const bf16x8_t*>(wp + (int64_t)min(s0 + u, ksteps - 1) * 32);
+    }
   };
 
   f32x4_t acc[MT];
@@ -92,6 +106,10 @@ __global__ __launch_bounds__(64 * MID_WAVES) void gemm_mid_partial_kernel(
       request_a(min(s0 + MID_KC, s_end - 1), a_stage);
       request_w(min(s0 + MID_KC, s_end - 1), w_next);
       const int steps = min(MID_KC, s_end - s0);
+      if constexpr (LINES) {  // what was requested a turn ago, as the operands of its k-steps
+#pragma unroll
+        for (int u = 0; u < MID_KC; u += 2) lines_to_operands(w_now[u], w_now[u + 1]);
+      }
 #pragma unroll
       for (int u = 0; u < MID_KC; ++u) {
         if (u < steps) {
@@ -160,13 +178,20 @@ extern "C" int mi_gemm_mid_partial_bf16(const void* a, int64_t lda, const void* 
   const int pieces = ceil_div(k / 32, MID_KC);
   const int per_range = ceil_div(pieces, ranges);
   const dim3 grid(ceil_div(n, 16 * MID_WAVES), ranges);
-#define MID_GO(MT_)                                                                                    \
-  gemm_mid_partial_kernel<MT_><<<grid, 64 * MID_WAVES, 0, stream>>>((const bf16_t*)a, lda, (const bf16_t*)w, ldw, \
-                                                                   part, m, n, k, per_range)
-  if (m <= 16) MID_GO(1);
-  else if (m <= 32) MID_GO(2);
-  else if (m <= 64) MID_GO(4);
-  else MID_GO(8);
+  // whole cache lines: rows of the matrix on 128-byte boundaries, an even number of k-steps,
+  // byte offsets into it that fit 32 bits
+  const bool lines = (uintptr_t)w % 128 == 0 && ldw % 64 == 0 && k % 64 == 0 && (int64_t)n * ldw * 2 < ((int64_t)1 << 32);
+#define MID_GO(MT_)                                                                                          \
+  if (lines)                                                                                                 \
+    gemm_mid_partial_kernel<MT_, true><<<grid, 64 * MID_WAVES, 0, stream>>>((const bf16_t*)a, lda, (const bf16_t*)w, ldw, \
+                                                                           part, m, n, k, per_range);         \
+  else                                                                                                       \
+    gemm_mid_partial_kernel<MT_, false><<<grid, 64 * MID_WAVES, 0, stream>>>((const bf16_t*)a, lda, (const bf16_t*)w, ldw, \
+                                                                            part, m, n, k, per_range)
+  if (m <= 16) { MID_GO(1); }
+  else if (m <= 32) { MID_GO(2); }
+  else if (m <= 64) { MID_GO(4); }
+  else gemm_mid_partial_kernel<8, false><<<grid, 64 * MID_WAVES, 0, stream>>>((const bf16_t*)a, lda, (const bf16_t*)w, ldw, part, m, n, k, per_range);
 #undef MID_GO
   MI_CHECK_LAUNCH("gemm_mid_partial_bf16");
   return MI_OK;
