@@ -727,24 +727,28 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
 // cache write in its last step: q_out[m, q_heads*head_dim] gets the rotated queries, the
 // rotated keys and the values go to their slots (slot_mapping[m]; kv_heads = 0: queries only,
 // w then holds the query rows alone).  Half-paired rotation over the whole head,
-// cos/sin [m, head_dim/2] float32.
-extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* q_out,
-                                        int64_t ldq, const float* cos_t, const float* sin_t,
-                                        const int* slot_mapping, void* k_pages, void* v_pages, int m, int k,
-                                        int q_heads, int kv_heads, int head_dim, int page_size, int num_pages,
-                                        int v_transposed, hipStream_t stream) {
+// cos/sin [m, head_dim/2] float32.  With `sumsq` the rows are a norm's output but for the
+// rows' factors (PRO_SCALED, as in mi_gemm_skinny_swiglu_scaled_bf16).
+static int rope_product(const char* name, const void* a, int64_t lda, const float* sumsq, int pieces, float eps,
+                        const void* w, int64_t ldw, void* q_out, int64_t ldq, const float* cos_t,
+                        const float* sin_t, const int* slot_mapping, void* k_pages, void* v_pages, int m, int k,
+                        int q_heads, int kv_heads, int head_dim, int page_size, int num_pages, int v_transposed,
+                        hipStream_t stream) {
   MI_REQUIRE(q_heads >= 1 && kv_heads >= 0 && head_dim >= 32 && head_dim % 32 == 0,
-             "gemm_skinny_rope_bf16: takes head_dim a multiple of 32; got q_heads=%d kv_heads=%d head_dim=%d",
-             q_heads, kv_heads, head_dim);
+             "%s: takes head_dim a multiple of 32; got q_heads=%d kv_heads=%d head_dim=%d", name, q_heads, kv_heads,
+             head_dim);
   const int n = (q_heads + 2 * kv_heads) * head_dim;
   MI_REQUIRE(mi_gemm_skinny_bf16_supported(m, n, k, lda, ldw),
-             "gemm_skinny_rope_bf16: takes 1 <= m <= 16, k a multiple of 32, rows aligned to 16 bytes; "
-             "got m=%d n=%d k=%d lda=%lld ldw=%lld", m, n, k, (long long)lda, (long long)ldw);
+             "%s: takes 1 <= m <= 16, k a multiple of 32, rows aligned to 16 bytes; "
+             "got m=%d n=%d k=%d lda=%lld ldw=%lld", name, m, n, k, (long long)lda, (long long)ldw);
   MI_REQUIRE(lda >= k && ldw >= k && ldq >= (int64_t)q_heads * head_dim && ldq % 4 == 0,
-             "gemm_skinny_rope_bf16: a row stride is shorter than its row or not 8-byte aligned");
-  MI_REQUIRE(cos_t && sin_t, "gemm_skinny_rope_bf16: needs the rotation tables");
+             "%s: a row stride is shorter than its row or not 8-byte aligned", name);
+  MI_REQUIRE(cos_t && sin_t, "%s: needs the rotation tables", name);
   MI_REQUIRE(kv_heads == 0 || (slot_mapping && k_pages && v_pages && page_size > 0 && num_pages > 0),
-             "gemm_skinny_rope_bf16: pages and slots are needed to write keys and values");
+             "%s: pages and slots are needed to write keys and values", name);
+  MI_REQUIRE(!sumsq || (pieces >= 1 && pieces <= SK_SCALE_PARTS * SK_SCALE_PIECES && eps >= 0.f),
+             "%s: needs the rows' sums of squares in 1..%d pieces, got %d", name, SK_SCALE_PARTS * SK_SCALE_PIECES,
+             pieces);
   FoldArgs fold = {};
   fold.cos_t = cos_t;
   fold.sin_t = sin_t;
@@ -756,20 +760,52 @@ extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* 
   fold.head_dim = head_dim;
   fold.page_size = page_size;
   fold.v_transposed = v_transposed;
+  fold.sumsq_in = sumsq;
+  fold.sumsq_pieces = pieces;
+  fold.norm_eps = eps;
+  fold.norm_width = k;
   // pairs per block: an even share over the CUs in whole rounds, as for the plain product
   const int cus = compute_units();
-  MI_REQUIRE(cus > 0, "gemm_skinny_rope_bf16: cannot read the device's compute unit count");
+  MI_REQUIRE(cus > 0, "%s: cannot read the device's compute unit count", name);
   const int total_pairs = n / 2;
   const int rounds = ceil_div(total_pairs, cus * 16);
   int pairs_per_block = ceil_div(ceil_div(total_pairs, cus * rounds), 4) * 4;
   if (pairs_per_block > 16) pairs_per_block = 16;
   const int blocks = ceil_div(total_pairs, pairs_per_block);
-  if (whole_lines(w, ldw, n, k))
-    gemm_skinny_bf16_kernel<1, 8, EPI_ROPE, PRO_NONE, true><<<blocks, 64 * SK_WAVES, 0, stream>>>(
-        (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, pairs_per_block, fold);
-  else
-    gemm_skinny_bf16_kernel<1, 8, EPI_ROPE><<<blocks, 64 * SK_WAVES, 0, stream>>>(
-        (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, pairs_per_block, fold);
-  MI_CHECK_LAUNCH("gemm_skinny_rope_bf16");
+  const bool lines = whole_lines(w, ldw, n, k);
+#define SK_ROPE(PRO_, LINES_)                                                                  \
+  gemm_skinny_bf16_kernel<1, 8, EPI_ROPE, PRO_, LINES_><<<blocks, 64 * SK_WAVES, 0, stream>>>( \
+      (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, pairs_per_block, fold)
+  if (sumsq) {
+    if (lines) SK_ROPE(PRO_SCALED, true); else SK_ROPE(PRO_SCALED, false);
+  } else {
+    if (lines) SK_ROPE(PRO_NONE, true); else SK_ROPE(PRO_NONE, false);
+  }
+#undef SK_ROPE
+  MI_CHECK_LAUNCH(name);
   return MI_OK;
+}
+
+extern "C" int mi_gemm_skinny_rope_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* q_out,
+                                        int64_t ldq, const float* cos_t, const float* sin_t,
+                                        const int* slot_mapping, void* k_pages, void* v_pages, int m, int k,
+                                        int q_heads, int kv_heads, int head_dim, int page_size, int num_pages,
+                                        int v_transposed, hipStream_t stream) {
+  return rope_product("gemm_skinny_rope_bf16", a, lda, nullptr, 0, 0.f, w, ldw, q_out, ldq, cos_t, sin_t, slot_mapping,
+                      k_pages, v_pages, m, k, q_heads, kv_heads, head_dim, page_size, num_pages, v_transposed, stream);
+}
+
+// The same on rows whose norm factor is still apart: a = the values of mi_gemm_skinny_addnorm_bf16,
+// sumsq[pieces][m] its sums of squares; the products are multiplied with
+// rsqrt(sum of the row's pieces / k + eps) before they are rounded and rotated.
+extern "C" int mi_gemm_skinny_rope_scaled_bf16(const void* a, int64_t lda, const float* sumsq, int pieces, float eps,
+                                               const void* w, int64_t ldw, void* q_out, int64_t ldq,
+                                               const float* cos_t, const float* sin_t, const int* slot_mapping,
+                                               void* k_pages, void* v_pages, int m, int k, int q_heads,
+                                               int kv_heads, int head_dim, int page_size, int num_pages,
+                                               int v_transposed, hipStream_t stream) {
+  MI_REQUIRE(sumsq, "gemm_skinny_rope_scaled_bf16: needs the rows' sums of squares");
+  return rope_product("gemm_skinny_rope_scaled_bf16", a, lda, sumsq, pieces, eps, w, ldw, q_out, ldq, cos_t, sin_t,
+                      slot_mapping, k_pages, v_pages, m, k, q_heads, kv_heads, head_dim, page_size, num_pages,
+                      v_transposed, stream);
 }

@@ -44,6 +44,15 @@ class DecoderModel:
         if self.final_norm.takes_partial_sums and all(block.takes_partial_sums for block in self.blocks):
             for block in self.blocks:
                 block.enable_partial_sums()
+        # a block may hand its last product on unmade where whatever follows it, at every place
+        # it has in the order, takes such a product
+        followers: dict[int, list] = {}
+        for i, call in enumerate(spec.order):
+            after = self.blocks[spec.order[i + 1].layer] if i + 1 < len(spec.order) else self.final_norm
+            followers.setdefault(call.layer, []).append(after)
+        for layer, after in followers.items():
+            if all(part.takes_pending_products for part in after):
+                self.blocks[layer].enable_pending_output()
 
     @property
     def graph_safe(self) -> bool:

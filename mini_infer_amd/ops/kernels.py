@@ -465,9 +465,26 @@ def linear(x: torch.Tensor, weight: torch.Tensor, partial_ok: bool = False) -> t
     return torch.matmul(x, weight.t())
 
 
-def qkv_rope_write_takes(x: torch.Tensor, weight: torch.Tensor, head_dim: int, rotary_dim: int, interleaved: bool) -> bool:
+def _scaled_rows_fit(x: "ScaledRows") -> bool:
+    """Whether a product's kernel can apply the rows' factors of `x` itself."""
+    return (
+        x.values.dtype == torch.bfloat16
+        and x.values.dim() == 2
+        and x.values.shape[0] <= PENDING_PRODUCT_MAX_ROWS
+        and x.sumsq.is_contiguous()
+        and x.sumsq.shape[0] <= SCALED_ROWS_MAX_PIECES
+    )
+
+
+def qkv_rope_write_takes(
+    x: "torch.Tensor | ScaledRows", weight: torch.Tensor, head_dim: int, rotary_dim: int, interleaved: bool
+) -> bool:
     """Whether `qkv_rope_write` runs these operands: at most 16 bfloat16 rows, rotation of
     whole heads in half pairing, head size a multiple of 32."""
+    if isinstance(x, ScaledRows):
+        if not _scaled_rows_fit(x):
+            return False
+        x = x.values
     return (
         x.dtype == torch.bfloat16
         and weight.dtype == torch.bfloat16
@@ -482,7 +499,7 @@ def qkv_rope_write_takes(x: torch.Tensor, weight: torch.Tensor, head_dim: int, r
 
 
 def qkv_rope_write(
-    x: torch.Tensor,
+    x: "torch.Tensor | ScaledRows",
     weight: torch.Tensor,
     cos: torch.Tensor,
     sin: torch.Tensor,
@@ -501,13 +518,18 @@ def qkv_rope_write(
     queries [M, q_heads*head_dim]; rotated keys and values go to their slots.  `kv_heads=0`
     with the query rows of the weight alone projects and rotates queries only.  The result
     is that of `linear` followed by `rope_kv_write` (both round the product to bfloat16
-    before rotating).
+    before rotating).  `x` may be `ScaledRows`: the rows' factors are then applied to the
+    products' sums before they are rounded.
     """
+    scaled = x if isinstance(x, ScaledRows) else None
+    if scaled is not None:
+        x = scaled.values
+        _need_cuda(scaled.sumsq)
     _need_cuda(x, weight, cos, sin, slot_mapping, k_pages, v_pages)
     for name, t in (("cos", cos), ("sin", sin), ("slot_mapping", slot_mapping), ("k_pages", k_pages), ("v_pages", v_pages)):
         _need_contiguous(name, t)
     _need_int32("slot_mapping", slot_mapping)
-    if not qkv_rope_write_takes(x, weight, head_dim, head_dim, False):
+    if not qkv_rope_write_takes(scaled if scaled is not None else x, weight, head_dim, head_dim, False):
         raise KernelShapeError(
             f"qkv_rope_write takes at most 16 bfloat16 rows and head sizes in steps of 32; got "
             f"x {tuple(x.shape)} {x.dtype}, head_dim={head_dim}"
@@ -533,14 +555,18 @@ def qkv_rope_write(
         num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
     q_out = torch.empty((m, q_heads * head_dim), dtype=torch.bfloat16, device=x.device)
     lib = library.load()
-    library.check(
-        lib.mi_gemm_skinny_rope_bf16(
-            _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(q_out), q_out.stride(0), _ptr(cos), _ptr(sin),
-            _ptr(slot_mapping) if kv_heads > 0 else None, _ptr(k_pages) if kv_heads > 0 else None,
-            _ptr(v_pages) if kv_heads > 0 else None, m, k, q_heads, kv_heads, head_dim, page_size, num_pages,
-            int(v_transposed), _stream(),
-        )
+    rest = (
+        _ptr(weight), weight.stride(0), _ptr(q_out), q_out.stride(0), _ptr(cos), _ptr(sin),
+        _ptr(slot_mapping) if kv_heads > 0 else None, _ptr(k_pages) if kv_heads > 0 else None,
+        _ptr(v_pages) if kv_heads > 0 else None, m, k, q_heads, kv_heads, head_dim, page_size, num_pages,
+        int(v_transposed), _stream(),
     )
+    if scaled is not None:
+        library.check(
+            lib.mi_gemm_skinny_rope_scaled_bf16(_ptr(x), x.stride(0), _ptr(scaled.sumsq), scaled.sumsq.shape[0], scaled.eps, *rest)
+        )
+    else:
+        library.check(lib.mi_gemm_skinny_rope_bf16(_ptr(x), x.stride(0), *rest))
     return q_out
 
 
@@ -561,14 +587,11 @@ def linear_swiglu(x: "torch.Tensor | ScaledRows", gate_up_weight: torch.Tensor) 
     if isinstance(x, ScaledRows):
         values = x.values
         if (
-            values.dtype == torch.bfloat16
+            _scaled_rows_fit(x)
             and gate_up_weight.dtype == torch.bfloat16
             and values.shape[1] == width
             and values.stride(1) == 1
             and gate_up_weight.stride(1) == 1
-            and x.sumsq.is_contiguous()
-            and x.sumsq.shape[0] <= SCALED_ROWS_MAX_PIECES
-            and values.shape[0] <= PENDING_PRODUCT_MAX_ROWS
             and skinny_gemm_takes(values.shape[0], width, values.stride(0), gate_up_weight.stride(0))
         ):
             scaled, x = x, values
@@ -685,6 +708,13 @@ PENDING_PRODUCT_MAX_ROWS = 16  # rows up to which a product is worth handing on 
 SCALED_ROWS_MAX_PIECES = 256  # pieces of a row's sum of squares the consuming kernel adds up
 
 
+def pending_product_pays(rows: int, n: int, k: int, partial_ok: bool) -> bool:
+    """Whether a part hands its last product [rows, k] x [n, k] on unmade (`PendingProduct`)
+    instead of making it: few rows, and not where the product is better left as sums over
+    ranges of K (`partial_sums_pay`, if its caller takes those)."""
+    return rows <= PENDING_PRODUCT_MAX_ROWS and not (partial_ok and partial_sums_pay(rows, n, k))
+
+
 @dataclasses.dataclass
 class PendingProduct:
     """`x @ weight.T` that has not been made yet: a part's contribution to the residual stream,
@@ -707,7 +737,7 @@ class ScaledRows:
     weight (rounded to the element type), `sumsq` [pieces, T] float32 = sums of squares of
     the residual rows over `pieces` ranges of H.  Row t is still to be multiplied with
     rsqrt(sum(sumsq[:, t]) / H + eps); a product that consumes the rows does that to its own
-    sums instead (`linear_swiglu`), since the factor commutes with the product.  Anything
+    sums instead (`linear_swiglu`, `qkv_rope_write`), since the factor commutes with the product.  Anything
     else calls `finish()`."""
 
     values: torch.Tensor

@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -42,6 +42,10 @@ _SIGNATURES: dict[str, list] = {
     "mi_gemm_skinny_rope_bf16": [
         _P, c_int64, _P, c_int64, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
         c_int, c_int, _P,
+    ],
+    "mi_gemm_skinny_rope_scaled_bf16": [
+        _P, c_int64, _P, c_int, c_float, _P, c_int64, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
+        c_int, c_int, c_int, c_int, _P,
     ],
     "mi_gemm_skinny_bf16_supported": [c_int, c_int, c_int, c_int64, c_int64],
     "mi_attn_generic": [

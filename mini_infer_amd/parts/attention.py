@@ -32,6 +32,7 @@ from mini_infer_amd.registry import POSITION_ENCODINGS, register_mixer
 class GQAttention(Mixer):
     graph_safe = True
     can_defer_output = True
+    takes_scaled_rows = True
 
     def __init__(
         self,
@@ -95,6 +96,11 @@ class GQAttention(Mixer):
         q_width = self.num_heads * self.head_dim
         assert self.qkv.weight is not None
         rotary = self.position.rotary(ctx) if self.position is not None else None
+        if isinstance(x, ops.ScaledRows) and not (
+            rotary is not None
+            and ops.qkv_rope_write_takes(x, self.qkv.weight, self.head_dim, rotary.rotary_dim, rotary.interleaved)
+        ):
+            x = x.finish()  # rows but for their norm factors, and no kernel here that applies them
         if rotary is not None and ops.qkv_rope_write_takes(
             x, self.qkv.weight, self.head_dim, rotary.rotary_dim, rotary.interleaved
         ):
@@ -132,7 +138,8 @@ class GQAttention(Mixer):
         assert self.out.weight is not None
         if self.emit_pending_output and self.dtype == torch.bfloat16:
             rows = attended.tokens if isinstance(attended, ops.AttentionPieces) else attended.shape[0]
-            if rows <= ops.PENDING_PRODUCT_MAX_ROWS:
+            q_width = self.num_heads * self.head_dim
+            if ops.pending_product_pays(rows, self.hidden_size, q_width, self.emit_partial_sums):
                 return ops.PendingProduct(attended, self.out.weight)
         if isinstance(attended, ops.AttentionPieces):
             return ops.linear_from_attention(attended, self.out.weight)

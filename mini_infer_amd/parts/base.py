@@ -229,11 +229,14 @@ class Mixer(Part):
     return an `ops.PartialSums` instead of a tensor (parts that ignore it are fine).
     `emit_pending_output` is set by the block where the norm that follows says
     `takes_pending_products` and the mixer `can_defer_output`: `forward` may then return an
-    `ops.PendingProduct` (its last product, not made yet) instead of a tensor."""
+    `ops.PendingProduct` (its last product, not made yet) instead of a tensor.
+    `takes_scaled_rows`: `x` may be an `ops.ScaledRows` (a norm's output but for the rows'
+    factors); the block then lets the norm before the mixer emit them."""
 
     emit_partial_sums = False
     can_defer_output = False
     emit_pending_output = False
+    takes_scaled_rows = False
 
     def cache_needs(self, page_size: int) -> CacheNeeds:
         """What the cache manager must keep for one call of this mixer, given its page size
@@ -249,10 +252,14 @@ class Mixer(Part):
 class FeedForward(Part):
     """Acts on each token alone: dense or routed experts.  `emit_partial_sums`: as for `Mixer`.
     `takes_scaled_rows`: `x` may be an `ops.ScaledRows` (a norm's output but for the rows'
-    factors)."""
+    factors).  `can_defer_output`, `emit_pending_output`: as for `Mixer`; here it is the
+    model that sets the latter (`Block.enable_pending_output`), since the norm that follows
+    belongs to whatever comes next in the model's order."""
 
     emit_partial_sums = False
     takes_scaled_rows = False
+    can_defer_output = False
+    emit_pending_output = False
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
@@ -294,6 +301,15 @@ class Block(Part):
     takes_partial_sums = False
 
     def enable_partial_sums(self) -> None:
+        pass
+
+    # Whether the block's `delta` may be an `ops.PendingProduct` (the previous block's last
+    # product, not made yet).  Where everything that follows a block in the model's order (the
+    # blocks after it, the final norm after the last) says so, the model calls the block's
+    # `enable_pending_output()`, which lets its last part hand its last product on unmade.
+    takes_pending_products = False
+
+    def enable_pending_output(self) -> None:
         pass
 
     def forward(

@@ -46,6 +46,11 @@ class PreNormBlock(Block):
         if mixer.can_defer_output and ffn_norm.takes_pending_products and feed_forward.takes_scaled_rows:
             mixer.emit_pending_output = True
             ffn_norm.emit_scaled_rows = True
+        # The same between the block before this one and this block's mixer: its first norm may
+        # be handed a product not made yet (if the model arranges that, `enable_pending_output`
+        # of the block before), and leaves the rows' factors to the mixer's first product.
+        if mixer_norm.takes_pending_products and mixer.takes_scaled_rows:
+            mixer_norm.emit_scaled_rows = True
 
     @property
     def graph_safe(self) -> bool:  # type: ignore[override]
@@ -58,6 +63,14 @@ class PreNormBlock(Block):
     def enable_partial_sums(self) -> None:
         self.mixer.emit_partial_sums = True
         self.feed_forward.emit_partial_sums = True
+
+    @property
+    def takes_pending_products(self) -> bool:  # type: ignore[override]
+        return self.mixer_norm.takes_pending_products
+
+    def enable_pending_output(self) -> None:
+        if self.feed_forward.can_defer_output:
+            self.feed_forward.emit_pending_output = True
 
     def _children(self):
         return (

@@ -20,6 +20,7 @@ from mini_infer_amd.registry import register_feed_forward
 class SwiGLU(FeedForward):
     graph_safe = True
     takes_scaled_rows = True
+    can_defer_output = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, dtype: torch.dtype, device) -> None:
         super().__init__(dtype, device)
@@ -39,7 +40,17 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: "torch.Tensor | ops.ScaledRows", ctx: StepContext) -> torch.Tensor:
         assert self.gate_up.weight is not None, "SwiGLU used before its weights were loaded"
-        return self.down.forward(ops.linear_swiglu(x, self.gate_up.weight), partial_ok=self.emit_partial_sums)
+        assert self.down.weight is not None
+        act = ops.linear_swiglu(x, self.gate_up.weight)
+        if (
+            self.emit_pending_output
+            and self.dtype == torch.bfloat16
+            and ops.pending_product_pays(act.shape[0], self.hidden_size, self.intermediate_size, self.emit_partial_sums)
+        ):
+            # few rows: the down product is left to the norm that follows (one kernel makes it,
+            # adds it to the residual and begins the norm)
+            return ops.PendingProduct(act, self.down.weight)
+        return self.down.forward(act, partial_ok=self.emit_partial_sums)
 
 
 @register_feed_forward("swiglu")

@@ -109,24 +109,32 @@ def test_single_tokens_over_a_longer_context_at_real_widths(wide, monkeypatch):
     """One request of 600 tokens, the last 10 one by one in bfloat16 through the replayed decode
     step: at these widths and this context a single token's attention is left in its key ranges
     and combined by the output projection (which also adds to the residual and begins the norm
-    that follows), and the down product is summed up by the next norm from 11 rows on (the
-    13-token portion)."""
+    that follows), the down product of a layer that another follows is left to that layer's first
+    norm and q|k|v product, and the down product is summed up by the next norm from 11 rows on
+    (the 13-token portion)."""
     import mini_infer_amd.ops as ops
     from mini_infer_amd.engine import ModelRunner, StepEntry
     from mini_infer_amd.ops import kernels
 
-    calls = {"from_attention": 0, "partial_sums": 0}
-    add_norm, partial_sums = ops.linear_add_norm, kernels.linear_partial_sums
+    calls = {"from_attention": 0, "from_feed_forward": 0, "partial_sums": 0, "scaled_q_k_v": 0}
+    add_norm, partial_sums, rope_write = ops.linear_add_norm, kernels.linear_partial_sums, ops.qkv_rope_write
 
     def count_from_attention(pending, *args):
         calls["from_attention"] += isinstance(pending.x, ops.AttentionPieces)
+        # (a feed-forward's down product handed to the next layer's first norm)
+        calls["from_feed_forward"] += isinstance(pending.x, torch.Tensor) and pending.weight.shape[1] == WIDE["intermediate_size"]
         return add_norm(pending, *args)
+
+    def count_scaled_rows(x, *args, **kwargs):
+        calls["scaled_q_k_v"] += isinstance(x, ops.ScaledRows)
+        return rope_write(x, *args, **kwargs)
 
     def count_partial_sums(*args):
         calls["partial_sums"] += 1
         return partial_sums(*args)
 
     monkeypatch.setattr(ops, "linear_add_norm", count_from_attention)
+    monkeypatch.setattr(ops, "qkv_rope_write", count_scaled_rows)
     monkeypatch.setattr(kernels, "linear_partial_sums", count_partial_sums)
     folder, oracle = wide
     tokens = tiny.random_tokens(WIDE, 600, seed=5)
@@ -138,6 +146,7 @@ def test_single_tokens_over_a_longer_context_at_real_widths(wide, monkeypatch):
         got.append(runner.step([StepEntry("r", tokens[at : at + 1], [0])]).cpu().numpy())
     ru.assert_close(np.concatenate(got), expected, "bfloat16", "8B widths, 600 tokens")
     assert calls["from_attention"] >= 1 and calls["partial_sums"] >= 1  # (a replayed step calls nothing)
+    assert calls["from_feed_forward"] >= 1 and calls["scaled_q_k_v"] == calls["from_feed_forward"]
     assert runner.decode_graphs.replays == 10
     runner.free_request("r")
     assert runner.num_free_blocks() == 40

@@ -711,6 +711,79 @@ def test_product_add_and_norm_from_uncombined_key_ranges(q_heads, kv_heads, head
     assert (rows.finish().float() - normed.float()).abs().max() <= 2.0 ** -6 * float(normed.float().abs().max())
 
 
+@pytest.mark.parametrize("v_transposed", [False, True])
+@pytest.mark.parametrize(
+    "m,inter,hidden,q_heads,kv_heads,head_dim",
+    [(8, 14336, 4096, 32, 8, 128), (1, 14336, 4096, 32, 8, 128), (16, 160, 96, 3, 1, 32), (5, 320, 160, 6, 2, 64), (3, 1536, 1536, 6, 2, 64)],
+)
+def test_down_product_add_and_norm_folded_into_the_next_q_k_v_product(v_transposed, m, inter, hidden, q_heads, kv_heads, head_dim):
+    """`linear_add_norm` on a feed-forward's last product, then `qkv_rope_write` on its
+    `ScaledRows`, against the three kernels they replace (product, add + norm, q|k|v with
+    rotation and cache write): the residual bit for bit, queries, keys and values as two
+    bfloat16 roundings of the same numbers agree, and against float64."""
+    from mini_infer_amd import ops
+
+    page_size, num_pages = 16, 5
+    width = (q_heads + 2 * kv_heads) * head_dim
+    act = _rand(m, inter, dtype=torch.bfloat16, seed=71)
+    down = _rand(hidden, inter, dtype=torch.bfloat16, seed=72, scale=0.05)
+    norm_w = (torch.rand(hidden, generator=torch.Generator().manual_seed(73)) + 0.5).bfloat16().to(DEV)
+    qkv_w = _rand(width, hidden, dtype=torch.bfloat16, seed=74, scale=0.1)
+    residual0 = _rand(m, hidden, dtype=torch.float32, seed=75)
+    positions = torch.tensor([0, 1, 700, 5, 131071, 17, 18, 19, 3000, 2, 4, 6, 8, 10, 12, 14][:m], dtype=torch.int32, device=DEV)
+    cos, sin = ops.rope_table(positions, torch.from_numpy(pl.inv_freq_default(head_dim, 500000.0)).to(DEV))
+    slots = torch.tensor([40, 3, 17, 16, 0, 43, -1, 9, 22, 5, 6, 7, 30, 31, 32, 33][:m], dtype=torch.int32, device=DEV)
+    eps = 2e-5
+
+    def pages():
+        k = torch.full((num_pages, kv_heads, page_size, head_dim), 7.0, dtype=torch.bfloat16, device=DEV)
+        v_shape = (num_pages, kv_heads, head_dim, page_size) if v_transposed else k.shape
+        return k, torch.full(v_shape, 7.0, dtype=torch.bfloat16, device=DEV)
+
+    heads = dict(q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, v_transposed=v_transposed)
+    apart_residual = residual0.clone()
+    normed = ops.add_rmsnorm(ops.linear(act, down), apart_residual, norm_w, eps)
+    k_apart, v_apart = pages()
+    q_apart = ops.qkv_rope_write(normed, qkv_w, cos, sin, slots, k_apart, v_apart, **heads)
+
+    residual = residual0.clone()
+    rows = ops.linear_add_norm(ops.PendingProduct(act, down), residual, norm_w, eps)
+    assert torch.equal(residual, apart_residual)
+    assert ops.qkv_rope_write_takes(rows, qkv_w, head_dim, head_dim, False)
+    k_fold, v_fold = pages()
+    q_fold = ops.qkv_rope_write(rows, qkv_w, cos, sin, slots, k_fold, v_fold, **heads)
+
+    # float64: the norm of the float32 residual the kernels left, the product rounded once, the rotation
+    exact_sumsq = (residual.double() ** 2).sum(dim=1)
+    exact_normed = residual.double() * torch.rsqrt(exact_sumsq / hidden + eps)[:, None] * norm_w.double()
+    qkv = (exact_normed @ qkv_w.double().T).bfloat16().double().view(m, q_heads + 2 * kv_heads, head_dim)
+    half = head_dim // 2
+    c, s_ = cos.double()[:, None, :], sin.double()[:, None, :]
+    rotated = torch.cat([qkv[..., :half] * c - qkv[..., half:] * s_, qkv[..., half:] * c + qkv[..., :half] * s_], dim=-1)
+    exact_q = rotated[:, :q_heads].reshape(m, q_heads * head_dim)
+    bound = 2.0 ** -5 * float(exact_q.abs().max()) + 1e-6
+    assert (q_fold.double() - exact_q).abs().max() < bound
+    assert (q_apart.double() - exact_q).abs().max() < bound  # (the yardstick: the three kernels are no closer)
+    for row in range(m):
+        slot = int(slots[row])
+        if slot < 0:
+            continue
+        page, off = divmod(slot % (num_pages * page_size), page_size)
+        exact_k = rotated[row, q_heads : q_heads + kv_heads]
+        exact_v = qkv[row, q_heads + kv_heads :]
+        got_v = v_fold[page, :, :, off] if v_transposed else v_fold[page, :, off]
+        assert (k_fold[page, :, off].double() - exact_k).abs().max() < bound
+        assert (got_v.double() - exact_v).abs().max() < bound
+    # slots nobody wrote keep what they held, in both ways of running
+    written = torch.zeros(num_pages * page_size, dtype=torch.bool, device=DEV)
+    written[slots[slots >= 0].long()] = True
+    untouched = ~written.view(num_pages, page_size)
+    assert torch.all(k_fold.permute(0, 2, 1, 3)[untouched] == 7.0) and torch.all(k_apart.permute(0, 2, 1, 3)[untouched] == 7.0)
+    # rows that meet a product without such a kernel are finished first: the same function
+    many = ops.ScaledRows(rows.values.float(), rows.sumsq, eps)
+    assert not ops.qkv_rope_write_takes(many, qkv_w.float(), head_dim, head_dim, False)
+
+
 def test_kernels_refuse_what_they_do_not_take():
     from mini_infer_amd import ops
     from mini_infer_amd.exceptions import KernelShapeError
