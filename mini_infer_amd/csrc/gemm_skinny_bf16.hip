@@ -235,6 +235,24 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     }
   }
 
+  // PRO_SCALED: SK_SCALE_PARTS threads per row each add up every SK_SCALE_PARTS-th piece of the
+  // row's sum of squares, in a fixed order.  Where the loop below leaves registers to spare the
+  // pieces are asked for before it, so that the trip to them is over when it ends (whole decode
+  // steps 0.9-1.3 % faster); with four weight tiles they would cost the registers of a resident
+  // block per CU (measured: 16 % slower), and are asked for after it.  (Capping the registers
+  // of the variants just above 80 at 80 measured 0.8-1.4 % slower.)
+  constexpr bool SCALE_EARLY = SCALED && WT <= 2;
+  float scale_piece[SCALED ? SK_SCALE_PIECES : 1];
+  auto load_scale_pieces = [&]() {
+    const int row = threadIdx.x % 16, part = threadIdx.x / 16;
+#pragma unroll
+    for (int i = 0; i < SK_SCALE_PIECES; ++i) {
+      const int piece = part + i * SK_SCALE_PARTS;
+      scale_piece[SCALED ? i : 0] = (row < m && piece < fold.sumsq_pieces) ? fold.sumsq_in[(int64_t)piece * m + row] : 0.f;
+    }
+  };
+  if constexpr (SCALE_EARLY) load_scale_pieces();
+
   f32x4_t acc[WT];
 #pragma unroll
   for (int t = 0; t < WT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
@@ -302,18 +320,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     }
   }
 
-  // PRO_SCALED: SK_SCALE_PARTS threads per row each add up every SK_SCALE_PARTS-th piece of the
-  // row's sum of squares, in a fixed order.  Asked for only now: held through the loop above
-  // they would cost the registers of a resident block per CU (measured: 16 % slower).
-  float scale_piece[SCALED ? SK_SCALE_PIECES : 1];
-  if constexpr (SCALED) {
-    const int row = threadIdx.x % 16, part = threadIdx.x / 16;
-#pragma unroll
-    for (int i = 0; i < SK_SCALE_PIECES; ++i) {
-      const int piece = part + i * SK_SCALE_PARTS;
-      scale_piece[i] = (row < m && piece < fold.sumsq_pieces) ? fold.sumsq_in[(int64_t)piece * m + row] : 0.f;
-    }
-  }
+  if constexpr (SCALED && !SCALE_EARLY) load_scale_pieces();
   // acc[t][r] = C^T[feature n0 + 16*(t % NT) + 4*quad + r][token col]; add the 8 waves in order
 #pragma unroll
   for (int t = 0; t < WT; ++t) {
