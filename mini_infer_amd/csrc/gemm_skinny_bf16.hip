@@ -694,7 +694,7 @@ extern "C" int mi_gemm_skinny_swiglu_scaled_bf16(const void* a, int64_t lda, con
   if (fpb <= 16) {
     if (lines) SK_SCALED(1, 4, true); else SK_SCALED(1, 4, false);
   } else {
-    if (lines) SK_SCALED(2, 2, true); else SK_SCALED(2, 2, false);
+    if (lines) SK_SCALED(2, 4, true); else SK_SCALED(2, 2, false);
   }
 #undef SK_SCALED
   MI_CHECK_LAUNCH("gemm_skinny_swiglu_scaled_bf16");
@@ -723,7 +723,7 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
   if (fpb <= 16) {
     if (lines) SK_GATED(1, 4, true); else SK_GATED(1, 4, false);
   } else {
-    if (lines) SK_GATED(2, 2, true); else SK_GATED(2, 2, false);
+    if (lines) SK_GATED(2, 4, true); else SK_GATED(2, 2, false);
   }
 #undef SK_GATED
   MI_CHECK_LAUNCH("gemm_skinny_swiglu_bf16");
