@@ -89,7 +89,7 @@ struct FoldArgs {  // what the folded neighbours of a product need
   int norm_width;
 };
 
-template <int NT, int U, int EPI, int PRO = PRO_NONE, bool LINES = false>
+template <int NT, int U, int EPI, int PRO = PRO_NONE, bool LINES = false, int RT = 1>
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t ldw,
     bf16_t* __restrict__ c, int64_t ldc, int m, int n, int k, int features_per_block, const FoldArgs fold) {
@@ -99,6 +99,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   constexpr bool SCALED = PRO == PRO_SCALED;
   static_assert(!ROPE || NT == 1, "the rotary epilogue takes one tile of dims and its partner tile");
   static_assert(!LINES || U % 2 == 0, "whole lines are read for pairs of k-steps");
+  // RT = tiles of 16 ROWS (tokens): a weight operand once in registers is used for every row tile
+  static_assert(RT == 1 || (PRO == PRO_NONE && !ADDNORM), "more than 16 rows: plain activations, no folded norm");
   constexpr int WT = (GATED || ROPE) ? 2 * NT : NT;  // weight tiles per block
   __shared__ float red[SK_WAVES][WT][256];
 
@@ -154,7 +156,9 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   };
   // activations: lane reads token `col`; lanes past M re-read the last token (the same
   // cache lines as its own lane, so no extra traffic) and their columns are never stored
-  const bf16_t* ap = a + (int64_t)min(col, m - 1) * lda + quad * 8;
+  const bf16_t* ap[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) ap[rt] = a + (int64_t)min(rt * 16 + col, m - 1) * lda + quad * 8;
   __shared__ __attribute__((aligned(16))) bf16_t a_own[PRO == PRO_ATTN ? SK_WAVES : 1][PRO == PRO_ATTN ? SK_PRO_VALUES : 8];
   const int own_stride = per_wave * 32;  // elements from one row of this wave's columns to the next
   // PRO_ATTN: the weights of the first U k-steps are requested before the activations are
@@ -253,14 +257,16 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   };
   if constexpr (SCALE_EARLY) load_scale_pieces();
 
-  f32x4_t acc[WT];
+  f32x4_t acc[RT][WT];
 #pragma unroll
-  for (int t = 0; t < WT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int t = 0; t < WT; ++t) acc[rt][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
   int s = s_begin;
   for (; s + U <= s_end; s += U) {
     bf16x8_t w_reg[U][WT];
-    bf16x8_t a_reg[U];
+    bf16x8_t a_reg[RT][U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -279,8 +285,11 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
           else w_reg[u][t] = *reinterpret_cast<const bf16x8_t*>(wp[LINES ? 0 : t] + (int64_t)(s + u) * 32);
         }
       }
-      if constexpr (PRO == PRO_ATTN) a_reg[u] = *reinterpret_cast<const bf16x8_t*>(own + (s + u - s_begin) * 32);
-      else a_reg[u] = *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)(s + u) * 32);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if constexpr (PRO == PRO_ATTN) a_reg[rt][u] = *reinterpret_cast<const bf16x8_t*>(own + (s + u - s_begin) * 32);
+        else a_reg[rt][u] = *reinterpret_cast<const bf16x8_t*>(ap[rt] + (int64_t)(s + u) * 32);
+      }
     }
     if constexpr (LINES) {
 #pragma unroll
@@ -292,40 +301,59 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int t = 0; t < WT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_reg[u][t], a_reg[u], acc[t], 0, 0, 0);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_reg[u][t], a_reg[rt][u], acc[rt][t], 0, 0, 0);
   }
   if constexpr (LINES) {
     for (; s + 2 <= s_end; s += 2) {  // fewer than U k-steps left: pair by pair (their number is even)
-      const bf16x8_t a_even = PRO == PRO_ATTN ? *reinterpret_cast<const bf16x8_t*>(own + (s - s_begin) * 32)
-                                              : *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)s * 32);
-      const bf16x8_t a_odd = PRO == PRO_ATTN ? *reinterpret_cast<const bf16x8_t*>(own + (s + 1 - s_begin) * 32)
-                                             : *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)(s + 1) * 32);
+      bf16x8_t a_even[RT], a_odd[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        a_even[rt] = PRO == PRO_ATTN ? *reinterpret_cast<const bf16x8_t*>(own + (s - s_begin) * 32)
+                                     : *reinterpret_cast<const bf16x8_t*>(ap[rt] + (int64_t)s * 32);
+        a_odd[rt] = PRO == PRO_ATTN ? *reinterpret_cast<const bf16x8_t*>(own + (s + 1 - s_begin) * 32)
+                                    : *reinterpret_cast<const bf16x8_t*>(ap[rt] + (int64_t)(s + 1) * 32);
+      }
 #pragma unroll
       for (int t = 0; t < WT; ++t) {
         bf16x8_t w_even, w_odd;
         load_lines(t, s, w_even, w_odd);
         lines_to_operands(w_even, w_odd);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_even, a_even, acc[t], 0, 0, 0);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_odd, a_odd, acc[t], 0, 0, 0);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_even, a_even[rt], acc[rt][t], 0, 0, 0);
+          acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_odd, a_odd[rt], acc[rt][t], 0, 0, 0);
+        }
       }
     }
   }
   for (; !LINES && s < s_end; ++s) {  // fewer than U k-steps left
-    const bf16x8_t a_tail = PRO == PRO_ATTN ? *reinterpret_cast<const bf16x8_t*>(own + (s - s_begin) * 32)
-                                            : *reinterpret_cast<const bf16x8_t*>(ap + (int64_t)s * 32);
+    bf16x8_t a_tail[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+      a_tail[rt] = PRO == PRO_ATTN ? *reinterpret_cast<const bf16x8_t*>(own + (s - s_begin) * 32)
+                                   : *reinterpret_cast<const bf16x8_t*>(ap[rt] + (int64_t)s * 32);
 #pragma unroll
     for (int t = 0; t < WT; ++t) {
       const bf16x8_t w_tail = *reinterpret_cast<const bf16x8_t*>(wp[LINES ? 0 : t] + (int64_t)s * 32);
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_tail, a_tail, acc[t], 0, 0, 0);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+        acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_tail, a_tail[rt], acc[rt][t], 0, 0, 0);
     }
   }
 
   if constexpr (SCALED && !SCALE_EARLY) load_scale_pieces();
-  // acc[t][r] = C^T[feature n0 + 16*(t % NT) + 4*quad + r][token col]; add the 8 waves in order
+  __shared__ float squares[ADDNORM ? NT * 4 : 1][16];  // EPI_ADDNORM: per (4 features, row) of the block
+  // acc[rt][t][r] = C^T[feature n0 + 16*(t % NT) + 4*quad + r][token 16*rt + col]; add the 8 waves
+  // in order, one row tile after the other through the same LDS
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+  if (rt > 0) __syncthreads();
 #pragma unroll
   for (int t = 0; t < WT; ++t) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][t][(quad * 4 + r) * 16 + col] = acc[t][r];
+    for (int r = 0; r < 4; ++r) red[wave][t][(quad * 4 + r) * 16 + col] = acc[rt][t][r];
   }
   if constexpr (SCALED) {
     float scale_mine = 0.f;
@@ -333,26 +361,26 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     for (int i = 0; i < SK_SCALE_PIECES; ++i) scale_mine += scale_piece[i];
     scale_part[threadIdx.x / 16][threadIdx.x % 16] = scale_mine;
   }
-  __shared__ float squares[ADDNORM ? NT * 4 : 1][16];  // EPI_ADDNORM: per (4 features, row) of the block
   __syncthreads();
   // 256*NT outputs, each a sum of 8 (two such when gated): a thread takes 4 consecutive
   // features of one token
   for (int item = threadIdx.x; item < NT * 64; item += 64 * SK_WAVES) {
     const int nt = item / 64;
-    const int token = (item % 64) % 16;
+    const int token_in_tile = (item % 64) % 16;
+    const int token = rt * 16 + token_in_tile;
     const int fq = (item % 64) / 16;
     if (token >= m) continue;
     float sum[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int wv = 0; wv < SK_WAVES; ++wv)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) sum[r] += red[wv][nt][(fq * 4 + r) * 16 + token];
+      for (int r = 0; r < 4; ++r) sum[r] += red[wv][nt][(fq * 4 + r) * 16 + token_in_tile];
     float up[4] = {0.f, 0.f, 0.f, 0.f};  // the twin tile's sums: the up half (gated), the partner dims (rotary)
     if (GATED || ROPE) {
 #pragma unroll
       for (int wv = 0; wv < SK_WAVES; ++wv)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) up[r] += red[wv][NT + nt][(fq * 4 + r) * 16 + token];
+        for (int r = 0; r < 4; ++r) up[r] += red[wv][NT + nt][(fq * 4 + r) * 16 + token_in_tile];
     }
     if constexpr (SCALED) {
       float total = 0.f;
@@ -457,6 +485,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
         if (feature + r < n_end) dst[r] = (bf16_t)sum[r];
     }
   }
+  }  // row tiles
   if constexpr (ADDNORM) {
     __syncthreads();
     if ((int)threadIdx.x < m) {
@@ -468,7 +497,14 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   }
 }
 
+// Rows.  The gated and the rotary product take two row tiles (17-32 rows: measured against the
+// vendor product followed by silu_mul / rope_kv_write, microseconds at 24 / 32 rows: gate|up
+// 2x14336x4096 42.9 / 46.2 against 54.6 / 54.6, q|k|v 6144x4096 17.0 / 17.2 against 20.2 / 19.5,
+// gate|up 2x8192x3072 22.4 / 23.3 against 23.8 / 23.9, q|k|v 5120x3072 13.9 / 14.6 against
+// 17.8 / 16.4; with four row tiles, 48 / 64 rows, they are level or slower: every block reads
+// all the rows' activations).  Everything else takes one.
 #define SK_MAX_ROWS 16
+#define SK_WIDE_MAX_ROWS 32
 
 // Compute units of the current device (asked once per device).
 static int compute_units() {
@@ -483,8 +519,17 @@ static int compute_units() {
   return cached[device];
 }
 
+static bool skinny_takes(int m, int n, int k, int64_t lda, int64_t ldw, int max_rows) {
+  return m >= 1 && m <= max_rows && n >= 1 && k >= 32 && k % 32 == 0 && lda % 8 == 0 && ldw % 8 == 0;
+}
+
 extern "C" int mi_gemm_skinny_bf16_supported(int m, int n, int k, int64_t lda, int64_t ldw) {
-  return (m >= 1 && m <= SK_MAX_ROWS && n >= 1 && k >= 32 && k % 32 == 0 && lda % 8 == 0 && ldw % 8 == 0) ? 1 : 0;
+  return skinny_takes(m, n, k, lda, ldw, SK_MAX_ROWS) ? 1 : 0;
+}
+
+// the gated and the rotary product (mi_gemm_skinny_swiglu_bf16, mi_gemm_skinny_rope_bf16)
+extern "C" int mi_gemm_skinny_wide_bf16_supported(int m, int n, int k, int64_t lda, int64_t ldw) {
+  return skinny_takes(m, n, k, lda, ldw, SK_WIDE_MAX_ROWS) ? 1 : 0;
 }
 
 // Features per block: as even a share of the output as a multiple of 4 allows, in
@@ -704,8 +749,8 @@ extern "C" int mi_gemm_skinny_swiglu_scaled_bf16(const void* a, int64_t lda, con
 // out[m, n] = silu(a . gate^T) * (a . up^T) with w = [gate; up] stacked, [2n, k].
 extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* out,
                                           int64_t ldo, int m, int n, int k, hipStream_t stream) {
-  MI_REQUIRE(mi_gemm_skinny_bf16_supported(m, n, k, lda, ldw),
-             "gemm_skinny_swiglu_bf16: takes 1 <= m <= 16, k a multiple of 32, rows aligned to 16 bytes; "
+  MI_REQUIRE(mi_gemm_skinny_wide_bf16_supported(m, n, k, lda, ldw),
+             "gemm_skinny_swiglu_bf16: takes 1 <= m <= 32, k a multiple of 32, rows aligned to 16 bytes; "
              "got m=%d n=%d k=%d lda=%lld ldw=%lld", m, n, k, (long long)lda, (long long)ldw);
   MI_REQUIRE(lda >= k && ldw >= k && ldo >= n, "gemm_skinny_swiglu_bf16: a row stride is shorter than its row");
   const bf16_t* ap = (const bf16_t*)a;
@@ -718,12 +763,20 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
   const bool lines = whole_lines(w, ldw, 2 * (int64_t)n, k);
-#define SK_GATED(NT_, U_, LINES_) \
-  gemm_skinny_bf16_kernel<NT_, U_, EPI_GATED, PRO_NONE, LINES_><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, nothing_folded)
-  if (fpb <= 16) {
-    if (lines) SK_GATED(1, 4, true); else SK_GATED(1, 4, false);
-  } else {
-    if (lines) SK_GATED(2, 4, true); else SK_GATED(2, 2, false);
+#define SK_GATED(NT_, U_, LINES_, RT_) \
+  gemm_skinny_bf16_kernel<NT_, U_, EPI_GATED, PRO_NONE, LINES_, RT_><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, nothing_folded)
+  if (m <= 16) {
+    if (fpb <= 16) {
+      if (lines) SK_GATED(1, 4, true, 1); else SK_GATED(1, 4, false, 1);
+    } else {
+      if (lines) SK_GATED(2, 4, true, 1); else SK_GATED(2, 2, false, 1);
+    }
+  } else {  // (two row tiles: fewer k-steps in flight, the registers hold both tiles' sums)
+    if (fpb <= 16) {
+      if (lines) SK_GATED(1, 4, true, 2); else SK_GATED(1, 4, false, 2);
+    } else {
+      if (lines) SK_GATED(2, 2, true, 2); else SK_GATED(2, 2, false, 2);
+    }
   }
 #undef SK_GATED
   MI_CHECK_LAUNCH("gemm_skinny_swiglu_bf16");
@@ -745,8 +798,8 @@ static int rope_product(const char* name, const void* a, int64_t lda, const floa
              "%s: takes head_dim a multiple of 32; got q_heads=%d kv_heads=%d head_dim=%d", name, q_heads, kv_heads,
              head_dim);
   const int n = (q_heads + 2 * kv_heads) * head_dim;
-  MI_REQUIRE(mi_gemm_skinny_bf16_supported(m, n, k, lda, ldw),
-             "%s: takes 1 <= m <= 16, k a multiple of 32, rows aligned to 16 bytes; "
+  MI_REQUIRE(mi_gemm_skinny_wide_bf16_supported(m, n, k, lda, ldw),
+             "%s: takes 1 <= m <= 32, k a multiple of 32, rows aligned to 16 bytes; "
              "got m=%d n=%d k=%d lda=%lld ldw=%lld", name, m, n, k, (long long)lda, (long long)ldw);
   MI_REQUIRE(lda >= k && ldw >= k && ldq >= (int64_t)q_heads * head_dim && ldq % 4 == 0,
              "%s: a row stride is shorter than its row or not 8-byte aligned", name);
@@ -780,13 +833,16 @@ static int rope_product(const char* name, const void* a, int64_t lda, const floa
   if (pairs_per_block > 16) pairs_per_block = 16;
   const int blocks = ceil_div(total_pairs, pairs_per_block);
   const bool lines = whole_lines(w, ldw, n, k);
-#define SK_ROPE(PRO_, LINES_)                                                                  \
-  gemm_skinny_bf16_kernel<1, 8, EPI_ROPE, PRO_, LINES_><<<blocks, 64 * SK_WAVES, 0, stream>>>( \
+#define SK_ROPE(U_, PRO_, LINES_, RT_)                                                                \
+  gemm_skinny_bf16_kernel<1, U_, EPI_ROPE, PRO_, LINES_, RT_><<<blocks, 64 * SK_WAVES, 0, stream>>>( \
       (const bf16_t*)a, lda, (const bf16_t*)w, ldw, (bf16_t*)q_out, ldq, m, n, k, pairs_per_block, fold)
   if (sumsq) {
-    if (lines) SK_ROPE(PRO_SCALED, true); else SK_ROPE(PRO_SCALED, false);
+    MI_REQUIRE(m <= SK_MAX_ROWS, "%s: rows with their norm factor apart come 16 at most, got %d", name, m);
+    if (lines) SK_ROPE(8, PRO_SCALED, true, 1); else SK_ROPE(8, PRO_SCALED, false, 1);
+  } else if (m <= 16) {
+    if (lines) SK_ROPE(8, PRO_NONE, true, 1); else SK_ROPE(8, PRO_NONE, false, 1);
   } else {
-    if (lines) SK_ROPE(PRO_NONE, true); else SK_ROPE(PRO_NONE, false);
+    if (lines) SK_ROPE(4, PRO_NONE, true, 2); else SK_ROPE(4, PRO_NONE, false, 2);
   }
 #undef SK_ROPE
   MI_CHECK_LAUNCH(name);

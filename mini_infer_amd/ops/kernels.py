@@ -367,8 +367,14 @@ def gemm_skinny_bf16(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return c
 
 
-def skinny_gemm_takes(m: int, k: int, lda: int, ldw: int) -> bool:
-    return 1 <= m <= SKINNY_MAX_ROWS and k >= 32 and k % 32 == 0 and lda % 8 == 0 and ldw % 8 == 0
+def skinny_gemm_takes(m: int, k: int, lda: int, ldw: int, max_rows: int = SKINNY_MAX_ROWS) -> bool:
+    return 1 <= m <= max_rows and k >= 32 and k % 32 == 0 and lda % 8 == 0 and ldw % 8 == 0
+
+
+# The gated product and the q|k|v product with rotation and cache write take two tiles of 16
+# rows: up to 32 rows they measured faster than the vendor product followed by `silu_mul` /
+# `rope_kv_write` (8B sizes 12-21 %, 3B sizes 3-22 %), with 48 and 64 rows level or slower.
+SKINNY_WIDE_MAX_ROWS = 32
 
 
 PARTIAL_SUMS_MAX_ROWS = 128
@@ -479,19 +485,20 @@ def _scaled_rows_fit(x: "ScaledRows") -> bool:
 def qkv_rope_write_takes(
     x: "torch.Tensor | ScaledRows", weight: torch.Tensor, head_dim: int, rotary_dim: int, interleaved: bool
 ) -> bool:
-    """Whether `qkv_rope_write` runs these operands: at most 16 bfloat16 rows, rotation of
-    whole heads in half pairing, head size a multiple of 32."""
+    """Whether `qkv_rope_write` runs these operands: at most 32 bfloat16 rows (16 as
+    `ScaledRows`), rotation of whole heads in half pairing, head size a multiple of 32."""
+    max_rows = SKINNY_WIDE_MAX_ROWS
     if isinstance(x, ScaledRows):
         if not _scaled_rows_fit(x):
             return False
-        x = x.values
+        x, max_rows = x.values, SKINNY_MAX_ROWS
     return (
         x.dtype == torch.bfloat16
         and weight.dtype == torch.bfloat16
         and x.dim() == 2
         and x.stride(1) == 1
         and weight.stride(1) == 1
-        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), weight.stride(0))
+        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), weight.stride(0), max_rows)
         and not interleaved
         and rotary_dim == head_dim
         and head_dim % 32 == 0
@@ -514,7 +521,7 @@ def qkv_rope_write(
 ) -> torch.Tensor:
     """The stacked q|k|v projection, the rotary encoding and the cache write as ONE kernel.
 
-    x [M <= 16, K] bfloat16, weight [(q_heads + 2*kv_heads)*head_dim, K]; returns the rotated
+    x [M <= 32, K] bfloat16, weight [(q_heads + 2*kv_heads)*head_dim, K]; returns the rotated
     queries [M, q_heads*head_dim]; rotated keys and values go to their slots.  `kv_heads=0`
     with the query rows of the weight alone projects and rotates queries only.  The result
     is that of `linear` followed by `rope_kv_write` (both round the product to bfloat16
@@ -531,7 +538,7 @@ def qkv_rope_write(
     _need_int32("slot_mapping", slot_mapping)
     if not qkv_rope_write_takes(scaled if scaled is not None else x, weight, head_dim, head_dim, False):
         raise KernelShapeError(
-            f"qkv_rope_write takes at most 16 bfloat16 rows and head sizes in steps of 32; got "
+            f"qkv_rope_write takes at most 32 bfloat16 rows and head sizes in steps of 32; got "
             f"x {tuple(x.shape)} {x.dtype}, head_dim={head_dim}"
         )
     m, k = x.shape
@@ -573,7 +580,7 @@ def qkv_rope_write(
 def linear_swiglu(x: "torch.Tensor | ScaledRows", gate_up_weight: torch.Tensor) -> torch.Tensor:
     """`silu(x @ gate.T) * (x @ up.T)` with `gate_up_weight` = [gate; up] stacked, [2I, K].
 
-    bfloat16 with at most 16 rows runs as ONE hand-written kernel (the product with the
+    bfloat16 with at most 32 rows runs as ONE hand-written kernel (the product with the
     activation in its last step); otherwise the product and `silu_mul` run in turn.
     Both ways round the two products to the element type before the activation, so a
     token's result does not depend on which one ran.  `x` may be `ScaledRows`: the rows'
@@ -604,7 +611,7 @@ def linear_swiglu(x: "torch.Tensor | ScaledRows", gate_up_weight: torch.Tensor) 
         and x.shape[1] == width
         and x.stride(1) == 1
         and gate_up_weight.stride(1) == 1
-        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), gate_up_weight.stride(0))
+        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), gate_up_weight.stride(0), SKINNY_WIDE_MAX_ROWS)
     ):
         _need_cuda(x, gate_up_weight)
         m, n = x.shape[0], rows // 2

@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -48,6 +48,7 @@ _SIGNATURES: dict[str, list] = {
         c_int, c_int, c_int, c_int, _P,
     ],
     "mi_gemm_skinny_bf16_supported": [c_int, c_int, c_int, c_int64, c_int64],
+    "mi_gemm_skinny_wide_bf16_supported": [c_int, c_int, c_int, c_int64, c_int64],
     "mi_attn_generic": [
         c_int, _P, c_int64, _P, _P, _P, c_int, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int,
         c_int, c_int, c_int, c_float, c_int, c_int, _P, _P,

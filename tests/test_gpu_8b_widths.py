@@ -186,6 +186,31 @@ def test_eight_requests_past_two_thousand_tokens_decoded_in_recorded_steps(wide,
     runner.cache.check()
 
 
+def test_twenty_four_single_tokens_in_one_step(wide):
+    """24 requests bring one token each to the same step: the batch-of-32 graph, whose gate|up
+    and q|k|v products are the weight-streaming kernels with two tiles of 16 rows (activation,
+    rotation and cache write in their last steps).  Twice, so that the second step is a replay."""
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+
+    folder, oracle = wide
+    lengths = [17 + (11 * i) % 200 for i in range(24)]
+    requests = {f"w{i}": tiny.random_tokens(WIDE, n + 2, seed=300 + i) for i, n in enumerate(lengths)}
+    runner = ModelRunner.from_pretrained(folder, dtype="bfloat16", num_blocks=24 * 14, block_size=16, max_concurrent=24)
+    ids = list(requests)
+    for first in range(0, 24, 8):
+        runner.step([StepEntry(rid, requests[rid][: lengths[ids.index(rid)]], []) for rid in ids[first : first + 8]])
+    got = []
+    for k in range(2):
+        got.append(runner.step([StepEntry(rid, [requests[rid][n + k]], [0]) for rid, n in zip(ids, lengths)]).cpu().numpy())
+    assert runner.decode_graphs.replays == 2 and [rows for rows, _ in runner.decode_graphs.graphs] == [32]
+    for row, (rid, n) in enumerate(zip(ids, lengths)):
+        expected = oracle(requests[rid], rows=[n, n + 1])
+        ru.assert_close(np.stack([got[0][row], got[1][row]]), expected, "bfloat16", f"8B widths, 24 rows, {rid} ({n} tokens)")
+    for rid in ids:
+        runner.free_request(rid)
+    runner.cache.check()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_forty_single_tokens_in_one_step(wide, dtype):
     """40 requests with contexts of 17 to 290 tokens each bring one token to the same step (in

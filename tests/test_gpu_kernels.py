@@ -195,7 +195,7 @@ def test_linear_leaves_partial_sums_only_where_asked_and_where_it_pays():
 @pytest.mark.parametrize(
     "m,inter,k",
     [(1, 14336, 4096), (8, 14336, 4096), (16, 160, 64), (7, 301, 96), (13, 4100, 160), (3, 5, 32), (9, 8192, 3072),
-     (5, 520, 1536), (2, 24, 512)],
+     (5, 520, 1536), (2, 24, 512), (17, 14336, 4096), (32, 8192, 3072), (24, 160, 64), (31, 301, 96), (20, 520, 1536)],
 )
 def test_linear_swiglu_is_the_product_followed_by_the_activation(m, inter, k):
     from mini_infer_amd import ops
@@ -204,8 +204,10 @@ def test_linear_swiglu_is_the_product_followed_by_the_activation(m, inter, k):
     w = _rand(2 * inter, k, dtype=torch.bfloat16, seed=13, scale=0.08)
     fused = ops.linear_swiglu(a, w)
     assert fused.shape == (m, inter)
-    # the two-kernel path: the product (rounded to bfloat16), then the activation
-    assert torch.equal(fused, ops.silu_mul(ops.gemm_skinny_bf16(a, w)))
+    # the two-kernel path: the product (rounded to bfloat16), then the activation (the plain
+    # weight-streaming product takes 16 rows; a row's result does not depend on the others)
+    for first in range(0, m, 16):
+        assert torch.equal(fused[first : first + 16], ops.silu_mul(ops.gemm_skinny_bf16(a[first : first + 16], w)))
     assert torch.equal(ops.linear_swiglu(a, _off_the_cache_lines(w)), fused)
     gate_up = (a.double() @ w.double().T).bfloat16().double()
     gate, up = gate_up[:, :inter], gate_up[:, inter:]
@@ -225,7 +227,7 @@ def test_linear_swiglu_is_the_product_followed_by_the_activation(m, inter, k):
 @pytest.mark.parametrize(
     "m,hidden,q_heads,kv_heads,head_dim,page_size",
     [(8, 4096, 32, 8, 128, 16), (1, 4096, 32, 8, 128, 16), (16, 96, 3, 1, 32, 16), (5, 160, 6, 2, 64, 32), (9, 64, 4, 4, 96, 48),
-     (3, 1536, 6, 2, 64, 16)],
+     (3, 1536, 6, 2, 64, 16), (17, 4096, 32, 8, 128, 16), (32, 1536, 6, 2, 64, 16), (25, 96, 3, 1, 32, 16)],
 )
 def test_qkv_rope_write_is_the_product_followed_by_rotation_and_cache_write(
     v_transposed, m, hidden, q_heads, kv_heads, head_dim, page_size
@@ -236,11 +238,14 @@ def test_qkv_rope_write_is_the_product_followed_by_rotation_and_cache_write(
     width = (q_heads + 2 * kv_heads) * head_dim
     x = _rand(m, hidden, dtype=torch.bfloat16, seed=31)
     w = _rand(width, hidden, dtype=torch.bfloat16, seed=32, scale=0.1)
-    positions = torch.tensor([0, 1, 700, 5, 131071, 17, 18, 19, 3000, 2, 4, 6, 8, 10, 12, 14][:m], dtype=torch.int32, device=DEV)
+    positions = torch.tensor(([0, 1, 700, 5, 131071, 17, 18, 19, 3000, 2, 4, 6, 8, 10, 12, 14] + list(range(50, 66)))[:m],
+                             dtype=torch.int32, device=DEV)
     inv_freq = torch.from_numpy(pl.inv_freq_default(head_dim, 500000.0)).to(DEV)
     cos, sin = ops.rope_table(positions, inv_freq)
-    slots = torch.tensor([40, 3, 17, 16, 0, 43, -1, 9, 22, 5, 6, 7, 30, 31, 32, 33][:m], dtype=torch.int32, device=DEV)
+    slots = torch.tensor(([40, 3, 17, 16, 0, 43, -1, 9, 22, 5, 6, 7, 30, 31, 32, 33] + list(range(60, 76)))[:m],
+                         dtype=torch.int32, device=DEV)
     slots = torch.where(slots >= 0, slots % (num_pages * page_size), slots)
+    assert len(set(slots[slots >= 0].tolist())) == int((slots >= 0).sum())  # (no two rows write one slot)
 
     def pages():
         k = torch.full((num_pages, kv_heads, page_size, head_dim), 7.0, dtype=torch.bfloat16, device=DEV)
@@ -248,7 +253,7 @@ def test_qkv_rope_write_is_the_product_followed_by_rotation_and_cache_write(
         return k, torch.full(v_shape, 7.0, dtype=torch.bfloat16, device=DEV)
 
     k_two, v_two = pages()
-    qkv = ops.gemm_skinny_bf16(x, w)
+    qkv = torch.cat([ops.gemm_skinny_bf16(x[first : first + 16], w) for first in range(0, m, 16)])
     ops.rope_kv_write(qkv, cos, sin, slots, k_two, v_two, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim,
                       rotary_dim=head_dim, interleaved=False, v_transposed=v_transposed)
     k_one, v_one = pages()
