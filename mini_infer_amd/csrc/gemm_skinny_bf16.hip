@@ -1,15 +1,19 @@
 // Weight-streaming matrix product for few rows (decode): C[M,N] = A[M,K] * W[N,K]^T,
-// bfloat16 in and out, float32 accumulate on the matrix cores, M <= 16.
+// bfloat16 in and out, float32 accumulate on the matrix cores, M <= 16 (<= 32 for the
+// gated and the rotary product).
 //
-// At these sizes the product is bound by reading W once from HBM.  A block owns 16
-// output features and all of K: its 8 waves each stream one eighth of every one of
-// the 16 weight rows (16 contiguous bytes per lane and k-step, MFMA 16x16x32 with
-// the weights as the A operand and the activations, transposed, as the B operand),
-// then add their partial tiles through LDS in a fixed order, so the result does not
-// depend on timing.  Activations are small and come from the cache hierarchy.
+// At these sizes the product is bound by reading W once from HBM.  A block owns 8 to 64
+// output features and all of K: its 8 waves each stream one eighth of every one of its
+// weight rows (MFMA 16x16x32 with the weights as the A operand and the activations,
+// transposed, as the B operand), then add their partial tiles through LDS in a fixed order,
+// so the result does not depend on timing.  Activations are small and come from the cache
+// hierarchy.  How the weight rows are read decides the kernel's speed: in whole cache lines
+// with non-temporal loads where the matrix lies so that they can be (LINES; common.h says
+// how and what was measured), else 16 contiguous bytes per lane and k-step.
 //
 // What follows a product in a decoder layer is folded into its last step where that saves a
-// launch: the SiLU-gated product, the rotary encoding with the cache write (EPI_*).
+// launch: the SiLU-gated product, the rotary encoding with the cache write, the residual
+// add with the beginning of the norm (EPI_*).
 //
 // This stands where the reference's engine calls the vendor BLAS
 // (distributed/linear.py:167); that library's kernels reach about half of the HBM
@@ -23,7 +27,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define SK_WAVES 8
 
 // LINES: the weights are read in whole cache lines (lines_to_operands in common.h), where
-// the matrix lies so that they can be.
+// the matrix lies so that they can be.  RT = tiles of 16 rows (tokens) a wave keeps sums for.
 // NT = 16-feature tiles of the OUTPUT per block (the activations a wave loads are used
 // for every weight tile of the block), U = k-steps whose loads are issued together
 // before their products run.  Register use is kept low on purpose: many resident waves,
