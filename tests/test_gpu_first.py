@@ -10,7 +10,7 @@ import tiny
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_whole_prompt_logits(tmp_path, name, dtype):
     from mini_infer_amd.engine import ModelRunner, StepEntry

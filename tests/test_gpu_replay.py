@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 LENGTHS = [5, 33, 70, 97, 41, 64]
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "D"])
 def case(request, tmp_path_factory):
     name = request.param
     cfg, block = tiny.CONFIGS[name]
@@ -50,10 +50,30 @@ def test_whole(case, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_prefill_then_decode(case, dtype):
+def test_prefill_then_decode(case, dtype, monkeypatch):
+    import mini_infer_amd.ops as ops
+
     name, cfg, block, folder, requests, expected = case
+    folded = {"products": 0, "scaled_rows": 0}
+    add_norm, rope_write = ops.linear_add_norm, ops.qkv_rope_write
+
+    def count_add_norm(*args):
+        folded["products"] += 1
+        return add_norm(*args)
+
+    def count_rope_write(x, *args, **kwargs):
+        folded["scaled_rows"] += isinstance(x, ops.ScaledRows)
+        return rope_write(x, *args, **kwargs)
+
+    monkeypatch.setattr(ops, "linear_add_norm", count_add_norm)
+    monkeypatch.setattr(ops, "qkv_rope_write", count_rope_write)
     schedule = ru.schedule_prefill_then_decode(requests)
     _check(_runner(folder, dtype, block, 64), requests, expected, schedule, dtype, f"{name} prefill+decode")
+    if name == "D" and dtype == "bfloat16":
+        # the configuration whose sizes the folded kernels take: both norms of a layer went that way
+        assert folded["products"] >= 2 * cfg["num_hidden_layers"] - 1 and folded["scaled_rows"] >= 1
+    if dtype == "float32":
+        assert folded == {"products": 0, "scaled_rows": 0}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

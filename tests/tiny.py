@@ -1,9 +1,12 @@
 """Tiny configurations and model folders for the tests.
 
-The three configurations differ in every size and option: layers, width, heads
+The configurations differ in every size and option: layers, width, heads
 and groups, head size, feed-forward width, vocabulary, rope base and scaling,
 the norms' eps, tied or untied head.  A and B are the two named in the project's
-baseline; C adds sizes that no vector width divides.  Weights are made here with
+baseline; C adds sizes that no vector width divides; D has the smallest sizes at
+which every fast path of the bfloat16 engine runs (weight rows of whole cache
+lines read as such, both norms of a layer folded into the neighbouring products,
+head size 64 on the matrix-core attention with streamed pages).  Weights are made here with
 NumPy (not with the engine's random mode), rounded to bfloat16 so the float32
 and the bfloat16 engine and the plain implementation all read the same numbers.
 """
@@ -80,7 +83,31 @@ TINY_C = {
 }
 TINY_C_BLOCK = 8
 
-CONFIGS = {"A": (TINY_A, TINY_A_BLOCK), "B": (TINY_B, TINY_B_BLOCK), "C": (TINY_C, TINY_C_BLOCK)}
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 2,
+    "hidden_size": 512,
+    "num_attention_heads": 8,
+    "num_key_value_heads": 2,
+    "head_dim": 64,
+    "intermediate_size": 1024,
+    "vocab_size": 333,
+    "rope_theta": 100000.0,
+    "rope_scaling": {
+        "rope_type": "llama3",
+        "factor": 16.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 8.0,
+        "original_max_position_embeddings": 48,
+    },
+    "rms_norm_eps": 2e-5,
+    "tie_word_embeddings": True,
+    "max_position_embeddings": 2048,
+}
+TINY_D_BLOCK = 16
+
+CONFIGS = {"A": (TINY_A, TINY_A_BLOCK), "B": (TINY_B, TINY_B_BLOCK), "C": (TINY_C, TINY_C_BLOCK),
+           "D": (TINY_D, TINY_D_BLOCK)}
 
 
 def bf16_round(values: np.ndarray) -> np.ndarray:
