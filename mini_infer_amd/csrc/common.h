@@ -95,8 +95,8 @@ __device__ __forceinline__ void lines_to_operands(bf16x8_t& lower_rows, bf16x8_t
 __device__ __forceinline__ int line_row_of_lane(int lane) { return lane / 8; }
 __device__ __forceinline__ uint32_t line_chunk_of_lane(int lane) { return (uint32_t)(lane % 8) * 16u; }
 
-// The two loads of a pair of k-steps: base (uniform, kept in scalar registers) + the lane's offsets.
-template <bool STREAMED = true>
+// The two loads of a pair of k-steps, non-temporal: base (uniform, kept in scalar registers) + the
+// lane's offsets.
 __device__ __forceinline__ void load_line_pair(const void* matrix, int64_t first_kstep, uint32_t lower_at,
                                                uint32_t upper_at, bf16x8_t& lower_rows, bf16x8_t& upper_rows) {
   using global_bytes = const __attribute__((address_space(1))) char;
@@ -107,13 +107,8 @@ __device__ __forceinline__ void load_line_pair(const void* matrix, int64_t first
   // (opaque to the compiler, or it widens the offsets to 64 bits once and for all and adds
   // whole addresses in vector registers for every load)
   asm("" : "+v"(lower_at), "+v"(upper_at));
-  if constexpr (STREAMED) {
-    lower_rows = __builtin_nontemporal_load((global_chunk*)(base + lower_at));
-    upper_rows = __builtin_nontemporal_load((global_chunk*)(base + upper_at));
-  } else {
-    lower_rows = *(global_chunk*)(base + lower_at);
-    upper_rows = *(global_chunk*)(base + upper_at);
-  }
+  lower_rows = __builtin_nontemporal_load((global_chunk*)(base + lower_at));
+  upper_rows = __builtin_nontemporal_load((global_chunk*)(base + upper_at));
 }
 
 __device__ __forceinline__ float wave_max(float v) {
