@@ -643,7 +643,7 @@ def test_output_projection_from_uncombined_key_ranges(q_heads, kv_heads, head_di
 @pytest.mark.parametrize(
     "m,n,k,inter",
     [(8, 4096, 4096, 14336), (1, 4096, 4096, 14336), (16, 96, 64, 160), (7, 160, 96, 301), (13, 4128, 160, 40), (3, 32, 32, 5),
-     (6, 1536, 1536, 520)],
+     (6, 1536, 1536, 520), (5, 1000, 512, 72), (16, 8200, 1024, 24)],
 )
 def test_product_add_and_norm_folded_into_two_products(m, n, k, inter):
     """`linear_add_norm` (product, add into the residual, norm but for the rows' factors) followed
