@@ -761,10 +761,22 @@ static int heads_per_block_for(int group, int rows) { return group < rows ? grou
 #define MI_PREFILL_WAVES 4  // waves per block in the prefill shape
 #define MI_PREFILL_RG 2  // row groups (of 16 rows) per wave in the prefill shape
 #define MI_PREFILL_ROWS (16 * MI_PREFILL_WAVES * MI_PREFILL_RG)
+// The shape of a launch: prefill (128 rows a block, two blocks a CU), decode (16 rows, waves
+// split the keys), or wide prefill (8 waves, 256 rows a block, one block a CU: every key and
+// value tile is fetched half as often; measured on one prompt of 8,192 / 32,768 / 131,072
+// tokens 666-679 us / 8.17 ms / 130 ms against 715 us / 8.75 ms / 140 ms, but 73 against 61 us
+// for 2,048 tokens, whose 256 blocks of unequal length fill the GPU badly; the caller chooses).
+#define MI_SHAPE_PREFILL 0
+#define MI_SHAPE_DECODE 1
+#define MI_SHAPE_PREFILL_WIDE 2
+#define MI_WIDE_WAVES 8
+static int rows_of_shape(int shape) {
+  return shape == MI_SHAPE_DECODE ? 16 : shape == MI_SHAPE_PREFILL_WIDE ? 16 * MI_WIDE_WAVES * MI_PREFILL_RG : MI_PREFILL_ROWS;
+}
 
-extern "C" int mi_attn_mfma_tokens_per_tile(int q_heads, int kv_heads, int decode_only) {
+extern "C" int mi_attn_mfma_tokens_per_tile(int q_heads, int kv_heads, int shape) {
   if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return 0;
-  const int rows = decode_only ? 16 : MI_PREFILL_ROWS;
+  const int rows = rows_of_shape(shape);
   const int hb = heads_per_block_for(q_heads / kv_heads, rows);
   const int t = rows / hb;
   return t < 1 ? 1 : t;
@@ -794,7 +806,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
                             int num_tokens, int num_tiles, void* out, int64_t out_row_stride,
                             float* part_acc, float* part_ml, int q_heads, int kv_heads,
                             int head_dim, int page_size, int num_pages, float scale, int window,
-                            int num_splits, int decode_only, int one_tile_per_request,
+                            int num_splits, int shape, int one_tile_per_request,
                             int first_token, int combine, hipStream_t stream) {
   MI_REQUIRE(first_token >= 0, "attn_mfma: first_token=%d is negative", first_token);
   MI_REQUIRE(num_tokens >= 0 && num_requests >= 0 && num_tiles >= 0,
@@ -823,10 +835,13 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
              "attn_mfma: one tile per request needs num_tiles == num_requests");
   if (num_tokens == 0 || num_tiles == 0) return MI_OK;
 
+  MI_REQUIRE(shape == MI_SHAPE_PREFILL || shape == MI_SHAPE_DECODE || (shape == MI_SHAPE_PREFILL_WIDE && head_dim <= 128),
+             "attn_mfma: shape %d (0 prefill, 1 decode, 2 wide prefill for head sizes up to 128)", shape);
+  const bool decode_only = shape == MI_SHAPE_DECODE;
   const int group = q_heads / kv_heads;
-  const int rows = decode_only ? 16 : MI_PREFILL_ROWS;
+  const int rows = rows_of_shape(shape);
   const int hb = heads_per_block_for(group, rows);
-  const int tq = mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, decode_only);
+  const int tq = mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, shape);
   const int head_blocks = ceil_div(group, hb);
   MI_REQUIRE((int64_t)num_tiles * kv_heads * head_blocks < (1ll << 31), "attn_mfma: too many tiles x heads");
   MI_REQUIRE(num_splits <= 65535, "attn_mfma: too many splits");
@@ -834,7 +849,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
   const float scale_log2 = scale * LOG2E;
   // prefill blocks run two to a CU: see the tile order in the kernel (8 XCDs share the CUs evenly)
   int pair_group = 0;
-  if (!decode_only && MI_PREFILL_OCC(head_dim) == 2) {
+  if (shape == MI_SHAPE_PREFILL && MI_PREFILL_OCC(head_dim) == 2) {
     int device = 0, cus = 0;
     if (hipGetDevice(&device) == hipSuccess &&
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess)
@@ -852,8 +867,9 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
       out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, page_magic, scale_log2,    \
       window,                                                                                     \
       num_splits, hb, tq, one_tile_per_request, pair_group, first_token)
-#define MI_LAUNCH_P(DD, PP)                                              \
-  if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, 2, false, PP); \
+#define MI_LAUNCH_P(DD, PP)                                                                       \
+  if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, 2, false, PP);                               \
+  else if (shape == MI_SHAPE_PREFILL_WIDE) MI_LAUNCH((DD <= 128 ? DD : 128), MI_WIDE_WAVES, 1, MI_PREFILL_RG, 2, true, PP); \
   else MI_LAUNCH(DD, MI_PREFILL_WAVES, 1, MI_PREFILL_RG, MI_PREFILL_OCC(DD), true, PP)
 #define MI_LAUNCH_D(DD)                 \
   if (page_size == 16) {                \

@@ -636,6 +636,15 @@ def linear_swiglu(x: "torch.Tensor | ScaledRows", gate_up_weight: torch.Tensor) 
     return silu_mul(linear(x, gate_up_weight))
 
 
+# Launch shapes of the matrix-core attention kernel: 128-row prefill blocks, two to a CU; decode
+# blocks of 16 rows whose waves split the keys; and 256-row prefill blocks, one to a CU, which
+# fetch every key and value tile half as often but need more blocks than there are CUs several
+# times over, since the blocks of a causal prompt differ in length (one prompt, 8 key-value heads:
+# 2,048 tokens 101 against 69 us, 8,192 tokens 670 against 716 us, 131,072 tokens 130 against 140 ms).
+ATTN_SHAPE_PREFILL, ATTN_SHAPE_DECODE, ATTN_SHAPE_PREFILL_WIDE = 0, 1, 2
+WIDE_PREFILL_MIN_BLOCKS = 512
+
+
 def attention_splits(work_items: int, max_seq_len: int, target: int = 2048, min_keys: int = 256) -> int:
     """How many key ranges each work item is cut into so that the GPU is full.
 
@@ -932,15 +941,21 @@ def paged_attention(
             first_token = host_cu_seqlens_q[first]
             run_tokens = host_cu_seqlens_q[last] - first_token
             decode_only = max(lens) <= 1
-            tokens_per_tile = lib.mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, int(decode_only))
+            shape = ATTN_SHAPE_DECODE if decode_only else ATTN_SHAPE_PREFILL
+            if not decode_only and head_dim <= 128:
+                wide_tile = lib.mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, ATTN_SHAPE_PREFILL_WIDE)
+                wide_blocks = sum(-(-n // wide_tile) for n in lens) * kv_heads * -(-group // min(group, 256))
+                if wide_blocks >= WIDE_PREFILL_MIN_BLOCKS:
+                    shape = ATTN_SHAPE_PREFILL_WIDE
+            tokens_per_tile = lib.mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, shape)
             # 2: exactly one token per request (the kernel then needs no request boundaries)
             one_tile_per_request = 2 if (decode_only and min(lens) == 1) else int(max(lens) <= tokens_per_tile)
             num_tiles = count if one_tile_per_request else sum(-(-n // tokens_per_tile) for n in lens)
-            rows = 16 if decode_only else 128
+            rows = {ATTN_SHAPE_DECODE: 16, ATTN_SHAPE_PREFILL: 128, ATTN_SHAPE_PREFILL_WIDE: 256}[shape]
             head_blocks = -(-group // min(group, rows))
             # decode blocks are register-heavy (about one per CU at a time measured best at
-            # batch 1, 8 and 64); prefill blocks run two to a CU
-            target = 256 if decode_only else 512
+            # batch 1, 8 and 64) and a wide prefill block fills a CU; prefill blocks run two to a CU
+            target = 512 if shape == ATTN_SHAPE_PREFILL else 256
             # few requests with long contexts are cut finer (measured at batch 1: 128k keys
             # run 19 % faster in 32 ranges than in 16, 3k keys 4 % slower)
             most = 16 if max_seq_len < 8192 else 32
@@ -953,7 +968,7 @@ def paged_attention(
                     _ptr(cu_seqlens_q) + 4 * first, _ptr(positions), count, run_tokens,
                     num_tiles, _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads,
                     head_dim, page_size, num_pages, float(scale), int(window or 0), splits,
-                    int(decode_only), int(one_tile_per_request), first_token,
+                    shape, int(one_tile_per_request), first_token,
                     0 if (leave_pieces and splits > 1) else 1, _stream(),
                 )
             )

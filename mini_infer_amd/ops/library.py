@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None

@@ -556,6 +556,33 @@ def test_paged_attention_whole_long_prompts_many_tiles(window):
     assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(torch.bfloat16, 2)
 
 
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,page_size,window", [s for s in MFMA_SHAPES if s[2] <= 128])
+@pytest.mark.parametrize("lengths,q_lens", [
+    ([70, 33, 129, 64, 200], [70, 5, 1, 2, 37]),
+    ([2210, 37, 300], [2210, 37, 300]),
+    ([2500, 900, 700], [40, 3, 699]),
+])
+def test_paged_attention_in_blocks_of_256_rows(monkeypatch, q_heads, kv_heads, head_dim, page_size, window, lengths, q_lens):
+    """The launch shape that long prompts get (8 waves, 256 rows a block), forced here on
+    short ones: mixed portions, whole prompts over many tiles, portions late in a long
+    context (key ranges), groups of 1 to 20 heads; and the same through the usual shape."""
+    from mini_infer_amd.ops import kernels
+
+    case = _paged_case(torch.bfloat16, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=head_dim + 1,
+                       v_transposed=True)
+    scale = 1.0 / math.sqrt(head_dim)
+    usual = _attend(case, q_heads, kv_heads, head_dim, scale, window, max(lengths))
+    monkeypatch.setattr(kernels, "WIDE_PREFILL_MIN_BLOCKS", 1)
+    shapes = []
+    launch = kernels.library.load().mi_attn_mfma
+    monkeypatch.setattr(kernels.library.load(), "mi_attn_mfma", lambda *a: (shapes.append(a[23]), launch(*a))[1])
+    wide = _attend(case, q_heads, kv_heads, head_dim, scale, window, max(lengths))
+    assert shapes == [kernels.ATTN_SHAPE_PREFILL_WIDE]
+    expected = _attention_expected(case, scale, window)
+    assert np.abs(wide.double().cpu().numpy() - expected).max() < _tol(torch.bfloat16, 2)
+    assert np.abs(usual.double().cpu().numpy() - expected).max() < _tol(torch.bfloat16, 2)
+
+
 @pytest.mark.parametrize("mode,dtype", ATTENTION_MODES)
 def test_paged_attention_finds_one_far_key_and_respects_edges(mode, dtype):
     """One key among a thousand is made to stand out; the output must be its value.
