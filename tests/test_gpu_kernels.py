@@ -49,11 +49,12 @@ def test_embed_gather(dtype, hidden, vocab):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden", [4096, 100, 90, 9000])
-def test_add_rmsnorm(dtype, hidden):
+@pytest.mark.parametrize("hidden", [4096, 100, 90, 9000, 1000])
+@pytest.mark.parametrize("tokens", [7, 300])  # few rows; the rows of a prompt's portion
+def test_add_rmsnorm(dtype, hidden, tokens):
     from mini_infer_amd import ops
 
-    tokens, eps = 7, 3e-6
+    eps = 3e-6
     residual = _rand(tokens, hidden, seed=1, scale=2.0)
     delta = _rand(tokens, hidden, dtype=dtype, seed=2)
     weight = (_rand(hidden, seed=3) * 0.2 + 1.0).to(dtype)
@@ -81,11 +82,12 @@ def test_add_rmsnorm(dtype, hidden):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("inter", [14336, 130, 7])
-def test_silu_mul(dtype, inter):
+@pytest.mark.parametrize("inter", [14336, 130, 7, 136])
+@pytest.mark.parametrize("tokens", [5, 300])  # few rows; the rows of a prompt's portion
+def test_silu_mul(dtype, inter, tokens):
     from mini_infer_amd import ops
 
-    gate_up = _rand(5, 2 * inter, dtype=dtype, seed=4, scale=3.0)
+    gate_up = _rand(tokens, 2 * inter, dtype=dtype, seed=4, scale=3.0)
     gate_up[0, 0] = 0.0
     gate_up[0, 1 % inter] = 80.0
     gate_up[1, 0] = -80.0
@@ -295,16 +297,21 @@ def test_linear_falls_back_to_the_library_where_the_skinny_kernel_does_not_apply
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize(
     "q_heads,kv_heads,head_dim,rotary_dim,interleaved",
-    [(32, 8, 128, 128, False), (3, 1, 32, 32, False), (6, 3, 48, 16, False), (4, 2, 64, 64, True), (2, 2, 16, 0, False)],
+    [(32, 8, 128, 128, False), (3, 1, 32, 32, False), (6, 3, 48, 16, False), (4, 2, 64, 64, True), (2, 2, 16, 0, False),
+     (5, 1, 40, 24, False)],
 )
-def test_rope_kv_write(dtype, q_heads, kv_heads, head_dim, rotary_dim, interleaved):
+@pytest.mark.parametrize("tokens", [9, 300])  # few rows; the rows of a prompt's portion
+def test_rope_kv_write(dtype, q_heads, kv_heads, head_dim, rotary_dim, interleaved, tokens):
     from mini_infer_amd import ops
 
-    tokens, page_size, num_pages = 9, 4, 11
+    page_size = 4
+    num_pages = tokens + 2
     width = (q_heads + 2 * kv_heads) * head_dim
     qkv = _rand(tokens, width, dtype=dtype, seed=8)
     original = qkv.clone()
-    positions = torch.tensor([0, 1, 2, 3, 700, 701, 5, 6, 131071], dtype=torch.int32, device=DEV)
+    rng = np.random.default_rng(tokens)
+    some = [0, 1, 2, 3, 700, 701, 5, 6, 131071]
+    positions = torch.tensor(some + rng.integers(0, 131072, tokens - len(some)).tolist(), dtype=torch.int32, device=DEV)
     half = rotary_dim // 2
     if half:
         inv_freq = torch.from_numpy(pl.inv_freq_default(rotary_dim, 500000.0)).to(DEV)
@@ -315,7 +322,8 @@ def test_rope_kv_write(dtype, q_heads, kv_heads, head_dim, rotary_dim, interleav
     else:
         cos = sin = torch.empty((tokens, 0), dtype=torch.float32, device=DEV)
     # scattered slots, one token not written at all
-    slots = torch.tensor([40, 3, 17, 16, 0, 43, -1, 9, 22], dtype=torch.int32, device=DEV)
+    more = [int(x) for x in rng.permutation(num_pages * page_size) if x not in (40, 3, 17, 16, 0, 43, 9, 22)]
+    slots = torch.tensor([40, 3, 17, 16, 0, 43, -1, 9, 22] + more[: tokens - 9], dtype=torch.int32, device=DEV)
     k_pages = torch.zeros((num_pages, kv_heads, page_size, head_dim), dtype=dtype, device=DEV)
     v_pages = torch.zeros_like(k_pages)
     ops.rope_kv_write(qkv, cos, sin, slots, k_pages, v_pages, q_heads=q_heads, kv_heads=kv_heads,
@@ -363,13 +371,14 @@ def test_rope_kv_write(dtype, q_heads, kv_heads, head_dim, rotary_dim, interleav
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("page_size", [16, 8])
-def test_rope_kv_write_whole_pages_of_transposed_values(dtype, page_size):
+@pytest.mark.parametrize("more_pages", [0, 40])  # 40 more whole pages: the rows of a prompt's portion
+def test_rope_kv_write_whole_pages_of_transposed_values(dtype, page_size, more_pages):
     """Tokens that fill a page in order have their transposed values written a whole page at a
     time by the page's first token; pages filled out of order, from the middle, or only in
     part go token by token.  All give what the plain layout gives, transposed."""
     from mini_infer_amd import ops
 
-    q_heads, kv_heads, head_dim, num_pages = 4, 2, 32, 7
+    q_heads, kv_heads, head_dim, num_pages = 4, 2, 32, 7 + more_pages
     ps = page_size
     slots = (
         list(range(2 * ps, 3 * ps))  # page 2, in order: written at once
@@ -379,6 +388,7 @@ def test_rope_kv_write_whole_pages_of_transposed_values(dtype, page_size):
         + [-1]  # a token that is not written
         + list(range(6 * ps, 7 * ps))  # page 6, in order, at the very end of the step
         + list(range(3 * ps, 3 * ps + ps - 1))  # page 3 but for its last slot
+        + list(range(7 * ps, (7 + more_pages) * ps))  # (a token too late to start on a page's edge)
     )
     tokens = len(slots)
     qkv = _rand(tokens, (q_heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=21)
