@@ -867,6 +867,8 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
       out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, page_magic, scale_log2,    \
       window,                                                                                     \
       num_splits, hb, tq, one_tile_per_request, pair_group, first_token)
+// (head sizes above 128 have no wide shape and were refused above: their cases name the 128 kernel,
+// so that nothing is compiled for them)
 #define MI_LAUNCH_P(DD, PP)                                                                       \
   if (decode_only) MI_LAUNCH(DD, 1, MI_DECODE_KW, 1, 2, false, PP);                               \
   else if (shape == MI_SHAPE_PREFILL_WIDE) MI_LAUNCH((DD <= 128 ? DD : 128), MI_WIDE_WAVES, 1, MI_PREFILL_RG, 2, true, PP); \

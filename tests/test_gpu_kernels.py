@@ -429,9 +429,10 @@ def _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, 
         at += pages_per[b]
         k = torch.from_numpy(rng.standard_normal((n, kv_heads, head_dim))).to(dtype)
         v = torch.from_numpy(rng.standard_normal((n, kv_heads, head_dim))).to(dtype)
-        for p in range(n):
-            k_pages[table[b, p // page_size], :, p % page_size] = k[p]
-            v_pages[table[b, p // page_size], :, p % page_size] = v[p]
+        at_page = torch.from_numpy(table[b, np.arange(n) // page_size].astype(np.int64))
+        at_slot = torch.arange(n) % page_size
+        k_pages[at_page, :, at_slot] = k
+        v_pages[at_page, :, at_slot] = v
         q = torch.from_numpy(rng.standard_normal((q_lens[b], q_heads, head_dim))).to(dtype)
         ks.append(k), vs.append(v), qs.append(q)
         token_request += [b] * q_lens[b]
@@ -569,8 +570,9 @@ def test_paged_attention_whole_long_prompts_many_tiles(window):
 @pytest.mark.parametrize("q_heads,kv_heads,head_dim,page_size,window", [s for s in MFMA_SHAPES if s[2] <= 128])
 @pytest.mark.parametrize("lengths,q_lens", [
     ([70, 33, 129, 64, 200], [70, 5, 1, 2, 37]),
-    ([2210, 37, 300], [2210, 37, 300]),
+    ([900, 37, 300], [900, 37, 300]),
     ([2500, 900, 700], [40, 3, 699]),
+    ([1500, 17, 640, 300], [1, 1, 140, 90]),  # single tokens first: a launch of their own in the decode shape
 ])
 def test_paged_attention_in_blocks_of_256_rows(monkeypatch, q_heads, kv_heads, head_dim, page_size, window, lengths, q_lens):
     """The launch shape that long prompts get (8 waves, 256 rows a block), forced here on
@@ -587,7 +589,7 @@ def test_paged_attention_in_blocks_of_256_rows(monkeypatch, q_heads, kv_heads, h
     launch = kernels.library.load().mi_attn_mfma
     monkeypatch.setattr(kernels.library.load(), "mi_attn_mfma", lambda *a: (shapes.append(a[23]), launch(*a))[1])
     wide = _attend(case, q_heads, kv_heads, head_dim, scale, window, max(lengths))
-    assert shapes == [kernels.ATTN_SHAPE_PREFILL_WIDE]
+    assert shapes == [kernels.ATTN_SHAPE_DECODE] * (q_lens[0] == 1) + [kernels.ATTN_SHAPE_PREFILL_WIDE]
     expected = _attention_expected(case, scale, window)
     assert np.abs(wide.double().cpu().numpy() - expected).max() < _tol(torch.bfloat16, 2)
     assert np.abs(usual.double().cpu().numpy() - expected).max() < _tol(torch.bfloat16, 2)
