@@ -595,6 +595,43 @@ def test_paged_attention_in_blocks_of_256_rows(monkeypatch, q_heads, kv_heads, h
     assert np.abs(usual.double().cpu().numpy() - expected).max() < _tol(torch.bfloat16, 2)
 
 
+@pytest.mark.parametrize("rows_per_block", [128, 256])
+@pytest.mark.parametrize("window", [None, 100])
+def test_paged_attention_prompt_rows_find_planted_keys(monkeypatch, rows_per_block, window):
+    """A whole prompt of 1,000 tokens in both prefill shapes: for chosen (query, key) pairs the
+    key is made to stand out for that query, so the query's output must be that key's value.
+    The pairs sit on the diagonal, at the first and last key, on both sides of the edges of the
+    32-key tiles and of the 64- and 128-token row tiles, and on the window's edge; a tile that
+    is skipped or masked wrongly, which random keys would hide in the tolerance, shows."""
+    from mini_infer_amd.ops import kernels
+
+    q_heads, kv_heads, head_dim, page_size, length = 2, 1, 64, 16, 1000
+    scale = 1.0 / 8.0
+    pairs = [(999, 0), (998, 998), (64, 64), (65, 63), (127, 96), (128, 127), (129, 129), (500, 31), (501, 32),
+             (700, 255), (701, 256), (300, 201), (330, 300), (63, 2), (257, 254)]
+    if window is not None:
+        pairs = [(t, p) for t, p in pairs if t - p < window] + [(999, 900), (400, 301), (161, 62), (192, 93)]
+    case = _paged_case(torch.bfloat16, q_heads, kv_heads, head_dim, page_size, [length], [length], seed=31,
+                       v_transposed=True)
+    assert len({p for _, p in pairs}) == len(pairs) == len({t for t, _ in pairs})
+    for t, p in pairs:
+        key = (case["qs"][0][t, 0].float() * 6.0).to(torch.bfloat16)  # score 6 |q|^2 / 8 = 48 +- a few
+        case["ks"][0][p, 0] = key
+        case["k_pages"][case["block_table"][0, p // page_size].item(), 0, p % page_size] = key.to(DEV)
+    if rows_per_block == 256:
+        monkeypatch.setattr(kernels, "WIDE_PREFILL_MIN_BLOCKS", 1)
+    shapes = []
+    launch = kernels.library.load().mi_attn_mfma
+    monkeypatch.setattr(kernels.library.load(), "mi_attn_mfma", lambda *a: (shapes.append(a[23]), launch(*a))[1])
+    out = _attend(case, q_heads, kv_heads, head_dim, scale, window, length)
+    assert shapes == [kernels.ATTN_SHAPE_PREFILL_WIDE if rows_per_block == 256 else kernels.ATTN_SHAPE_PREFILL]
+    out = out.float().cpu().reshape(length, q_heads, head_dim)
+    for t, p in pairs:
+        assert (out[t, 0] - case["vs"][0][p, 0].float()).abs().max() < 2e-2, (t, p)
+    expected = _attention_expected(case, scale, window)
+    assert np.abs(out.reshape(length, -1).double().numpy() - expected).max() < _tol(torch.bfloat16, 2)
+
+
 @pytest.mark.parametrize("mode,dtype", ATTENTION_MODES)
 def test_paged_attention_finds_one_far_key_and_respects_edges(mode, dtype):
     """One key among a thousand is made to stand out; the output must be its value.
