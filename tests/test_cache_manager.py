@@ -33,6 +33,16 @@ def test_pool_allocates_unique_pages_and_notices_double_free():
     pool.check()
 
 
+def test_fresh_pool_hands_out_scattered_ids_the_same_every_time():
+    """Requests that grow side by side must not end up with neighbouring pages: a fresh pool's
+    ids come in a scattered order, the same one for a pool size."""
+    first = PagePool(256).allocate_many(256)
+    assert first == PagePool(256).allocate_many(256)
+    assert sorted(first) == list(range(256))
+    neighbours = sum(1 for a, b in zip(first, first[1:]) if abs(a - b) == 1)
+    assert neighbours < 16
+
+
 def test_allocate_many_is_all_or_nothing():
     pool = PagePool(3)
     pool.allocate()
