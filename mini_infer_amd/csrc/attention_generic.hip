@@ -2,8 +2,17 @@
 // the fallback for sizes the matrix-core kernels refuse.  One 64-lane wave per
 // (query token, key/value head, up to 4 query heads of its group, key split).
 // Lanes own keys while scores are computed (one key row per lane, q broadcast
-// from LDS) and own output dims while values are accumulated.  Scores, softmax
-// and the value sum are float32 with an online (running max) softmax.
+// from LDS) and own output dims while values are accumulated.  The softmax is an
+// online one (running max).  For bfloat16 inputs the scores, the softmax's sum and the
+// value sum are float32.  For float32 inputs (the engine's 32-bit path) they are kept in
+// 64-bit: a float32 sum over thousands of keys is rounded at every key, which alone put
+// the relative error of a 2,000-key row at 6e-7, twenty-five times what rounding the
+// result once costs (and more than everything else in a layer together); in 64-bit the
+// row is rounded once, when it is written.
+//
+// Head sizes: any even one up to 256.  Multiples of 16 read keys and values 16 bytes at a
+// time; the others read them in pairs of elements (rows of an even head size are always
+// aligned to that) and guard every access past the row's end.
 //
 // Semantics follow the reference's oracle (cache/packed_attention.py:296-338):
 // query head h reads key/value head h / (Hq/Hkv); a query at absolute position p
@@ -28,7 +37,24 @@ struct alignas(sizeof(T) * N) Pack {
   T v[N];
 };
 
-template <typename T, int VPL>
+// what sums are kept in: see the note at the top
+template <typename T>
+struct SumType {
+  using type = float;
+};
+template <>
+struct SumType<float> {
+  using type = double;
+};
+
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+  for (int off = MI_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, MI_WAVE);
+  return v;
+}
+
+// VEC: head_dim is a multiple of 16 (16-byte loads, no guards inside a row)
+template <typename T, int VPL, bool VEC>
 __global__ __launch_bounds__(64) void attn_generic_kernel(
     const T* __restrict__ q, int64_t q_row_stride, const T* __restrict__ k_pages,
     const T* __restrict__ v_pages, const int* __restrict__ block_table, int max_blocks,
@@ -36,8 +62,10 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     int64_t out_row_stride, float* __restrict__ part_acc, float* __restrict__ part_ml, int q_heads,
     int kv_heads, int head_dim, int page_size, float scale, int window, int num_splits,
     const float* __restrict__ slopes) {
-  extern __shared__ float q_lds[];  // [GT][head_dim], pre-multiplied by the scale
-  constexpr int KV = 16 / sizeof(T);  // elements in a 16-byte load
+  using S = typename SumType<T>::type;
+  extern __shared__ __align__(8) unsigned char q_lds_bytes[];
+  S* q_lds = reinterpret_cast<S*>(q_lds_bytes);  // [GT][head_dim], pre-multiplied by the scale
+  constexpr int KV = VEC ? 16 / sizeof(T) : 4;  // elements per step along a key row
 
   const int t = blockIdx.x;
   const int group = q_heads / kv_heads;
@@ -51,7 +79,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
 
   const T* q_row = q + (int64_t)t * q_row_stride + (int64_t)head0 * head_dim;
   for (int i = lane; i < GT * head_dim; i += MI_WAVE)
-    q_lds[i] = (i < nh * head_dim) ? to_f32(q_row[i]) * scale : 0.f;
+    q_lds[i] = (i < nh * head_dim) ? (S)to_f32(q_row[i]) * (S)scale : (S)0;
   __syncthreads();
 
   const int pos = positions[t];
@@ -64,13 +92,14 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
   const int b = min(a + chunk, hi);
   const int* bt = block_table + (int64_t)req * max_blocks;
 
-  float m[GT], l[GT], acc[GT][VPL];
+  float m[GT];
+  S l[GT], acc[GT][VPL];
 #pragma unroll
   for (int g = 0; g < GT; ++g) {
     m[g] = -INFINITY;
-    l[g] = 0.f;
+    l[g] = 0;
 #pragma unroll
-    for (int v = 0; v < VPL; ++v) acc[g][v] = 0.f;
+    for (int v = 0; v < VPL; ++v) acc[g][v] = 0;
   }
   const bool owns_dims = lane * VPL < head_dim;
   float slope[GT];
@@ -81,44 +110,73 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     const int key = base + lane;
     const bool valid = key < b;
     int row_idx = 0;
-    float s[GT];
+    float s[GT];  // the score less nothing yet; below: less the running maximum
+    S s_sum[GT];
 #pragma unroll
-    for (int g = 0; g < GT; ++g) s[g] = -INFINITY;
+    for (int g = 0; g < GT; ++g) {
+      s[g] = -INFINITY;
+      s_sum[g] = 0;
+    }
     if (valid) {
       const int page = bt[key / page_size];
       row_idx = (page * kv_heads + kvh) * page_size + key % page_size;
       const T* k_row = k_pages + (int64_t)row_idx * head_dim;
       // four running sums per score (dims d, d+1, d+2, d+3 of every group of four), added
       // at the end: shorter chains of roundings than one sum over the whole head
-      float s4[GT][4];
+      S s4[GT][4];
 #pragma unroll
       for (int g = 0; g < GT; ++g)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) s4[g][e] = 0.f;
+        for (int e = 0; e < 4; ++e) s4[g][e] = 0;
       for (int d = 0; d < head_dim; d += KV) {
-        const Pack<T, KV> kk = *reinterpret_cast<const Pack<T, KV>*>(k_row + d);
+        float kf[KV];
+        if constexpr (VEC) {
+          const Pack<T, KV> kk = *reinterpret_cast<const Pack<T, KV>*>(k_row + d);
+#pragma unroll
+          for (int e = 0; e < KV; ++e) kf[e] = to_f32(kk.v[e]);
+        } else {
+          // pairs of elements; an even head size ends after the first or the second pair
+          const Pack<T, 2> k0 = *reinterpret_cast<const Pack<T, 2>*>(k_row + d);
+          kf[0] = to_f32(k0.v[0]);
+          kf[1] = to_f32(k0.v[1]);
+          kf[2] = kf[3] = 0.f;
+          if (d + 2 < head_dim) {
+            const Pack<T, 2> k1 = *reinterpret_cast<const Pack<T, 2>*>(k_row + d + 2);
+            kf[2] = to_f32(k1.v[0]);
+            kf[3] = to_f32(k1.v[1]);
+          }
+        }
 #pragma unroll
         for (int e = 0; e < KV; ++e) {
-          const float kf = to_f32(kk.v[e]);
+          if (!VEC && d + e >= head_dim) break;
 #pragma unroll
-          for (int g = 0; g < GT; ++g) s4[g][e % 4] = fmaf(q_lds[g * head_dim + d + e], kf, s4[g][e % 4]);
+          for (int g = 0; g < GT; ++g) {
+            const S qv = q_lds[g * head_dim + d + e];
+            if constexpr (sizeof(S) == 8) s4[g][e % 4] = fma(qv, (S)kf[e], s4[g][e % 4]);
+            else s4[g][e % 4] = fmaf(qv, kf[e], s4[g][e % 4]);
+          }
         }
       }
+      const S distance = (S)(key - pos);
 #pragma unroll
-      for (int g = 0; g < GT; ++g) s[g] = (s4[g][0] + s4[g][1]) + (s4[g][2] + s4[g][3]);
-      const float distance = (float)(key - pos);
-#pragma unroll
-      for (int g = 0; g < GT; ++g) s[g] += slope[g] * distance;
+      for (int g = 0; g < GT; ++g) {
+        s_sum[g] = (s4[g][0] + s4[g][1]) + (s4[g][2] + s4[g][3]);
+        s_sum[g] += (S)slope[g] * distance;
+        s[g] = (float)s_sum[g];
+      }
     }
     float p[GT];
 #pragma unroll
     for (int g = 0; g < GT; ++g) {
       const float m_new = fmaxf(m[g], wave_max(s[g]));
       const float alpha = expf(m[g] - m_new);
-      p[g] = valid ? expf(s[g] - m_new) : 0.f;
-      l[g] = l[g] * alpha + wave_sum(p[g]);
+      // (64-bit sums: the difference is taken and the exponential made before anything is
+      // rounded to float32, so a key's weight is off by one rounding, not by the score's)
+      if constexpr (sizeof(S) == 8) p[g] = valid ? (float)exp(s_sum[g] - (S)m_new) : 0.f;
+      else p[g] = valid ? expf(s_sum[g] - m_new) : 0.f;
+      l[g] = l[g] * (S)alpha + wave_sum((S)p[g]);
 #pragma unroll
-      for (int v = 0; v < VPL; ++v) acc[g][v] *= alpha;
+      for (int v = 0; v < VPL; ++v) acc[g][v] *= (S)alpha;
       m[g] = m_new;
     }
     const int n_valid = min(MI_WAVE, b - base);
@@ -128,16 +186,27 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
 #pragma unroll
       for (int v = 0; v < VPL; ++v) vv[v] = 0.f;
       if (owns_dims) {
-        const Pack<T, VPL> pk =
-            *reinterpret_cast<const Pack<T, VPL>*>(v_pages + (int64_t)rj * head_dim + lane * VPL);
+        const T* v_row = v_pages + (int64_t)rj * head_dim + lane * VPL;
+        if constexpr (VEC || VPL <= 2) {  // (an even head size: a pair never straddles the row's end)
+          const Pack<T, VPL> pk = *reinterpret_cast<const Pack<T, VPL>*>(v_row);
 #pragma unroll
-        for (int v = 0; v < VPL; ++v) vv[v] = to_f32(pk.v[v]);
+          for (int v = 0; v < VPL; ++v) vv[v] = to_f32(pk.v[v]);
+        } else {
+#pragma unroll
+          for (int v = 0; v < VPL; v += 2) {
+            if (lane * VPL + v < head_dim) {
+              const Pack<T, 2> pk = *reinterpret_cast<const Pack<T, 2>*>(v_row + v);
+              vv[v] = to_f32(pk.v[0]);
+              vv[v + 1] = to_f32(pk.v[1]);
+            }
+          }
+        }
       }
 #pragma unroll
       for (int g = 0; g < GT; ++g) {
         const float pj = __shfl(p[g], j, MI_WAVE);
 #pragma unroll
-        for (int v = 0; v < VPL; ++v) acc[g][v] += pj * vv[v];
+        for (int v = 0; v < VPL; ++v) acc[g][v] += (S)pj * (S)vv[v];
       }
     }
   }
@@ -148,9 +217,10 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
       for (int g = 0; g < GT; ++g) {
         if (g < nh) {
           T* o = out + (int64_t)t * out_row_stride + (int64_t)(head0 + g) * head_dim + lane * VPL;
-          const float inv = 1.f / l[g];
+          const S inv = (S)1 / l[g];
 #pragma unroll
-          for (int v = 0; v < VPL; ++v) o[v] = from_f32<T>(acc[g][v] * inv);
+          for (int v = 0; v < VPL; ++v)
+            if (VEC || lane * VPL + v < head_dim) o[v] = from_f32<T>((float)(acc[g][v] * inv));
         }
       }
     }
@@ -161,11 +231,12 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
         const int64_t slot = ((int64_t)t * q_heads + head0 + g) * num_splits + split;
         if (owns_dims) {
 #pragma unroll
-          for (int v = 0; v < VPL; ++v) part_acc[slot * head_dim + lane * VPL + v] = acc[g][v];
+          for (int v = 0; v < VPL; ++v)
+            if (VEC || lane * VPL + v < head_dim) part_acc[slot * head_dim + lane * VPL + v] = (float)acc[g][v];
         }
         if (lane == 0) {
           part_ml[slot * 2] = m[g];
-          part_ml[slot * 2 + 1] = l[g];
+          part_ml[slot * 2 + 1] = (float)l[g];
         }
       }
     }
@@ -180,6 +251,7 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
                                                          const float* __restrict__ part_ml,
                                                          T* __restrict__ out, int64_t out_row_stride,
                                                          int q_heads, int head_dim, int num_splits) {
+  using S = typename SumType<T>::type;
   const int t = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x;
   const int64_t base = ((int64_t)t * q_heads + h) * num_splits;
@@ -205,9 +277,9 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
   const float l_s = (lane < num_splits) ? part_ml[(base + lane) * 2 + 1] : 0.f;
   const float m_all = wave_max(m_s);
   const float w_s = (lane < num_splits) ? expf(m_s - m_all) : 0.f;
-  float l_all = 0.f;
-  for (int s = 0; s < num_splits; ++s) l_all += __shfl(l_s * w_s, s, MI_WAVE);
-  const float inv = 1.f / l_all;
+  S l_all = 0;
+  for (int s = 0; s < num_splits; ++s) l_all += (S)__shfl(l_s, s, MI_WAVE) * (S)__shfl(w_s, s, MI_WAVE);
+  const S inv = (S)1 / l_all;
   // The partial accumulators are read in batches of independent loads (a load per split
   // issued one after the other's use would cost a memory latency per split) and added in
   // split order.
@@ -215,13 +287,13 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int d = half * MI_WAVE + lane;
-      float o = 0.f;
+      S o = 0;
 #pragma unroll
       for (int i = 0; i < BATCH; ++i) {
         const float w = __shfl(w_s, i, MI_WAVE);
-        if (i < num_splits) o += early[half][i] * w;
+        if (i < num_splits) o += (S)early[half][i] * (S)w;
       }
-      if (d < head_dim) out[(int64_t)t * out_row_stride + (int64_t)h * head_dim + d] = from_f32<T>(o * inv);
+      if (d < head_dim) out[(int64_t)t * out_row_stride + (int64_t)h * head_dim + d] = from_f32<T>((float)(o * inv));
     }
     return;
   }
@@ -229,7 +301,7 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
     const int d = d0 + lane;
     const bool active = d < head_dim;
     const float* src = part_acc + base * head_dim + (active ? d : 0);
-    float o = 0.f;
+    S o = 0;
     for (int s0 = 0; s0 < num_splits; s0 += BATCH) {
       float v[BATCH];
 #pragma unroll
@@ -240,10 +312,10 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
 #pragma unroll
       for (int i = 0; i < BATCH; ++i) {
         const float w = __shfl(w_s, min(s0 + i, MI_WAVE - 1), MI_WAVE);
-        if (s0 + i < num_splits) o += v[i] * w;
+        if (s0 + i < num_splits) o += (S)v[i] * (S)w;
       }
     }
-    if (active) out[(int64_t)t * out_row_stride + (int64_t)h * head_dim + d] = from_f32<T>(o * inv);
+    if (active) out[(int64_t)t * out_row_stride + (int64_t)h * head_dim + d] = from_f32<T>((float)(o * inv));
   }
 }
 
@@ -257,15 +329,16 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
                                const float* slopes, hipStream_t stream) {
   const int group = q_heads / kv_heads;
   dim3 grid(num_tokens, kv_heads * ceil_div(group, GT), num_splits);
-  const size_t lds = sizeof(float) * GT * head_dim;
-#define MI_ATTN_LAUNCH(VPL)                                                                       \
-  attn_generic_kernel<T, VPL><<<grid, MI_WAVE, lds, stream>>>(                                    \
+  const size_t lds = sizeof(typename SumType<T>::type) * GT * head_dim;
+  const bool vec = head_dim % 16 == 0;
+#define MI_ATTN_LAUNCH(VPL, VEC)                                                                  \
+  attn_generic_kernel<T, VPL, VEC><<<grid, MI_WAVE, lds, stream>>>(                               \
       (const T*)q, q_row_stride, (const T*)k_pages, (const T*)v_pages, block_table, max_blocks,   \
       token_request, positions, (T*)out, out_row_stride, part_acc, part_ml, q_heads, kv_heads,    \
       head_dim, page_size, scale, window, num_splits, slopes)
-  if (head_dim <= 64) MI_ATTN_LAUNCH(1);
-  else if (head_dim <= 128) MI_ATTN_LAUNCH(2);
-  else MI_ATTN_LAUNCH(4);
+  if (head_dim <= 64) { if (vec) MI_ATTN_LAUNCH(1, true); else MI_ATTN_LAUNCH(1, false); }
+  else if (head_dim <= 128) { if (vec) MI_ATTN_LAUNCH(2, true); else MI_ATTN_LAUNCH(2, false); }
+  else { if (vec) MI_ATTN_LAUNCH(4, true); else MI_ATTN_LAUNCH(4, false); }
 #undef MI_ATTN_LAUNCH
   MI_CHECK_LAUNCH("attn_generic");
   if (num_splits > 1) {
@@ -284,8 +357,8 @@ static int attn_generic_check(int dtype, int64_t q_row_stride, int max_blocks, i
              num_tokens, q_heads, kv_heads);
   MI_REQUIRE(q_heads % kv_heads == 0, "attn_generic: q_heads=%d is not a multiple of kv_heads=%d",
              q_heads, kv_heads);
-  MI_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
-             "attn_generic: head_dim=%d must be a multiple of 16 and at most 256", head_dim);
+  MI_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= 256,
+             "attn_generic: head_dim=%d must be even and at most 256", head_dim);
   MI_REQUIRE(page_size > 0 && num_pages > 0 && max_blocks > 0, "attn_generic: bad page sizes page_size=%d num_pages=%d max_blocks=%d",
              page_size, num_pages, max_blocks);
   MI_REQUIRE((int64_t)num_pages * kv_heads * page_size < (int64_t)1 << 31,

@@ -1,9 +1,11 @@
 // True float32 matrix product for the 32-bit path: C[M,N] = A[M,K] * W[N,K]^T.
 // Plain FMA, no reduced-precision matrix mode.  Each output element is summed by
-// one thread in a fixed order (16-deep slices, slice by slice), so a row's result
-// does not depend on how many other rows are in the batch or on where its tile lies.
-// The slices' sums are added up with compensation (Kahan), so the rounding error of a
-// long row (K in the thousands) stays at a few units in the last place whatever K is.
+// one thread in the order of k, so a row's result does not depend on how many other
+// rows are in the batch or on where its tile lies.  The sum is carried in 64-bit and
+// rounded to float32 once, when it is written: an output differs from the exact product
+// of its float32 operands by that one rounding (relative 2.5e-8 on average), whatever K
+// is.  (Float32 sums in 16-deep slices added up with compensation measured 8e-8 at K =
+// 4,096, a plain float32 sum 2.7e-6; over 32 layers such errors are what the logits show.)
 //
 // 64x64 output tile per 256-thread block, 16-deep K slices staged in LDS, 4x4
 // outputs per thread.  Any M, N, K; rows of A and W may have strides.
@@ -29,11 +31,11 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
   const int l_row = tid / 4;
   const int l_k = (tid % 4) * 4;
 
-  float acc[4][4], lost[4][4];  // running sums and what their roundings have dropped so far
+  double acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = lost[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.0;
 
   for (int k0 = 0; k0 < k; k0 += BK) {
     {
@@ -51,33 +53,18 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
         w_s[l_k + i][l_row] = (r < n && k0 + l_k + i < k) ? src[i] : 0.f;
     }
     __syncthreads();
-    // two-level sum: each 16-deep slice is summed on its own, then added to the total
-    float part[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) part[i][j] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < BK; ++kk) {
-      float av[4], wv[4];
+      double av[4], wv[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) av[i] = a_s[kk][ty * 4 + i];
+      for (int i = 0; i < 4; ++i) av[i] = (double)a_s[kk][ty * 4 + i];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) wv[j] = w_s[kk][tx * 4 + j];
+      for (int j = 0; j < 4; ++j) wv[j] = (double)w_s[kk][tx * 4 + j];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) part[i][j] = fmaf(av[i], wv[j], part[i][j]);
+        for (int j = 0; j < 4; ++j) acc[i][j] = fma(av[i], wv[j], acc[i][j]);
     }
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float y = part[i][j] - lost[i][j];
-        const float t = acc[i][j] + y;
-        lost[i][j] = (t - acc[i][j]) - y;
-        acc[i][j] = t;
-      }
     __syncthreads();
   }
 
@@ -88,7 +75,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int col = col0 + tx * 4 + j;
-      if (col < n) c[(int64_t)r * ldc + col] = acc[i][j];
+      if (col < n) c[(int64_t)r * ldc + col] = (float)acc[i][j];
     }
   }
 }
@@ -96,9 +83,9 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 // The same product for at most 16 rows (decode): a 64x64 tile would be three quarters empty and
 // its 16-byte loads per thread leave most of the memory system idle.  A block owns all rows
 // and 32 or 64 features; W is staged 64 deep (256 contiguous bytes of a row by a few threads),
-// and a thread sums one row x two or four features.  Every output is summed EXACTLY as above: 16-deep
-// slices, each from zero in the order of k, added up with the same compensation; so a row
-// gives the same bits whichever of the two kernels its step takes.
+// and a thread sums one row x two or four features.  Every output is summed EXACTLY as above (in
+// the order of k, in 64-bit, rounded once); so a row gives the same bits whichever of the two
+// kernels its step takes.
 #define RM 16
 #define RK 64
 
@@ -120,9 +107,9 @@ __global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restr
   const int w_feature = tid / (RK / W_PER), w_k = (tid % (RK / W_PER)) * W_PER;
   const int w_row = col0 + w_feature;
   const int a_row = tid / 16, a_k = (tid % 16) * 4;
-  float acc[TN], lost[TN];
+  double acc[TN];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) acc[j] = lost[j] = 0.f;
+  for (int j = 0; j < TN; ++j) acc[j] = 0.0;
   for (int k0 = 0; k0 < k; k0 += RK) {
     {
       const float* src = w + (int64_t)w_row * ldw + k0 + w_k;
@@ -146,25 +133,12 @@ __global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restr
       for (int i = 0; i < 4; ++i) a_s[a_k + i][a_row] = (a_row < m && k0 + a_k + i < k) ? src[i] : 0.f;
     }
     __syncthreads();
+    // (staged values past K are zeros: they add nothing, exactly)
 #pragma unroll
-    for (int slice = 0; slice < RK / BK; ++slice) {
-      if (k0 + slice * BK >= k) break;  // (the same for every thread; a slice past K is not summed at all)
-      float part[TN];
+    for (int kk = 0; kk < RK; ++kk) {
+      const double av = (double)a_s[kk][row];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) part[j] = 0.f;
-#pragma unroll
-      for (int kk = 0; kk < BK; ++kk) {
-        const float av = a_s[slice * BK + kk][row];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) part[j] = fmaf(av, w_s[slice * BK + kk][TN * tx + j], part[j]);
-      }
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const float y = part[j] - lost[j];
-        const float t = acc[j] + y;
-        lost[j] = (t - acc[j]) - y;
-        acc[j] = t;
-      }
+      for (int j = 0; j < TN; ++j) acc[j] = fma(av, (double)w_s[kk][TN * tx + j], acc[j]);
     }
     __syncthreads();
   }
@@ -172,7 +146,7 @@ __global__ __launch_bounds__(256) void gemm_f32_rows_kernel(const float* __restr
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int col = col0 + TN * tx + j;
-      if (col < n) c[(int64_t)row * ldc + col] = acc[j];
+      if (col < n) c[(int64_t)row * ldc + col] = (float)acc[j];
     }
   }
 }

@@ -55,8 +55,9 @@ def _check_v_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, v_transposed: b
 
 
 MFMA_HEAD_DIMS = (32, 64, 96, 128, 192, 256)
-# what the plain attention kernel (and so the engine as a whole) takes
-ATTENTION_HEAD_DIM_STEP = 16
+# what the plain attention kernel (and so the engine as a whole) takes: any even head size up
+# to 256 (a rotation pairs dims, so an odd one has no meaning here)
+ATTENTION_HEAD_DIM_STEP = 2
 ATTENTION_MAX_HEAD_DIM = 256
 
 

@@ -54,8 +54,8 @@ class GQAttention(Mixer):
             raise ValueError(f"window must be positive, got {window}")
         if head_dim <= 0 or head_dim % ops.ATTENTION_HEAD_DIM_STEP != 0 or head_dim > ops.ATTENTION_MAX_HEAD_DIM:
             raise ValueError(
-                f"head_dim={head_dim}: the attention kernels take head sizes in steps of "
-                f"{ops.ATTENTION_HEAD_DIM_STEP} up to {ops.ATTENTION_MAX_HEAD_DIM}"
+                f"head_dim={head_dim}: the attention kernels take even head sizes "
+                f"up to {ops.ATTENTION_MAX_HEAD_DIM}"
             )
         self.hidden_size = hidden_size
         self.num_heads = num_heads

@@ -479,6 +479,12 @@ PLAIN_SHAPES = [
     (10, 2, 80, 64, None),
     (4, 4, 256, 16, 40),
     (12, 2, 112, 32, None),
+    # head sizes no 16-byte load divides: read in pairs of elements, every row's end guarded
+    (8, 2, 100, 16, None),
+    (6, 3, 40, 4, 21),
+    (3, 1, 2, 4, None),
+    (4, 2, 130, 16, None),
+    (5, 1, 254, 8, 50),
 ]
 MFMA_SHAPES = [
     (32, 8, 128, 16, None),
@@ -551,6 +557,36 @@ def test_paged_attention_single_tokens_first_then_portions(mode, dtype):
     out = _attend(case, q_heads, kv_heads, head_dim, 0.15, None, max(lengths))
     expected = _attention_expected(case, 0.15, None)
     assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
+
+
+def test_float32_attention_over_thousands_of_keys_is_rounded_once():
+    """The 32-bit path's attention keeps its sums in 64-bit: the output of a row over 2,500 keys
+    differs from the exact one by about one float32 rounding (relative 2.5e-8 on average).  A
+    float32 sum that is rounded at every key is 6e-7 away at this length, which 32 layers
+    turn into logits off by more than 1e-4."""
+    q_heads, kv_heads, head_dim, page_size = 8, 2, 128, 16
+    lengths, q_lens = [2500, 1800], [300, 1]
+    case = _paged_case(torch.float32, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=9)
+    scale = 0.35  # scores of a few units either way: some keys stand out, hundreds still count
+    out = _attend(case, q_heads, kv_heads, head_dim, scale, None, max(lengths)).double().cpu().numpy()
+    expected = _attention_expected(case, scale, None)
+    relative = np.linalg.norm(out - expected) / np.linalg.norm(expected)
+    assert relative < 6e-8, f"relative error {relative:.2e}"
+
+
+def test_float32_product_is_rounded_once():
+    """`gemm_f32` carries its sums in 64-bit: a sum over 14,336 terms is one float32 rounding
+    away from exact (2.5e-8 on average), in the many-row and in the few-row kernel alike."""
+    from mini_infer_amd import ops
+
+    a = _rand(40, 14336, seed=1).to(DEV)
+    w = _rand(96, 14336, seed=2).to(DEV)
+    exact = a.double() @ w.double().T
+    for rows in (40, 7):
+        got = ops.gemm_f32(a[:rows], w).double()
+        relative = float((got - exact[:rows]).norm() / exact[:rows].norm())
+        assert relative < 4e-8, f"{rows} rows: relative error {relative:.2e}"
+    assert torch.equal(ops.gemm_f32(a[:7], w), ops.gemm_f32(a, w)[:7])  # a row's bits do not depend on its company
 
 
 @pytest.mark.parametrize("window", [None, 700])
@@ -869,9 +905,10 @@ def test_kernels_refuse_what_they_do_not_take():
     from mini_infer_amd import ops
     from mini_infer_amd.exceptions import KernelShapeError
 
-    case = _paged_case(torch.float32, 4, 2, 24, 4, [5], [1])
-    with pytest.raises(KernelShapeError, match="multiple of 16"):
-        _attend(case, 4, 2, 24, 1.0, None, 5)
+    for head_dim, message in ((25, "even"), (258, "at most 256")):
+        case = _paged_case(torch.float32, 4, 2, head_dim, 4, [5], [1])
+        with pytest.raises(KernelShapeError, match=message):
+            _attend(case, 4, 2, head_dim, 1.0, None, 5)
     # transposed value pages belong to the matrix-core kernel, which takes bfloat16 only
     case = _paged_case(torch.float32, 4, 2, 32, 16, [5], [1], v_transposed=True)
     with pytest.raises(KernelShapeError, match="matrix-core"):

@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 LENGTHS = [5, 33, 70, 97, 41, 64]
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C", "D"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "D", "E", "F"])
 def case(request, tmp_path_factory):
     name = request.param
     cfg, block = tiny.CONFIGS[name]

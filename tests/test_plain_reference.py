@@ -310,7 +310,7 @@ def test_torch_twin_of_the_plain_model_equals_it():
     of the stored tensors, whole and at chosen rows."""
     import plain_llama_torch as plt
 
-    for name in "ABCD":
+    for name in "ABCDEF":
         cfg, _ = tiny.CONFIGS[name]
         weights = tiny.make_weights(cfg, 40 + ord(name))
         tokens = tiny.random_tokens(cfg, 70, 5)

@@ -27,7 +27,7 @@ def _model(cfg, dtype=torch.float32):
     return DecoderModel(arch.build_spec(arch.parse_config(cfg)), dtype, "cpu")
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F"])
 def test_model_names_are_the_checkpoint_names(name):
     cfg, _ = tiny.CONFIGS[name]
     specs = _model(cfg).param_specs()

@@ -6,7 +6,8 @@ the norms' eps, tied or untied head.  A and B are the two named in the project's
 baseline; C adds sizes that no vector width divides; D has the smallest sizes at
 which every fast path of the bfloat16 engine runs (weight rows of whole cache
 lines read as such, both norms of a layer folded into the neighbouring products,
-head size 64 on the matrix-core attention with streamed pages).  Weights are made here with
+head size 64 on the matrix-core attention with streamed pages); E and F have head
+sizes of 100 and 40, which no 16-byte load divides.  Weights are made here with
 NumPy (not with the engine's random mode), rounded to bfloat16 so the float32
 and the bfloat16 engine and the plain implementation all read the same numbers.
 """
@@ -106,8 +107,48 @@ TINY_D = {
 }
 TINY_D_BLOCK = 16
 
+# E and F: head sizes that are not a multiple of 16.  E names no `head_dim`: it is
+# hidden_size / num_attention_heads = 100, the head size of a 3200-wide model with 32 heads.
+TINY_E = {
+    "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 2,
+    "hidden_size": 200,
+    "num_attention_heads": 2,
+    "num_key_value_heads": 1,
+    "intermediate_size": 176,
+    "vocab_size": 211,
+    "rope_theta": 10000.0,
+    "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": False,
+    "max_position_embeddings": 256,
+}
+TINY_E_BLOCK = 16
+
+TINY_F = {
+    "architectures": ["LlamaForCausalLM"],
+    "num_hidden_layers": 3,
+    "hidden_size": 160,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 2,
+    "head_dim": 40,
+    "intermediate_size": 96,
+    "vocab_size": 199,
+    "rope_theta": 50000.0,
+    "rope_scaling": {
+        "rope_type": "llama3",
+        "factor": 2.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 4.0,
+        "original_max_position_embeddings": 40,
+    },
+    "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": True,
+    "max_position_embeddings": 512,
+}
+TINY_F_BLOCK = 8
+
 CONFIGS = {"A": (TINY_A, TINY_A_BLOCK), "B": (TINY_B, TINY_B_BLOCK), "C": (TINY_C, TINY_C_BLOCK),
-           "D": (TINY_D, TINY_D_BLOCK)}
+           "D": (TINY_D, TINY_D_BLOCK), "E": (TINY_E, TINY_E_BLOCK), "F": (TINY_F, TINY_F_BLOCK)}
 
 
 def bf16_round(values: np.ndarray) -> np.ndarray:
