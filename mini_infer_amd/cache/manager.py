@@ -96,7 +96,7 @@ class CacheManager:
         self.groups: list[PageGroup] = []
         self._group_of_call: dict[int, int] = {}
         by_shape: dict[tuple, PageGroup] = {}
-        state_needs: dict[int, StateNeeds] = {}
+        state_needs: "dict[int, StateNeeds | dict[str, StateNeeds]]" = {}
         for call, need in enumerate(needs):
             if need is None:
                 continue
@@ -122,7 +122,13 @@ class CacheManager:
                 group.calls.append(call)
                 self._group_of_call[call] = group.index
             if need.state is not None:
-                state_needs[call] = need.state
+                if isinstance(need.state, StateNeeds):
+                    state_needs[call] = need.state
+                else:
+                    named = dict(need.state)
+                    if not named or not all(isinstance(k, str) and isinstance(v, StateNeeds) for k, v in named.items()):
+                        raise ValueError(f"call {call}: state needs are one StateNeeds or a non-empty mapping of names to them")
+                    state_needs[call] = named
         for group in self.groups:
             if allocate_storage:
                 calls, heads = len(group.calls), group.num_kv_heads
@@ -180,6 +186,12 @@ class CacheManager:
 
     # -- pages --------------------------------------------------------------
 
+    @property
+    def has_pages(self) -> bool:
+        """Whether any layer call keeps keys and values in pages (a model of state mixers
+        alone has none, and then no page count bounds what it can hold)."""
+        return bool(self.groups)
+
     def num_free_pages(self, group: int = 0) -> int:
         return self.groups[group].pool.num_free
 
@@ -190,7 +202,7 @@ class CacheManager:
         return [max(0, total - len(group.tables[request_id])) for group in self.groups]
 
     def pages_for_tokens(self, tokens: int) -> int:
-        return -(-tokens // self.page_size)
+        return -(-tokens // self.page_size) if self.groups else 0
 
     def reserve(self, extents: dict[Hashable, int]) -> None:
         """Pages for all `request -> new tokens` of a step, or `OutOfMemoryError` and no change."""
@@ -210,9 +222,11 @@ class CacheManager:
             for group, count in zip(self.groups, self.pages_needed(request_id, new_tokens)):
                 group.tables[request_id].extend(group.pool.allocate_many(count))
 
-    def cancel_reservation(self, extents: dict[Hashable, int]) -> None:
+    def cancel_reservation(self, extents: dict[Hashable, int], push: bool = True) -> None:
         """Undo a `reserve` whose step did not happen: pages past what each request's
-        committed length needs go back; lengths were never advanced."""
+        committed length needs go back; lengths were never advanced.  All of the host's books
+        are put right first; only then (`push`) are the positions sent to the device again,
+        which the step's first kernel may already have overwritten (`push_positions`)."""
         for request_id in extents:
             keep = self.pages_for_tokens(self._lengths[request_id])
             for group in self.groups:
@@ -221,8 +235,14 @@ class CacheManager:
                     page = table.pop()
                     if page != RELEASED:
                         group.pool.free(page)
-            # the step's first kernel may already have written the new position on the device
-            self.states.push(self._slots[request_id])
+        if push:
+            self.push_positions(extents)
+
+    def push_positions(self, request_ids) -> None:
+        """Send the host's position of each of these requests to its slot on the device."""
+        for request_id in request_ids:
+            if request_id in self._slots:
+                self.states.push_position(self._slots[request_id])
 
     def commit(self, extents: dict[Hashable, int]) -> None:
         """Advance lengths after a step and give back what windows have passed."""
@@ -260,7 +280,7 @@ class CacheManager:
                     group.pool.free(page)
         self._lengths[request_id] = length
         self.states.set_position(self._slots[request_id], length)
-        self.states.push(self._slots[request_id])
+        self.states.push_position(self._slots[request_id])
 
     # -- per-step index -------------------------------------------------------
 

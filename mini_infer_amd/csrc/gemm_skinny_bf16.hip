@@ -37,6 +37,11 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 // What the last step does with the products (each folds a neighbouring launch of a
 // decoder layer into this one):
 //   EPI_STORE  c = bf16(product).
+//   EPI_STORE_F32  c (float32) = float(bf16(product)): the output head's logits, which are
+//              wanted in float32 (no cast launch after the product).  Rounded to bfloat16 on the
+//              way like every product of this path, so that a position's logits are the same
+//              numbers whether its step had few rows (this kernel) or many (the vendor
+//              library's bfloat16 product, widened afterwards).
 //   EPI_GATED  W holds two stacked matrices [gate; up] of n rows each and the output is
 //              silu(gate . a) * (up . a): a block computes both halves of its features,
 //              so the [m, 2n] intermediate is never written.
@@ -55,7 +60,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 //              The norm's launch between two products is saved.
 // In every case the sums are rounded to bfloat16 before the activation or rotation,
 // exactly as when the product and the second step run as two kernels.
-enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2, EPI_ADDNORM = 3 };
+enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2, EPI_ADDNORM = 3, EPI_STORE_F32 = 4 };
 // Where the activations come from: a matrix in memory, or (PRO_ATTN, few rows) the
 // uncombined key ranges of attn_mfma: each wave first combines its own columns of the
 // attention output (what attn_reduce would have written) into LDS, so the combining launch
@@ -477,6 +482,13 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
       continue;
     }
     const int feature = n0 + nt * 16 + fq * 4;
+    if constexpr (EPI == EPI_STORE_F32) {
+      float* dst32 = reinterpret_cast<float*>(c) + (int64_t)token * ldc + feature;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (feature + r < n_end) dst32[r] = (float)(bf16_t)sum[r];
+      continue;
+    }
     bf16_t* dst = c + (int64_t)token * ldc + feature;
     if (feature + 3 < n_end && (ldc % 4 == 0)) {
       bf16x4_t packed;
@@ -555,8 +567,9 @@ static bool whole_lines(const void* w, int64_t ldw, int64_t rows, int k) {
          rows * ldw * 2 < ((int64_t)1 << 32);
 }
 
-extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* c,
-                                   int64_t ldc, int m, int n, int k, hipStream_t stream) {
+// `out_f32`: c is float32 [m, ldc] (EPI_STORE_F32).
+static int skinny_plain(const void* a, int64_t lda, const void* w, int64_t ldw, void* c, int64_t ldc, int m, int n,
+                        int k, bool out_f32, hipStream_t stream) {
   MI_REQUIRE(mi_gemm_skinny_bf16_supported(m, n, k, lda, ldw),
              "gemm_skinny_bf16: takes 1 <= m <= 16, k a multiple of 32, rows aligned to 16 bytes; "
              "got m=%d n=%d k=%d lda=%lld ldw=%lld", m, n, k, (long long)lda, (long long)ldw);
@@ -571,11 +584,14 @@ extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, in
   const int blocks = ceil_div(n, fpb);
   const int threads = 64 * SK_WAVES;
   const bool lines = whole_lines(w, ldw, n, k);
-#define SK_PLAIN(NT_, U_)                                                                                          \
+#define SK_PLAIN_AS(NT_, U_, EPI_)                                                                                 \
   if (lines)                                                                                                       \
-    gemm_skinny_bf16_kernel<NT_, U_, EPI_STORE, PRO_NONE, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); \
+    gemm_skinny_bf16_kernel<NT_, U_, EPI_, PRO_NONE, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); \
   else                                                                                                             \
-    gemm_skinny_bf16_kernel<NT_, U_, EPI_STORE><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded)
+    gemm_skinny_bf16_kernel<NT_, U_, EPI_><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded)
+#define SK_PLAIN(NT_, U_)                                \
+  if (out_f32) { SK_PLAIN_AS(NT_, U_, EPI_STORE_F32); } \
+  else { SK_PLAIN_AS(NT_, U_, EPI_STORE); }
   switch (ceil_div(fpb, 16)) {
     case 1: SK_PLAIN(1, 8); break;
     case 2: SK_PLAIN(2, 8); break;
@@ -583,8 +599,20 @@ extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, in
     default: SK_PLAIN(4, 2); break;
   }
 #undef SK_PLAIN
+#undef SK_PLAIN_AS
   MI_CHECK_LAUNCH("gemm_skinny_bf16");
   return MI_OK;
+}
+
+extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* c,
+                                   int64_t ldc, int m, int n, int k, hipStream_t stream) {
+  return skinny_plain(a, lda, w, ldw, c, ldc, m, n, k, false, stream);
+}
+
+// The same product, the same values, written as float32 [m, ldc].
+extern "C" int mi_gemm_skinny_f32out_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, float* c,
+                                          int64_t ldc, int m, int n, int k, hipStream_t stream) {
+  return skinny_plain(a, lda, w, ldw, c, ldc, m, n, k, true, stream);
 }
 
 // c[m, n] = attention output [m, heads*head_dim] . w^T, the attention output still lying in

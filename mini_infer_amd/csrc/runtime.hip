@@ -16,4 +16,4 @@ void mi_set_error(const char* fmt, ...) {
 extern "C" const char* mi_last_error() { return g_last_error; }
 
 // Bumped whenever an entry point's arguments change, so a stale library is refused.
-extern "C" int mi_abi_version() { return 17; }
+extern "C" int mi_abi_version() { return 18; }

@@ -113,7 +113,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, const uint32_t* __restrict__ seed_lo,
     const uint32_t* __restrict__ seed_hi, const uint32_t* __restrict__ draw_index,
-    int* __restrict__ out, const int* __restrict__ slots, int* __restrict__ slot_table) {
+    int* __restrict__ out, const int* __restrict__ slots, int* __restrict__ slot_table, int num_slots) {
   __shared__ ArgBest best_scratch[SAMPLE_WAVES];
   __shared__ uint32_t cnt[256];
   __shared__ unsigned long long mass[256];
@@ -125,13 +125,17 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const int tid = threadIdx.x;
   const T* x = logits + (int64_t)row * row_stride;
   // the row's settings: from the request's state slot, or from one array per setting
-  int* slot = slot_table ? slot_table + (int64_t)slots[row] * SLOT_WORDS : nullptr;
-  const float temp = slot ? __int_as_float(slot[SLOT_TEMPERATURE]) : temperature[row];
-  const int k = slot ? slot[SLOT_TOP_K] : top_k[row];
-  const float p = slot ? __int_as_float(slot[SLOT_TOP_P]) : top_p[row];
-  const uint32_t k0 = slot ? (uint32_t)slot[SLOT_SEED_LO] : seed_lo[row];
-  const uint32_t k1 = slot ? (uint32_t)slot[SLOT_SEED_HI] : seed_hi[row];
-  const uint32_t draw = slot ? (uint32_t)slot[SLOT_DRAW] : draw_index[row];
+  // (a slot id outside the table, such as the -1 of a padding row, belongs to no request: the
+  // row is sampled greedily and nothing is written back)
+  const bool by_slot = slot_table != nullptr;
+  const int slot_id = by_slot ? slots[row] : -1;
+  int* slot = (by_slot && slot_id >= 0 && slot_id < num_slots) ? slot_table + (int64_t)slot_id * SLOT_WORDS : nullptr;
+  const float temp = slot ? __int_as_float(slot[SLOT_TEMPERATURE]) : (by_slot ? 0.f : temperature[row]);
+  const int k = slot ? slot[SLOT_TOP_K] : (by_slot ? 0 : top_k[row]);
+  const float p = slot ? __int_as_float(slot[SLOT_TOP_P]) : (by_slot ? 1.f : top_p[row]);
+  const uint32_t k0 = slot ? (uint32_t)slot[SLOT_SEED_LO] : (by_slot ? 0u : seed_lo[row]);
+  const uint32_t k1 = slot ? (uint32_t)slot[SLOT_SEED_HI] : (by_slot ? 0u : seed_hi[row]);
+  const uint32_t draw = slot ? (uint32_t)slot[SLOT_DRAW] : (by_slot ? 0u : draw_index[row]);
   // every thread has read the draw index before thread 0 may advance it at the end
   __syncthreads();
 
@@ -304,11 +308,11 @@ extern "C" int mi_sample(int dtype, const void* logits, int64_t row_stride, int 
   if (dtype == MI_F32) {
     sample_kernel<float><<<num_rows, SAMPLE_THREADS, 0, stream>>>(
         (const float*)logits, row_stride, vocab, temperature, top_k, top_p, seed_lo, seed_hi,
-        draw_index, out, nullptr, nullptr);
+        draw_index, out, nullptr, nullptr, 0);
   } else {
     sample_kernel<bf16_t><<<num_rows, SAMPLE_THREADS, 0, stream>>>(
         (const bf16_t*)logits, row_stride, vocab, temperature, top_k, top_p, seed_lo, seed_hi,
-        draw_index, out, nullptr, nullptr);
+        draw_index, out, nullptr, nullptr, 0);
   }
   MI_CHECK_LAUNCH("sample");
   return MI_OK;
@@ -318,23 +322,24 @@ extern "C" int mi_sample(int dtype, const void* logits, int64_t row_stride, int 
 // `slots[row]` indexes `slot_table` [num_slots][8] (position, seed low, seed high, draw
 // index, temperature bits, top_k, top_p bits, unused).  The draw index of each sampled
 // slot is advanced by one, so the next call draws the request's next number without
-// the host sending anything.  A request appears in at most one row.
+// the host sending anything.  A request appears in at most one row.  A slot id outside
+// 0..num_slots-1 (the -1 of a padding row) is sampled greedily and nothing is written for it.
 extern "C" int mi_sample_slots(int dtype, const void* logits, int64_t row_stride, int num_rows, int vocab,
-                               const int* slots, int* slot_table, int* out, hipStream_t stream) {
+                               const int* slots, int* slot_table, int num_slots, int* out, hipStream_t stream) {
   MI_REQUIRE(num_rows >= 0 && vocab > 0, "sample_slots: bad sizes rows=%d vocab=%d", num_rows, vocab);
   MI_REQUIRE(row_stride >= vocab, "sample_slots: row stride %lld is shorter than the vocabulary %d",
              (long long)row_stride, vocab);
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "sample_slots: unknown dtype %d", dtype);
-  MI_REQUIRE(slots && slot_table, "sample_slots: needs the slot ids and the slot table");
+  MI_REQUIRE(slots && slot_table && num_slots > 0, "sample_slots: needs the slot ids and the slot table");
   if (num_rows == 0) return MI_OK;
   if (dtype == MI_F32) {
     sample_kernel<float><<<num_rows, SAMPLE_THREADS, 0, stream>>>(
         (const float*)logits, row_stride, vocab, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, out,
-        slots, slot_table);
+        slots, slot_table, num_slots);
   } else {
     sample_kernel<bf16_t><<<num_rows, SAMPLE_THREADS, 0, stream>>>(
         (const bf16_t*)logits, row_stride, vocab, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, out,
-        slots, slot_table);
+        slots, slot_table, num_slots);
   }
   MI_CHECK_LAUNCH("sample_slots");
   return MI_OK;

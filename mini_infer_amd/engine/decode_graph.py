@@ -73,6 +73,7 @@ class DecodeGraph:
             host_state_slots=[0] * batch,
         )
         self.graph: torch.cuda.CUDAGraph | None = None
+        self.real = 0  # rows of the staged step that belong to requests
         self.logits: torch.Tensor | None = None
         self._copied: torch.cuda.Event | None = None  # set once the staging buffer may be rewritten
 
@@ -145,15 +146,15 @@ class DecodeGraph:
                 gc.enable()
         self.graph = graph
 
-    def run(
+    def stage(
         self,
         token_ids: np.ndarray,
         index,
         from_rows: np.ndarray | None = None,
         device_tokens: torch.Tensor | None = None,
-    ) -> tuple[torch.Tensor, torch.Tensor]:
-        """Logits [real rows, vocab] of this step and the state-slot id of each row; both live
-        until the next replay."""
+    ) -> torch.Tensor:
+        """Send this step's integers to the device; returns the state-slot id of each real row
+        (on the device, valid in stream order from here on, until the next `stage`)."""
         self.fill(token_ids, index, from_rows)
         self.device.copy_(self.host, non_blocking=True)
         if from_rows is not None and device_tokens is not None:
@@ -161,11 +162,16 @@ class DecodeGraph:
         if self._copied is None:
             self._copied = torch.cuda.Event()
         self._copied.record()
+        self.real = len(index.request_ids)
+        return self.ctx.state_slots[: self.real]
+
+    def replay(self) -> tuple[torch.Tensor, torch.Tensor]:
+        """Run the staged step.  Logits [real rows, vocab] and the state-slot id of each row;
+        both live until the next replay."""
         if self.graph is None:
             self.capture()
         self.graph.replay()
-        real = len(index.request_ids)
-        return self.logits[:real], self.ctx.state_slots[:real]
+        return self.logits[: self.real], self.ctx.state_slots[: self.real]
 
 
 class DecodeGraphs:
@@ -187,13 +193,15 @@ class DecodeGraphs:
             and (device_tokens is None or device_tokens.numel() <= self.max_batch)
         )
 
-    def run(
+    def stage(
         self,
         token_ids: np.ndarray,
         index,
         from_rows: np.ndarray | None = None,
         device_tokens: torch.Tensor | None = None,
-    ) -> tuple[torch.Tensor, torch.Tensor]:
+    ) -> tuple[DecodeGraph, torch.Tensor]:
+        """The recorded step that takes this batch, its integers sent to the device, and the
+        state-slot ids of its rows; `graph.replay()` then runs it."""
         batch = bucket_of(len(index.request_ids))
         width = bucket_of(max([t.shape[1] for t in index.block_tables] + [1]), MIN_WIDTH)
         key = (batch, width)
@@ -201,4 +209,4 @@ class DecodeGraphs:
         if graph is None:
             graph = self.graphs[key] = DecodeGraph(self.runner, batch, width, self.max_batch)
         self.replays += 1
-        return graph.run(token_ids, index, from_rows, device_tokens)
+        return graph, graph.stage(token_ids, index, from_rows, device_tokens)

@@ -66,7 +66,9 @@ class ModelRunner:
         self.config = config
         self.dtype = model.dtype
         self.device = model.device
-        self.vocab_size = model.spec.vocab_size
+        self.vocab_size = model.vocab_size
+        # the most positions a request may reach, if the model says (admission goes by it)
+        self.max_model_len: int | None = getattr(model, "max_position_embeddings", None)
         self.block_size = block_size
         self.num_blocks = num_blocks
         self.cache = CacheManager(
@@ -157,7 +159,11 @@ class ModelRunner:
         self.cache.free_request(request_id)
 
     def num_free_blocks(self) -> int:
-        return min(self.cache.num_free_pages(g.index) for g in self.cache.groups) if self.cache.groups else 0
+        """Free pages of the fullest page group; all `num_blocks` for a model that keeps no
+        pages at all (state of fixed size only), which seats alone then bound."""
+        if not self.cache.groups:
+            return self.num_blocks
+        return min(self.cache.num_free_pages(g.index) for g in self.cache.groups)
 
     # -- the step ---------------------------------------------------------------
 
@@ -169,8 +175,10 @@ class ModelRunner:
         `step` again.  Requests seen for the first time are admitted.  Raises `OutOfMemoryError`
         before anything changes if the pages for this step are not there; any other failure
         (a kernel that refuses a size, an error on the device) gives the step's pages back
-        and forgets the requests it admitted, so lengths and free pages are what they were.
-        State of fixed size that a mixer had already updated in place is not restored.
+        and forgets the requests it admitted, so lengths and free pages are what they were;
+        where the model keeps state of fixed size, the rows of the step's requests are copied
+        aside before the forward pass and put back, so a mixer that had already updated them in
+        place leaves no trace either.
 
         `device_tokens` (int32, on the device) holds token ids the host has not read yet,
         e.g. what `sample_tokens` returned for the last step; an entry with `device_row`
@@ -228,6 +236,8 @@ class ModelRunner:
         # as it was before the step (the reference's rollback on a failed step:
         # scheduler/continuous_scheduler.py:418-445).  Keys and values the failed step may
         # have written lie past every request's length and are overwritten later.
+        states = self.cache.states
+        saved: tuple[torch.Tensor, list[torch.Tensor]] | None = None
         try:
             index = self.cache.build_step_index([(e.request_id, len(e.tokens)) for e in entries])
             rows = np.fromiter(
@@ -235,22 +245,38 @@ class ModelRunner:
                 dtype=np.int32,
             )
             token_ids = token_ids.astype(np.int32)
+            states.flush()  # slot-table rows of requests admitted since the last step
             if self.decode_graphs is not None and self.decode_graphs.takes(index, rows, device_tokens):
-                logits, self.last_row_slots = self.decode_graphs.run(token_ids, index, from_rows, device_tokens)
+                graph, step_slots = self.decode_graphs.stage(token_ids, index, from_rows, device_tokens)
+                if states.has_state:
+                    saved = (step_slots, states.snapshot(step_slots))
+                logits, self.last_row_slots = graph.replay()
             else:
                 row_slots = np.fromiter(
                     (index.state_slots[b] for b, e in enumerate(entries) for _ in e.want), dtype=np.int32
                 )
                 ctx, from_rows_device, self.last_row_slots = self._to_device(token_ids, rows, index, from_rows, row_slots)
+                if states.has_state:
+                    saved = (ctx.state_slots, states.snapshot(ctx.state_slots))
                 # tokens still on the device are taken from there, positions go into the state slots
                 if self.device.type == "cuda":
                     ops.begin_step(ctx.token_ids, from_rows_device, device_tokens, self.vocab_size,
-                                   self.cache.states.table, ctx.state_slots, ctx.seq_lens)
+                                   states.table, ctx.state_slots, ctx.seq_lens)
                 logits = self.model.forward(ctx, self._layer_caches)
         except BaseException:
-            self.cache.cancel_reservation(extents)
+            # the host's books first (nothing here touches the device), then what the device holds:
+            # if the device itself is what failed, that part may fail again, and the first
+            # error is the one to report
+            self.cache.cancel_reservation(extents, push=False)
             for request_id in admitted:
+                extents.pop(request_id, None)
                 self.cache.free_request(request_id)
+            try:
+                if saved is not None:
+                    states.restore(*saved)
+                self.cache.push_positions(extents)
+            except Exception:  # noqa: BLE001
+                pass
             raise
         self.cache.commit(extents)
         return logits

@@ -184,7 +184,11 @@ class ContinuousScheduler:
         self._thread: threading.Thread | None = None
         self._stop = threading.Event()
         self._crashed: BaseException | None = None
-        self.stats = {"steps": 0, "preemptions": 0, "tokens_run": 0, "rejected": 0}
+        # `rejected`: requests that could never fit the page pool; `rejected_too_long`: requests
+        # whose prompt and `max_tokens` together pass the positions the model was made for
+        self.stats = {"steps": 0, "preemptions": 0, "tokens_run": 0, "rejected": 0, "rejected_too_long": 0}
+        # the most positions a request may reach (the model's `max_position_embeddings`), or None
+        self.max_model_len: int | None = getattr(runner, "max_model_len", None)
         # A timeline of the steps in the Chrome trace-event format, as the reference records
         # it (scheduler/continuous_scheduler.py:223-229, :502-527): one duration event per
         # step that ran the model, written by `stop()` or `write_trace()`.
@@ -515,6 +519,14 @@ class ContinuousScheduler:
                 continue
             to_feed = len(running.feed)
             remaining_new = running.request.max_tokens - len(running.tokens_generated)
+            # positions the request would reach: everything it feeds (the last token it is
+            # given is never fed) must lie inside what the model's position encoding was made for
+            if self.max_model_len is not None and to_feed + remaining_new - 1 > self.max_model_len:
+                with self._lock:
+                    self._waiting.popleft()
+                self.stats["rejected_too_long"] += 1
+                self._finish(running, "cancelled")
+                continue
             need_now = self._pages_for(to_feed)
             if need_now > self.runner.num_blocks:
                 # can never fit, not even alone

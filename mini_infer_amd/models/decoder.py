@@ -55,6 +55,15 @@ class DecoderModel:
                 self.blocks[layer].enable_pending_output()
 
     @property
+    def vocab_size(self) -> int:
+        return self.spec.vocab_size
+
+    @property
+    def max_position_embeddings(self) -> int | None:
+        """The positions the model's encoding was made for (None: no bound is known)."""
+        return self.spec.max_position_embeddings
+
+    @property
     def graph_safe(self) -> bool:
         """Whether a decode step of this model can be recorded as a HIP graph."""
         parts = [self.embedding, self.final_norm, self.head, *self.blocks]

@@ -368,6 +368,38 @@ def gemm_skinny_bf16(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return c
 
 
+def linear_f32_out(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """`x @ weight.T` as float32, whatever the operands' dtype: what an output head returns.
+
+    Few bfloat16 rows: the weight-streaming kernel writes float32 itself (no cast launch); its
+    values are those of `linear(...).float()`, rounded to bfloat16 on the way, so that a row's
+    logits do not depend on how many rows its step had.  More rows: the vendor library's
+    product, cast.  float32 operands: `gemm_f32`."""
+    if x.dtype == torch.float32:
+        return gemm_f32(x, weight)
+    _need_cuda(x, weight)
+    if (
+        x.dtype == torch.bfloat16
+        and weight.dtype == torch.bfloat16
+        and x.dim() == 2
+        and weight.dim() == 2
+        and x.shape[1] == weight.shape[1]
+        and x.stride(1) == 1
+        and weight.stride(1) == 1
+        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), weight.stride(0))
+    ):
+        m, k = x.shape
+        n = weight.shape[0]
+        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+        library.check(
+            library.load().mi_gemm_skinny_f32out_bf16(
+                _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(out), out.stride(0), m, n, k, _stream()
+            )
+        )
+        return out
+    return torch.matmul(x, weight.t()).float()
+
+
 def skinny_gemm_takes(m: int, k: int, lda: int, ldw: int, max_rows: int = SKINNY_MAX_ROWS) -> bool:
     return 1 <= m <= max_rows and k >= 32 and k % 32 == 0 and lda % 8 == 0 and ldw % 8 == 0
 
@@ -483,6 +515,18 @@ def _scaled_rows_fit(x: "ScaledRows") -> bool:
     )
 
 
+def scaled_rows_product_takes(rows: int, weight: torch.Tensor | None, norm_width: int) -> bool:
+    """Whether a weight-streaming product with `weight` can take `rows` rows as `ScaledRows` of a
+    norm over `norm_width` features: what a part answers its norm with before a step
+    (`wants_scaled_rows`), so that no row is handed over in a form nobody has a kernel for."""
+    if weight is None or weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.stride(1) != 1:
+        return False
+    if weight.shape[1] != norm_width or not skinny_gemm_takes(rows, norm_width, norm_width, weight.stride(0), PENDING_PRODUCT_MAX_ROWS):
+        return False
+    pieces = library.load().mi_gemm_skinny_addnorm_pieces(norm_width)
+    return 0 < pieces <= SCALED_ROWS_MAX_PIECES
+
+
 def qkv_rope_write_takes(
     x: "torch.Tensor | ScaledRows", weight: torch.Tensor, head_dim: int, rotary_dim: int, interleaved: bool
 ) -> bool:
@@ -583,10 +627,13 @@ def linear_swiglu(x: "torch.Tensor | ScaledRows", gate_up_weight: torch.Tensor) 
 
     bfloat16 with at most 32 rows runs as ONE hand-written kernel (the product with the
     activation in its last step); otherwise the product and `silu_mul` run in turn.
-    Both ways round the two products to the element type before the activation, so a
-    token's result does not depend on which one ran.  `x` may be `ScaledRows`: the rows'
-    factors are then applied to the sums of the two products (the same kernel with one
-    more step), or to `x` first where that kernel does not take the shapes.
+    Both ways round the two products to the element type before the activation, so given
+    the same rows a token's result does not depend on which one ran.  `x` may be
+    `ScaledRows`: the rows' factors are then applied to the sums of the two products (the same
+    kernel with one more step), or to `x` first where that kernel does not take the shapes.
+    Rows that come as `ScaledRows` were rounded before their factor was applied
+    (`bf16(x * w)`, the factor then meets float32 sums), rows from a norm's own launch after
+    it (`bf16(x * r * w)`): which way a step went shows in the last bit of a bfloat16 value.
     """
     rows, width = gate_up_weight.shape
     if rows % 2:
@@ -1050,7 +1097,9 @@ def sample(
 def sample_slots(logits: torch.Tensor, slots: torch.Tensor, slot_table: torch.Tensor) -> torch.Tensor:
     """One token id per row of `logits` [B, V], each row's settings (temperature, top_k, top_p,
     seed, draw index) read from row `slots[b]` of `slot_table` [slots, 8] int32; the draw
-    index of every sampled slot is advanced by one on the device."""
+    index of every sampled slot is advanced by one on the device.  No slot may appear in two
+    rows; a row whose slot id lies outside the table (the -1 of a padding row) is sampled
+    greedily and writes nothing."""
     _need_cuda(logits, slots, slot_table)
     if logits.dim() != 2 or logits.stride(1) != 1:
         raise KernelShapeError("logits must be [rows, vocab] with unit inner stride")
@@ -1065,7 +1114,7 @@ def sample_slots(logits: torch.Tensor, slots: torch.Tensor, slot_table: torch.Te
     library.check(
         lib.mi_sample_slots(
             _dtype_code(logits), _ptr(logits), logits.stride(0), rows, vocab, _ptr(slots), _ptr(slot_table),
-            _ptr(out), _stream(),
+            slot_table.shape[0], _ptr(out), _stream(),
         )
     )
     return out

@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -33,6 +33,7 @@ _SIGNATURES: dict[str, list] = {
     "mi_silu_mul": [c_int, _P, _P, c_int, c_int, _P],
     "mi_gemm_f32": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_gemm_skinny_bf16": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
+    "mi_gemm_skinny_f32out_bf16": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_gemm_mid_partial_bf16": [_P, c_int64, _P, c_int64, _P, c_int, c_int, c_int, _P],
     "mi_gemm_mid_bf16_ranges": [c_int, c_int],
     "mi_gemm_mid_bf16_supported": [c_int, c_int, c_int, c_int64, c_int64],
@@ -65,7 +66,7 @@ _SIGNATURES: dict[str, list] = {
     "mi_attn_mfma_tokens_per_tile": [c_int, c_int, c_int],
     "mi_attn_mfma_supported": [c_int, c_int],
     "mi_sample": [c_int, _P, c_int64, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P],
-    "mi_sample_slots": [c_int, _P, c_int64, c_int, c_int, _P, _P, _P, _P],
+    "mi_sample_slots": [c_int, _P, c_int64, c_int, c_int, _P, _P, c_int, _P, _P],
 }
 
 

@@ -81,6 +81,17 @@ class GQAttention(Mixer):
         self.qkv.load_params(prefix, get)
         self.out.load_params(prefix, get)
 
+    def wants_scaled_rows(self, rows: int) -> bool:
+        """Only where projection, rotation and cache write will run as the one kernel that
+        applies the rows' factors: few bfloat16 rows, whole heads rotated in half pairing."""
+        layout = self.position.rotary_layout() if self.position is not None else None
+        return (
+            self.dtype == torch.bfloat16
+            and layout == (self.head_dim, False)
+            and self.head_dim % 32 == 0
+            and ops.scaled_rows_product_takes(rows, self.qkv.weight, self.hidden_size)
+        )
+
     def cache_needs(self, page_size: int) -> CacheNeeds:
         # values lie transposed inside a page where the matrix-core kernel will read them
         # (that kernel knows no score bias: such layers keep the plain layout and kernel)

@@ -97,8 +97,16 @@ class StateNeeds:
 
 @dataclasses.dataclass(frozen=True)
 class CacheNeeds:
+    """What one call of a mixer keeps per request: pages, state of fixed size, both or neither.
+
+    `state` is one `StateNeeds` (the mixer then finds one tensor under `LayerCache.state`) or a
+    mapping of names to `StateNeeds` (a dict of tensors under the same names): a mixer with a
+    short convolution tail in the compute dtype beside a float32 recurrent state asks for
+    `{"tail": StateNeeds((width, 3), dtype), "recurrent": StateNeeds((heads, d, d))}`.
+    """
+
     pages: PagedKVNeeds | None = None
-    state: StateNeeds | None = None
+    state: "StateNeeds | dict[str, StateNeeds] | None" = None
 
 
 @dataclasses.dataclass
@@ -111,7 +119,9 @@ class LayerCache:
     # if transposed; None for a mixer that asked for no value stream
     v_pages: torch.Tensor | None = None
     v_transposed: bool = False
-    state: torch.Tensor | None = None  # [max_requests, *state shape]
+    # [max_requests + 1, *state shape], one row per state slot (the last row is nobody's: slot -1);
+    # a dict of such tensors by name if the mixer asked for several
+    state: "torch.Tensor | dict[str, torch.Tensor] | None" = None
 
 
 # ----------------------------------------------------------------------------
@@ -179,6 +189,9 @@ class Norm(Part):
     takes_partial_sums = False
     takes_pending_products = False
     emit_scaled_rows = False
+    # the part that consumes this norm's output, set by the block together with
+    # `emit_scaled_rows`; the norm asks its `wants_scaled_rows(rows)` step by step
+    scaled_rows_consumer = None
 
     def forward(
         self,
@@ -218,6 +231,12 @@ class PositionEncoding(Part):
     def rotary(self, ctx: "StepContext") -> RotaryTables | None:
         return None
 
+    def rotary_layout(self) -> tuple[int, bool] | None:
+        """`(rotary_dim, interleaved)` of the tables `rotary` will return, if that is the same
+        for every step, else None.  Lets a mixer say before a step which of its kernels the
+        step will take; an encoding that does not answer costs nothing but that foresight."""
+        return None
+
     def score_slopes(self, num_heads: int) -> torch.Tensor | None:
         return None
 
@@ -231,12 +250,18 @@ class Mixer(Part):
     `takes_pending_products` and the mixer `can_defer_output`: `forward` may then return an
     `ops.PendingProduct` (its last product, not made yet) instead of a tensor.
     `takes_scaled_rows`: `x` may be an `ops.ScaledRows` (a norm's output but for the rows'
-    factors); the block then lets the norm before the mixer emit them."""
+    factors); the block then lets the norm before the mixer emit them, and the norm asks
+    `wants_scaled_rows(rows)` before it does so in a step of `rows` rows."""
 
     emit_partial_sums = False
     can_defer_output = False
     emit_pending_output = False
     takes_scaled_rows = False
+
+    def wants_scaled_rows(self, rows: int) -> bool:
+        """Whether, in a step of `rows` rows, the part has a kernel that applies the rows'
+        factors itself.  A part that answers False gets a finished tensor."""
+        return self.takes_scaled_rows
 
     def cache_needs(self, page_size: int) -> CacheNeeds:
         """What the cache manager must keep for one call of this mixer, given its page size
@@ -260,6 +285,10 @@ class FeedForward(Part):
     takes_scaled_rows = False
     can_defer_output = False
     emit_pending_output = False
+
+    def wants_scaled_rows(self, rows: int) -> bool:
+        """As `Mixer.wants_scaled_rows`."""
+        return self.takes_scaled_rows
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError

@@ -46,11 +46,13 @@ class PreNormBlock(Block):
         if mixer.can_defer_output and ffn_norm.takes_pending_products and feed_forward.takes_scaled_rows:
             mixer.emit_pending_output = True
             ffn_norm.emit_scaled_rows = True
+            ffn_norm.scaled_rows_consumer = feed_forward
         # The same between the block before this one and this block's mixer: its first norm may
         # be handed a product not made yet (if the model arranges that, `enable_pending_output`
         # of the block before), and leaves the rows' factors to the mixer's first product.
         if mixer_norm.takes_pending_products and mixer.takes_scaled_rows:
             mixer_norm.emit_scaled_rows = True
+            mixer_norm.scaled_rows_consumer = mixer
 
     @property
     def graph_safe(self) -> bool:  # type: ignore[override]

@@ -81,7 +81,7 @@ class OutputHead(Head):
 
     def forward(self, h: torch.Tensor, ctx: StepContext | None = None) -> torch.Tensor:
         """Logits [rows, vocab] in float32."""
-        return ops.linear(h, self.weight).float()
+        return ops.linear_f32_out(h, self.weight)
 
 
 @register_embedding("token_embedding")

@@ -38,6 +38,10 @@ class SwiGLU(FeedForward):
         self.gate_up.load_params(prefix, get)
         self.down.load_params(prefix, get)
 
+    def wants_scaled_rows(self, rows: int) -> bool:
+        """Where the gated product runs as the weight-streaming kernel that applies the rows' factors."""
+        return self.dtype == torch.bfloat16 and ops.scaled_rows_product_takes(rows, self.gate_up.weight, self.hidden_size)
+
     def forward(self, x: "torch.Tensor | ops.ScaledRows", ctx: StepContext) -> torch.Tensor:
         assert self.gate_up.weight is not None, "SwiGLU used before its weights were loaded"
         assert self.down.weight is not None

@@ -41,8 +41,15 @@ class RMSNorm(Norm):
         assert self.weight is not None, "RMSNorm used before its weight was loaded"
         if isinstance(delta, ops.PendingProduct):
             # few rows: the product, the add and the norm but for the rows' factors are one
-            # kernel, if the part that follows takes the rows that way
-            if self.emit_scaled_rows and rows is None and ops.linear_add_norm_takes(delta, residual, self.weight):
+            # kernel, if the part that follows has a kernel that applies the factors in this step
+            consumer = self.scaled_rows_consumer
+            if (
+                self.emit_scaled_rows
+                and rows is None
+                and consumer is not None
+                and consumer.wants_scaled_rows(residual.shape[0])
+                and ops.linear_add_norm_takes(delta, residual, self.weight)
+            ):
                 return ops.linear_add_norm(delta, residual, self.weight, self.eps)
             delta = delta.finish()
         return ops.add_rmsnorm(delta, residual, self.weight, self.eps, rows)

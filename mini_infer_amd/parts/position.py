@@ -93,6 +93,9 @@ class RotaryPosition(PositionEncoding):
             ctx.shared[key] = ops.rope_table(ctx.positions, self.inv_freq)
         return ctx.shared[key]
 
+    def rotary_layout(self) -> tuple[int, bool]:
+        return self.rotary_dim, self.interleaved
+
     def rotary(self, ctx: StepContext) -> RotaryTables:
         cos, sin = self.tables(ctx)
         return RotaryTables(cos, sin, self.rotary_dim, self.interleaved)

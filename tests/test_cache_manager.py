@@ -290,3 +290,58 @@ def test_slot_table_row_follows_the_request():
     m.add_request("b")
     assert m.state_slot("b") == slot and m.states.draws(slot) == 0 and m.states.position(slot) == 0
     assert m.states.table[slot].tolist()[:4] == [0, 0, 0, 0]
+
+
+def test_cancel_reservation_gives_back_exactly_what_reserve_took():
+    """A step that did not happen: a windowed group that has already released pages, a group
+    that keeps everything, a request that grows and one admitted for this very step.  After
+    `cancel_reservation` tables, pools and lengths are what they were, and `check()` holds."""
+    needs = [CacheNeeds(pages=PagedKVNeeds(2, 16)), CacheNeeds(pages=PagedKVNeeds(2, 16, window=6))]
+    m = CacheManager(needs, page_size=4, num_pages=12, max_requests=3, allocate_storage=False)
+    m.add_request("old")
+    m.reserve({"old": 17})
+    m.commit({"old": 17})
+    windowed = m.groups[1]
+    assert windowed.tables["old"][:3] == [-1, -1, -1]  # the window has passed three pages
+    tables_before = [list(g.tables["old"]) for g in m.groups]
+    free_before = [g.pool.num_free for g in m.groups]
+    m.add_request("new")
+    extents = {"old": 9, "new": 6}
+    m.reserve(extents)
+    assert [g.pool.num_free for g in m.groups] == [f - 4 for f in free_before]
+    m.cancel_reservation(extents)
+    m.check()
+    assert [list(g.tables["old"]) for g in m.groups] == tables_before
+    assert [g.tables["new"] for g in m.groups] == [[], []]
+    assert [g.pool.num_free for g in m.groups] == free_before
+    assert m.length("old") == 17 and m.length("new") == 0
+    m.free_request("new")
+    m.free_request("old")
+    m.check()
+    assert [g.pool.num_free for g in m.groups] == [12, 12]
+
+
+def test_several_named_state_tensors_per_call_are_zeroed_on_reuse():
+    needs = [CacheNeeds(state={"tail": StateNeeds((3,), torch.bfloat16), "recurrent": StateNeeds((2, 2))}), None,
+             CacheNeeds(pages=PagedKVNeeds(1, 16), state=StateNeeds((5,)))]
+    m = CacheManager(needs, page_size=4, num_pages=4, max_requests=2, dtype=torch.float32, device="cpu")
+    caches = m.layer_caches()
+    assert set(caches[0].state) == {"tail", "recurrent"} and caches[1].state is None
+    assert caches[0].state["tail"].dtype == torch.bfloat16 and caches[0].state["recurrent"].shape == (3, 2, 2)
+    assert caches[2].state.shape == (3, 5) and caches[2].k_pages is not None
+    slot = m.add_request("a")
+    caches[0].state["tail"][slot] = 7.0
+    caches[0].state["recurrent"][slot] = 3.0
+    caches[2].state[slot] = 1.0
+    saved = m.states.snapshot(torch.tensor([slot, -1]))
+    caches[0].state["recurrent"][slot] = 9.0
+    caches[0].state["recurrent"][-1] = 4.0
+    m.states.restore(torch.tensor([slot, -1]), saved)
+    assert caches[0].state["recurrent"][slot].flatten().tolist() == [3.0] * 4
+    assert caches[0].state["recurrent"][-1].flatten().tolist() == [0.0] * 4  # nobody's row, put back too
+    m.free_request("a")
+    assert m.add_request("b") == slot
+    for tensor in (caches[0].state["tail"], caches[0].state["recurrent"], caches[2].state):
+        assert float(tensor[slot].float().abs().sum()) == 0.0
+    with pytest.raises(ValueError, match="mapping of names"):
+        CacheManager([CacheNeeds(state={})], page_size=4, num_pages=1, max_requests=1, allocate_storage=False)

@@ -574,6 +574,24 @@ def test_float32_attention_over_thousands_of_keys_is_rounded_once():
     assert relative < 6e-8, f"relative error {relative:.2e}"
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 1000, 256), (8, 333, 96), (16, 4100, 512)])
+def test_product_with_float32_output_keeps_its_sums(m, n, k):
+    """The output head's product for few bfloat16 rows writes float32 itself: the values of
+    `gemm_skinny_bf16`, widened (what the many-row path gives too)."""
+    from mini_infer_amd import ops
+
+    a, w = _rand(m, k, dtype=torch.bfloat16, seed=1).to(DEV), _rand(n, k, dtype=torch.bfloat16, seed=2).to(DEV)
+    got = ops.linear_f32_out(a, w)
+    assert got.dtype == torch.float32 and got.shape == (m, n)
+    exact = a.double() @ w.double().T
+    assert float((got.double() - exact).abs().max()) < _tol(torch.bfloat16) * k ** 0.5
+    assert torch.equal(got, ops.gemm_skinny_bf16(a, w).float())
+    # float32 operands and many rows go their own ways to the same kind of result
+    assert ops.linear_f32_out(a.float(), w.float()).dtype == torch.float32
+    many = _rand(40, k, dtype=torch.bfloat16, seed=3).to(DEV)
+    assert ops.linear_f32_out(many, w).dtype == torch.float32
+
+
 def test_float32_product_is_rounded_once():
     """`gemm_f32` carries its sums in 64-bit: a sum over 14,336 terms is one float32 rounding
     away from exact (2.5e-8 on average), in the many-row and in the few-row kernel alike."""

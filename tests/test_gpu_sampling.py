@@ -143,6 +143,28 @@ def test_sampling_from_state_slots_is_sampling_with_the_same_settings_and_advanc
         sample_from_slots(logits, row_slots, slots.table)
 
 
+def test_a_row_whose_slot_id_lies_outside_the_table_is_sampled_greedily_and_writes_nothing():
+    """The padding rows of a recorded step carry slot -1: a caller that samples the whole bucket
+    must not read or write memory before the table.  Such rows (and ids past the table's end)
+    get the first largest logit, and the table is left as it was but for the real row's draw."""
+    from mini_infer_amd.cache import StateSlots
+    from mini_infer_amd.sampling import sample_from_slots
+
+    slots = StateSlots(3, {}, DEV)
+    real = slots.allocate("r")
+    slots.set_sampling(real, temperature=0.9, top_k=0, top_p=1.0, seed=5, draw=2)
+    before = slots.table.clone()
+    logits = torch.randn(3, 777, generator=torch.Generator().manual_seed(3)).to(DEV)
+    row_slots = torch.tensor([-1, real, 3], dtype=torch.int32, device=DEV)
+    got = sample_from_slots(logits, row_slots, slots.table).tolist()
+    assert got[0] == int(logits[0].argmax()) and got[2] == int(logits[2].argmax())
+    assert got[1] == _sample(logits[1:2], [_params(temperature=0.9)], [5], [2])[0]
+    after = slots.table.clone()
+    assert int(after[real, 3]) == 3
+    after[real, 3] = 2
+    assert torch.equal(after, before)
+
+
 def test_positions_and_draws_in_the_slot_table_follow_the_engine(tmp_path):
     """After steps of every kind (portions, recorded single-token steps, a request left out of a
     step) the device's slot table holds each request's length, as the host's copy does; a

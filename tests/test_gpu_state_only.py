@@ -1,0 +1,216 @@
+"""A model whose only cache is state of fixed size: no attention layer, no page group.
+
+The architecture is defined here and registered from outside the package: Llama's embedding,
+norms, feed-forwards and head around a toy mixer that keeps, per request, a decaying sum of its
+inputs (float32) and the last input row (the compute dtype), i.e. two state tensors of
+different dtypes under names of their own.  The mixer works on device tensors alone, so its
+single-token steps are recorded and replayed.  Compared with its plain recurrence, a loop
+over the tokens in float64 (the reference routes such models to a cache family of their own:
+models/base.py:57-60, cache/state_cache.py:130-333).
+"""
+
+import copy
+import dataclasses
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as pl
+import replay_util as ru
+import tiny
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = ["float32", "bfloat16"]
+DECAY = 0.75
+NAME = "StateOnlyTestLM"
+
+
+@pytest.fixture()
+def state_only(tmp_path):
+    from mini_infer_amd.config import ModelConfig
+    from mini_infer_amd.models.llama import llama_spec
+    from mini_infer_amd.models.spec import Architecture, LayerSpec
+    from mini_infer_amd.parts import CacheNeeds, Mixer, ParamSpec, StateNeeds
+    from mini_infer_amd.registry import ARCHITECTURES, MIXERS
+
+    cfg = dict(tiny.TINY_A, architectures=[NAME], max_position_embeddings=4096)
+    hidden = cfg["hidden_size"]
+
+    class SumAndTail(Mixer):
+        graph_safe = True
+
+        def param_specs(self, prefix):
+            return {prefix + "sum.weight": ParamSpec((hidden, hidden)), prefix + "tail.weight": ParamSpec((hidden, hidden))}
+
+        def load_params(self, prefix, get):
+            self.w_sum, self.w_tail = get(prefix + "sum.weight"), get(prefix + "tail.weight")
+
+        def cache_needs(self, page_size):
+            return CacheNeeds(state={"sum": StateNeeds((hidden,), torch.float32), "tail": StateNeeds((hidden,), self.dtype)})
+
+        def forward(self, x, ctx, cache, writes_cache=True):
+            request = ctx.token_request.long()  # [T]
+            slots = ctx.state_slots.long()  # [B]; -1 (nobody's row) for padding rows
+            at = torch.arange(x.shape[0], device=x.device)
+            starts = ctx.cu_seqlens_q.long()
+            distance = at[:, None] - at[None, :]
+            same = (request[:, None] == request[None, :]) & (distance >= 0)
+            weights = torch.where(same, DECAY ** distance.clamp(min=0).float(), 0.0)
+            carried = (DECAY ** (at - starts[request] + 1).float())[:, None] * cache.state["sum"][slots[request]]
+            sums = weights @ x.float() + carried  # the decaying sum after each token
+            first = (at == starts[request])[:, None]
+            before = torch.where(first, cache.state["tail"][slots[request]], torch.roll(x, 1, 0))  # the row before each token
+            cache.state["sum"][slots] = sums[starts[1:] - 1]
+            cache.state["tail"][slots] = x[starts[1:] - 1]
+            return (sums @ self.w_sum.float().T + 0.5 * (before.float() @ self.w_tail.float().T)).to(x.dtype)
+
+    MIXERS.register("sum_and_tail", lambda desc, dtype_, device, shared=None: SumAndTail(dtype_, device))
+
+    def spec_of(config):
+        spec = llama_spec(config)
+        layers = []
+        for layer in spec.layers:
+            block = copy.deepcopy(layer.block)
+            block["mixer"] = {"kind": "sum_and_tail"}
+            layers.append(LayerSpec(layer.prefix, block))
+        return dataclasses.replace(spec, layers=layers)
+
+    ARCHITECTURES.register(NAME, Architecture(NAME, ModelConfig.from_dict, spec_of))
+    weights = tiny.make_weights(cfg, 90)
+    rng = np.random.default_rng(7)
+    for layer in range(cfg["num_hidden_layers"]):
+        for n in "qkvo":
+            del weights[f"model.layers.{layer}.self_attn.{n}_proj.weight"]
+        for n in ("sum", "tail"):
+            weights[f"model.layers.{layer}.self_attn.{n}.weight"] = tiny.bf16_round(rng.standard_normal((hidden, hidden)) / 16)
+    folder = tiny.write_model_dir(tmp_path / "state_only", cfg, weights)
+
+    def plain(tokens, dtype):
+        """The recurrence token by token in float64 (the norm's output rounded where the engine stores it in bfloat16)."""
+        eps = cfg["rms_norm_eps"]
+        r = pl.embedding(weights["model.embed_tokens.weight"], np.array(tokens))
+        for layer in range(cfg["num_hidden_layers"]):
+            p = f"model.layers.{layer}."
+            h = pl.rms_norm(r, weights[p + "input_layernorm.weight"], eps)
+            if dtype == "bfloat16":
+                h = tiny.bf16_round(h).astype(np.float64)
+            w_sum = weights[p + "self_attn.sum.weight"].astype(np.float64)
+            w_tail = weights[p + "self_attn.tail.weight"].astype(np.float64)
+            state, before, mixed = np.zeros(hidden), np.zeros(hidden), []
+            for row in h:
+                state = DECAY * state + row
+                mixed.append(w_sum @ state + 0.5 * (w_tail @ before))
+                before = row
+            r = r + np.array(mixed)
+            r = r + pl.swiglu(pl.rms_norm(r, weights[p + "post_attention_layernorm.weight"], eps),
+                              *(weights[p + f"mlp.{n}_proj.weight"] for n in ("gate", "up", "down")))
+        return pl.rms_norm(r, weights["model.norm.weight"], eps) @ weights["model.embed_tokens.weight"].astype(np.float64).T
+
+    yield cfg, folder, plain
+    ARCHITECTURES.unregister(NAME)
+    MIXERS.unregister("sum_and_tail")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_logits_of_a_state_only_model_under_a_mixed_schedule_with_recorded_steps(state_only, dtype):
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+
+    cfg, folder, plain = state_only
+    runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=1, block_size=4, max_concurrent=4)
+    assert not runner.cache.has_pages and runner.num_free_blocks() == 1 and runner.decode_graphs is not None
+    caches = runner._layer_caches
+    assert all(set(c.state) == {"sum", "tail"} and c.k_pages is None for c in caches)
+    assert caches[0].state["sum"].dtype == torch.float32 and caches[1].state["tail"].dtype == runner.dtype
+    prompts, decoded = (13, 6, 9), 6
+    requests = {f"s{i}": tiny.random_tokens(cfg, n + decoded, seed=40 + i) for i, n in enumerate(prompts)}
+    expected = {rid: plain(t, dtype) for rid, t in requests.items()}
+    got = {rid: [] for rid in requests}
+    runner.step([StepEntry("s0", requests["s0"][:5], [])])
+    got["s0"].append(runner.step([StepEntry("s0", requests["s0"][5:13], list(range(8)))]).cpu().numpy())
+    both = runner.step([StepEntry("s1", requests["s1"][:6], [5]), StepEntry("s2", requests["s2"][:9], [8])]).cpu().numpy()
+    got["s1"].append(both[:1])
+    got["s2"].append(both[1:])
+    for k in range(decoded):
+        logits = runner.step([StepEntry(rid, [requests[rid][n + k]], [0]) for rid, n in zip(requests, prompts)]).cpu().numpy()
+        for row, rid in enumerate(requests):
+            got[rid].append(logits[row : row + 1])
+    assert runner.decode_graphs.replays == decoded and list(runner.decode_graphs.graphs) == [(4, 16)]
+    for rid, first in zip(requests, (5, 5, 8)):
+        ru.assert_close(np.concatenate(got[rid]), expected[rid][first:], dtype, f"state only {rid}")
+    for rid in requests:
+        runner.free_request(rid)
+    runner.cache.check()
+    assert runner.cache.states.num_free == 4
+
+
+def test_a_state_only_model_generates_through_llm_what_its_recurrence_gives(state_only):
+    """Five prompts for three seats, prompts cut into portions of 8 under a 20-token budget: admission
+    goes by seats alone (the model has no pages to wait for), single-token steps are replayed."""
+    from mini_infer_amd.engine.llm import LLM
+
+    cfg, folder, plain = state_only
+    lengths, new_tokens = (5, 17, 32, 3, 11), 7
+    prompts = [tiny.random_tokens(cfg, n, seed=70 + n) for n in lengths]
+    llm = LLM(folder, dtype="float32", num_blocks=1, block_size=4, max_concurrent=3, max_num_batched_tokens=20, chunk_size=8)
+    results = llm.generate(prompts, max_tokens=new_tokens)
+    for prompt, result in zip(prompts, results):
+        sequence = list(prompt)
+        for _ in range(new_tokens):
+            sequence.append(pl.greedy(plain(sequence, "float32")[-1]))
+        assert result.tokens == sequence[len(prompt):] and result.finish_reason == "length"
+    stats = llm.scheduler.stats
+    assert stats["tokens_run"] == sum(lengths) + len(lengths) * (new_tokens - 1)
+    assert stats["preemptions"] == 0 and stats["rejected"] == 0
+    assert llm.runner.decode_graphs.replays > 0
+    assert llm.runner.cache.states.num_free == 3
+
+
+@pytest.mark.parametrize("recorded", [False, True])
+def test_a_failing_step_leaves_every_state_row_and_the_slot_table_bit_equal(state_only, monkeypatch, recorded):
+    """The second layer's feed-forward raises after both layers' mixers have updated their state
+    rows in place and the step's first kernel has written the new positions: afterwards the state
+    tensors and the slot table on the device hold what they held, and the step can be run again."""
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.exceptions import KernelShapeError
+
+    cfg, folder, plain = state_only
+    runner = ModelRunner.from_pretrained(folder, dtype="float32", num_blocks=1, block_size=4, max_concurrent=3)
+    tokens = {"a": tiny.random_tokens(cfg, 12, seed=1), "b": tiny.random_tokens(cfg, 9, seed=2)}
+    runner.step([StepEntry("a", tokens["a"][:7], []), StepEntry("b", tokens["b"][:4], [])])
+    if recorded:  # a single-token step of these two requests has been recorded before the failing one
+        runner.step([StepEntry("a", tokens["a"][7:8], [0]), StepEntry("b", tokens["b"][4:5], [0])])
+    fed = {"a": 8, "b": 5} if recorded else {"a": 7, "b": 4}
+
+    live = [runner.cache.state_slot("a"), runner.cache.state_slot("b")]
+
+    def everything():
+        """Every state tensor whole (nobody's row and the free slot's included), and the slot-table
+        rows of the two live requests (a free slot's row is rewritten whenever it is handed out)."""
+        tensors = [t for cache in runner._layer_caches for t in cache.state.values()]
+        return [t.clone() for t in tensors] + [runner.cache.states.table[live].clone()]
+
+    before = everything()
+    feed_forward = runner.model.blocks[1].feed_forward
+    real_forward = feed_forward.forward
+
+    def refuse(x, ctx):
+        raise KernelShapeError("a kernel refuses this size")
+
+    monkeypatch.setattr(feed_forward, "forward", refuse)
+    portion = 1 if recorded else 3  # (a recorded step raises only while it is being recorded: force an eager one)
+    failing = [StepEntry("a", tokens["a"][fed["a"] : fed["a"] + portion], [portion - 1]),
+               StepEntry("b", tokens["b"][fed["b"] : fed["b"] + 2], [1]), StepEntry("new", [1, 2, 3], [2])]
+    with pytest.raises(KernelShapeError):
+        runner.step(failing)
+    torch.cuda.synchronize()
+    for was, now in zip(before, everything()):
+        assert torch.equal(was, now)
+    assert not runner.has_request("new") and runner.cache.length("a") == fed["a"] and runner.cache.states.num_free == 1
+    monkeypatch.setattr(feed_forward, "forward", real_forward)
+    again = runner.step([StepEntry("a", tokens["a"][fed["a"] :], [len(tokens["a"]) - fed["a"] - 1]),
+                         StepEntry("b", tokens["b"][fed["b"] :], [len(tokens["b"]) - fed["b"] - 1])]).cpu().numpy()
+    ru.assert_close(again[:1], plain(tokens["a"], "float32")[-1:], "float32", "after the failed step, a")
+    ru.assert_close(again[1:], plain(tokens["b"], "float32")[-1:], "float32", "after the failed step, b")
+    runner.cache.check()

@@ -325,17 +325,24 @@ class _FailingModel:
     dtype = torch.float32
     device = torch.device("cpu")
 
-    class spec:  # noqa: N801 - attribute-compatible with ModelSpec
-        vocab_size = VOCAB
+    vocab_size = VOCAB
 
-    def __init__(self):
+    def __init__(self, needs=None):
         self.fail_with = None
         self.positions_seen = []
+        self.needs = needs if needs is not None else [CacheNeeds(pages=PagedKVNeeds(1, 16))]
 
     def cache_needs(self, page_size):
-        return [CacheNeeds(pages=PagedKVNeeds(1, 16))]
+        return self.needs
 
     def forward(self, ctx, caches):
+        # a mixer with state of fixed size updates it in place as it goes: every request's row
+        # of every state tensor counts the tokens the request has brought so far
+        for cache in caches:
+            tensors = cache.state.values() if isinstance(cache.state, dict) else [cache.state] if cache.state is not None else []
+            for tensor in tensors:
+                for b, slot in enumerate(ctx.host_state_slots):
+                    tensor[slot] += ctx.host_cu_seqlens_q[b + 1] - ctx.host_cu_seqlens_q[b]
         if self.fail_with is not None:
             raise self.fail_with
         self.positions_seen.append(ctx.positions.tolist())
@@ -370,6 +377,127 @@ def test_a_step_that_raises_leaves_lengths_pages_and_admissions_as_they_were():
     runner.free_request("old")
     runner.free_request("new")
     assert runner.num_free_blocks() == 8
+
+
+def test_a_step_that_raises_leaves_state_of_fixed_size_bit_equal():
+    """A model with pages and with two state tensors of different shapes and dtypes per call:
+    the failing step has already added to the state rows of its requests (and would have
+    written their positions) when it raises; afterwards every state tensor and the slot table
+    hold what they held before, and a request the step had admitted is gone."""
+    from mini_infer_amd.engine.batch import StepEntry
+    from mini_infer_amd.engine.model_runner import ModelRunner
+    from mini_infer_amd.exceptions import KernelShapeError
+    from mini_infer_amd.parts.base import StateNeeds
+
+    needs = [
+        CacheNeeds(pages=PagedKVNeeds(1, 16), state=StateNeeds((3,))),
+        CacheNeeds(state={"tail": StateNeeds((2, 2), torch.bfloat16), "recurrent": StateNeeds((5,), torch.float64)}),
+    ]
+    model = _FailingModel(needs)
+    runner = ModelRunner(model, None, num_blocks=8, block_size=4, max_concurrent=3, cuda_graph=False)
+    caches = runner._layer_caches
+    assert caches[0].state.shape == (4, 3) and caches[0].state.dtype == torch.float32
+    assert set(caches[1].state) == {"tail", "recurrent"}
+    assert caches[1].state["tail"].shape == (4, 2, 2) and caches[1].state["tail"].dtype == torch.bfloat16
+    assert caches[1].state["recurrent"].shape == (4, 5) and caches[1].state["recurrent"].dtype == torch.float64
+    runner.step([StepEntry("old", [1, 2, 3, 4, 5, 6], [5]), StepEntry("other", [9, 9], [])])
+    slot = runner.cache.state_slot("old")
+    assert caches[0].state[slot].tolist() == [6.0] * 3 and caches[1].state["recurrent"][slot].tolist() == [6.0] * 5
+
+    def everything():
+        # (the host's copy of the slot table: without a GPU no kernel writes the device's)
+        tensors = [caches[0].state, caches[1].state["tail"], caches[1].state["recurrent"]]
+        return [t.clone() for t in tensors] + [torch.from_numpy(runner.cache.states.host[[slot]].copy())]
+
+    before = everything()
+    model.fail_with = KernelShapeError("a kernel refuses this size")
+    with pytest.raises(KernelShapeError):
+        runner.step([StepEntry("old", [7, 8, 9], [2]), StepEntry("new", [1, 2, 3, 4, 5], [4])])
+    for was, now in zip(before, everything()):
+        assert torch.equal(was, now)
+    runner.cache.check()
+    assert runner.cache.length("old") == 6 and not runner.has_request("new") and runner.cache.states.num_free == 1
+    model.fail_with = None
+    runner.step([StepEntry("old", [7, 8, 9], [2])])
+    assert caches[0].state[slot].tolist() == [9.0] * 3 and caches[1].state["tail"][slot].float().flatten().tolist() == [9.0] * 4
+
+
+def test_a_failing_device_copy_during_rollback_still_frees_everything_and_reports_the_first_error(monkeypatch):
+    """The rollback of a failed step puts the host's books right before it touches the device;
+    if sending the positions back fails too (the device is what broke), pages and admissions
+    are back all the same and the step's own error is the one raised."""
+    from mini_infer_amd.engine.batch import StepEntry
+    from mini_infer_amd.engine.model_runner import ModelRunner
+    from mini_infer_amd.exceptions import KernelShapeError
+
+    model = _FailingModel()
+    runner = ModelRunner(model, None, num_blocks=8, block_size=4, max_concurrent=3, cuda_graph=False)
+    runner.step([StepEntry("old", [1, 2, 3, 4, 5, 6], [5])])
+    model.fail_with = KernelShapeError("the step's own error")
+
+    def broken(slot):
+        raise RuntimeError("the device is gone")
+
+    monkeypatch.setattr(runner.cache.states, "push_position", broken)
+    with pytest.raises(KernelShapeError, match="the step's own error"):
+        runner.step([StepEntry("old", [7, 8, 9], [2]), StepEntry("new", [1, 2, 3, 4, 5], [4])])
+    runner.cache.check()
+    assert runner.num_free_blocks() == 6 and not runner.has_request("new") and runner.cache.states.num_free == 2
+
+
+class StateOnlyRunner(FakeRunner):
+    """A runner whose model keeps no pages at all: state of fixed size per request only."""
+
+    def __init__(self, max_concurrent=2):
+        from mini_infer_amd.parts.base import StateNeeds
+
+        self.num_blocks, self.block_size = 16, 4
+        self.cache = CacheManager([CacheNeeds(state=StateNeeds((4,)))], page_size=4, num_pages=16,
+                                  max_requests=max_concurrent, allocate_storage=False)
+        self.history, self.steps = {}, []
+
+    def num_free_blocks(self):
+        return self.num_blocks  # what `ModelRunner.num_free_blocks` answers without page groups
+
+
+def test_a_model_whose_only_cache_is_state_of_fixed_size_is_admitted_by_seats_and_finishes():
+    """No page group: admission goes by seats alone, prompts of any length are taken, the
+    requests run and finish, the third waits for a seat (it does not wait for pages for ever)."""
+    runner = StateOnlyRunner(max_concurrent=2)
+    assert not runner.cache.has_pages and runner.cache.pages_for_tokens(1000) == 0
+    sched = make(runner, max_concurrent=2, chunk_size=16, max_num_batched_tokens=32)
+    lengths = (70, 3, 200)  # far more tokens than 16 pages of 4 would hold
+    handles = [sched.submit(Request(prompt(n, n), SamplingParams(), max_tokens=5)) for n in lengths]
+    for _ in range(200):
+        if not sched.step() and not sched.has_work():
+            break
+    assert all(h.done() for h in handles)
+    for handle, n in zip(handles, lengths):
+        result = handle.wait()
+        assert result.finish_reason == "length" and result.tokens == expected_tokens(prompt(n, n), 5)
+    assert max(len(step) for step in runner.steps) == 2  # never more requests than seats
+    assert sched.stats["preemptions"] == 0 and sched.stats["rejected"] == 0
+    assert runner.cache.states.num_free == 2
+    assert sched.load_stats().kv_cache_usage == 0.0
+
+
+def test_a_request_past_the_models_positions_is_cancelled_and_counted():
+    """`max_position_embeddings` bounds admission: a request whose prompt and `max_tokens`
+    together would feed a position past it ends as cancelled, with a reason of its own in the
+    statistics; one that just fits runs."""
+    runner = FakeRunner()
+    runner.max_model_len = 20
+    sched = make(runner)
+    fits = sched.submit(Request(prompt(12, 1), SamplingParams(), max_tokens=9))  # feeds positions 0..19
+    too_long = sched.submit(Request(prompt(12, 2), SamplingParams(), max_tokens=10))
+    long_prompt = sched.submit(Request(prompt(30, 3), SamplingParams(), max_tokens=1))
+    while sched.step():
+        pass
+    assert fits.wait().finish_reason == "length" and len(fits.wait().tokens) == 9
+    assert too_long.wait().finish_reason == "cancelled" and too_long.wait().tokens == []
+    assert long_prompt.wait().finish_reason == "cancelled"
+    assert sched.stats["rejected_too_long"] == 2 and sched.stats["rejected"] == 0
+    assert runner.num_free_blocks() == runner.num_blocks
 
 
 def test_an_oversubscribed_load_is_admitted_in_waves_without_preemption():
