@@ -21,7 +21,7 @@ from mini_infer_amd.cache.manager import CacheManager
 from mini_infer_amd.config import DEFAULT_BLOCK_SIZE, DEFAULT_NUM_BLOCKS, EngineConfig, read_config_json
 from mini_infer_amd.engine.batch import StepEntry
 from mini_infer_amd.engine.decode_graph import DecodeGraphs
-from mini_infer_amd.models import DecoderModel, architecture_for
+from mini_infer_amd.models import architecture_for
 from mini_infer_amd.parts.base import StepContext
 from mini_infer_amd.weights import load_checkpoint
 from mini_infer_amd.weights.random_init import fill_random_on_device
@@ -54,7 +54,7 @@ def require_gpu(device: str | torch.device) -> torch.device:
 class ModelRunner:
     def __init__(
         self,
-        model: DecoderModel,
+        model: Any,
         config: Any,
         *,
         num_blocks: int = DEFAULT_NUM_BLOCKS,
@@ -83,7 +83,8 @@ class ModelRunner:
         self.engine_config: EngineConfig | None = None  # set when built from one
         # state-slot id of every row of the logits the last step returned (int32, on the device)
         self.last_row_slots: torch.Tensor | None = None
-        # decode steps are replayed as HIP graphs where every part of the model allows it
+        # small steps (single tokens, and few tokens with portions among them) are replayed as HIP
+        # graphs where every part of the model allows it
         self.decode_graphs = DecodeGraphs(self, max_batch=64) if cuda_graph and model.graph_safe else None
 
     # -- construction -----------------------------------------------------------
@@ -114,7 +115,7 @@ class ModelRunner:
         raw = read_config_json(model_name)
         arch = architecture_for(raw)
         config = arch.parse_config(raw)
-        model = DecoderModel(arch.build_spec(config), resolve_dtype(engine.dtype), dev)
+        model = arch.make_model(config, resolve_dtype(engine.dtype), dev)
         load_checkpoint(model, model_name)
         runner = cls(model, config, num_blocks=engine.num_blocks, block_size=engine.block_size,
                      max_concurrent=engine.max_concurrent, cuda_graph=engine.cuda_graph)
@@ -140,7 +141,7 @@ class ModelRunner:
         dev = require_gpu(device)
         arch = architecture_for(raw_config)
         config = arch.parse_config(raw_config)
-        model = DecoderModel(arch.build_spec(config), resolve_dtype(dtype), dev)
+        model = arch.make_model(config, resolve_dtype(dtype), dev)
         fill_random_on_device(model, seed, std=std, norm_jitter=norm_jitter)
         return cls(model, config, num_blocks=num_blocks, block_size=block_size, max_concurrent=max_concurrent,
                    cuda_graph=cuda_graph)
@@ -248,6 +249,13 @@ class ModelRunner:
             states.flush()  # slot-table rows of requests admitted since the last step
             if self.decode_graphs is not None and self.decode_graphs.takes(index, rows, device_tokens):
                 graph, step_slots = self.decode_graphs.stage(token_ids, index, from_rows, device_tokens)
+                if states.has_state:
+                    saved = (step_slots, states.snapshot(step_slots))
+                logits, self.last_row_slots = graph.replay()
+            elif self.decode_graphs is not None and self.decode_graphs.takes_mixed(index, [e.want for e in entries], device_tokens):
+                graph, step_slots = self.decode_graphs.stage_mixed(
+                    token_ids, index, [e.want for e in entries], from_rows, device_tokens
+                )
                 if states.has_state:
                     saved = (step_slots, states.snapshot(step_slots))
                 logits, self.last_row_slots = graph.replay()

@@ -893,7 +893,7 @@ def paged_attention(
     token_request: torch.Tensor,
     positions: torch.Tensor,
     cu_seqlens_q: torch.Tensor,
-    host_cu_seqlens_q: list[int],
+    host_cu_seqlens_q: list[int] | None,
     *,
     q_heads: int,
     kv_heads: int,
@@ -919,6 +919,10 @@ def paged_attention(
     (rows may be strided, so the merged projection's buffer can be passed as it is).
     Tokens of a request are consecutive and sit at consecutive positions;
     `cu_seqlens_q` (device) and `host_cu_seqlens_q` give the request boundaries.
+    `host_cu_seqlens_q=None`: the boundaries are known on the device only (a step that is
+    recorded once and replayed with other boundaries); the launch is then shaped by the number
+    of tokens and requests alone, with as many tiles as any division of the tokens among the
+    requests can need, and requests without tokens are allowed.
     bfloat16 caches with transposed values run on the matrix cores; everything else
     (float32, other head or page sizes) runs the plain kernel.
     """
@@ -945,9 +949,11 @@ def paged_attention(
     if block_table.dim() != 2:
         raise KernelShapeError("block_table must be [requests, max_blocks]")
     num_requests = block_table.shape[0]
-    if cu_seqlens_q.numel() != num_requests + 1 or len(host_cu_seqlens_q) != num_requests + 1:
+    if cu_seqlens_q.numel() != num_requests + 1 or (
+        host_cu_seqlens_q is not None and len(host_cu_seqlens_q) != num_requests + 1
+    ):
         raise KernelShapeError("cu_seqlens_q needs one more entry than there are requests")
-    if host_cu_seqlens_q[-1] != tokens:
+    if host_cu_seqlens_q is not None and host_cu_seqlens_q[-1] != tokens:
         raise KernelShapeError(f"cu_seqlens_q ends at {host_cu_seqlens_q[-1]}, but there are {tokens} tokens")
     num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
     out = torch.empty((tokens, q_heads * head_dim), dtype=q.dtype, device=q.device)
@@ -978,6 +984,25 @@ def paged_attention(
             torch.empty((rows * q_heads * splits, 2), dtype=torch.float32, device=q.device),
         )
 
+    if use_mfma and host_cu_seqlens_q is None:
+        # boundaries on the device only: one launch in the prefill shape, every wave finding its
+        # tile's request itself; a request of q tokens has ceil(q / tile) tiles, at most
+        # tokens // tile + requests of them in all, and the tiles past the real ones find nothing
+        shape = ATTN_SHAPE_PREFILL
+        tokens_per_tile = lib.mi_attn_mfma_tokens_per_tile(q_heads, kv_heads, shape)
+        num_tiles = tokens // tokens_per_tile + num_requests
+        head_blocks = -(-group // min(group, 128))
+        splits = min(16, attention_splits(num_tiles * kv_heads * head_blocks, max_seq_len, target=512, min_keys=128))
+        part_acc, part_ml = partials(splits)
+        library.check(
+            lib.mi_attn_mfma(
+                _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), block_table.shape[1],
+                _ptr(cu_seqlens_q), _ptr(positions), num_requests, tokens, num_tiles, _ptr(out), out.stride(0),
+                _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads, head_dim, page_size, num_pages, float(scale),
+                int(window or 0), splits, shape, 0, 0, 1, _stream(),
+            )
+        )
+        return out
     if use_mfma:
         q_lens = [host_cu_seqlens_q[b + 1] - host_cu_seqlens_q[b] for b in range(num_requests)]
         max_blocks = block_table.shape[1]

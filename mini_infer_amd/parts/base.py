@@ -155,10 +155,15 @@ class StepContext:
     block_tables: list[torch.Tensor]
     max_q_len: int
     max_seq_len: int
-    # host copies, for parts that loop over requests on the host
-    host_cu_seqlens_q: list[int] = dataclasses.field(default_factory=list)
-    host_seq_lens: list[int] = dataclasses.field(default_factory=list)
-    host_state_slots: list[int] = dataclasses.field(default_factory=list)
+    # Host copies, for parts that loop over requests on the host or shape a launch by the
+    # requests' lengths.  None in a step that is being recorded to be replayed with other
+    # boundaries (only models whose parts are all `graph_safe` are recorded): `num_tokens`,
+    # `num_requests`, `max_q_len` and `max_seq_len` are then upper bounds that hold for every
+    # replay, some requests may bring no token at all, and everything else about the step is
+    # to be read from the device tensors.
+    host_cu_seqlens_q: list[int] | None = dataclasses.field(default_factory=list)
+    host_seq_lens: list[int] | None = dataclasses.field(default_factory=list)
+    host_state_slots: list[int] | None = dataclasses.field(default_factory=list)
     # per-step results shared between layers (rotation tables and the like), by key
     shared: dict = dataclasses.field(default_factory=dict)
 

@@ -60,12 +60,11 @@ def write_random_model(
     `raw_config` holds the architecture's own config.json keys; the model class is
     chosen by `architectures[0]` as everywhere else.
     """
-    from mini_infer_amd.models import DecoderModel, architecture_for
+    from mini_infer_amd.models import architecture_for
 
     store = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
     arch = architecture_for(raw_config)
-    spec = arch.build_spec(arch.parse_config(raw_config))
-    model = DecoderModel(spec, store, "cpu")
+    model = arch.make_model(arch.parse_config(raw_config), store, "cpu")
     tensors = random_tensors(model.param_specs(), seed, std=std, norm_jitter=norm_jitter, dtype=store)
     out_dir = Path(out_dir)
     out_dir.mkdir(parents=True, exist_ok=True)

@@ -117,6 +117,26 @@ def test_llama_spec_is_data():
     assert not spec.tie_word_embeddings
 
 
+def test_a_spec_needs_only_what_its_embedding_and_head_need():
+    """The checkpoint names of the plain table and the plain head are a short form: a spec that
+    describes its own embedding and head parts gives neither, one that gives nothing is told so."""
+    import dataclasses
+
+    from mini_infer_amd.models.spec import ModelSpec
+
+    arch = architecture_for(tiny.TINY_A)
+    llama = arch.build_spec(arch.parse_config(tiny.TINY_A))
+    own = ModelSpec(vocab_size=7, hidden_size=8, layers=[], order=[], final_norm=llama.final_norm, final_norm_prefix="n.",
+                    embedding={"kind": "my_embedding"}, head={"kind": "my_head"})
+    assert own.embedding_description() == {"kind": "my_embedding"} and own.head_description() == {"kind": "my_head"}
+    bare = dataclasses.replace(own, embedding=None, head=None)
+    with pytest.raises(ValueError, match="embedding_name"):
+        bare.embedding_description()
+    with pytest.raises(ValueError, match="head_name"):
+        bare.head_description()
+    assert dataclasses.replace(bare, tie_word_embeddings=True).head_description()["tied"]
+
+
 def test_engine_config_checks():
     assert EngineConfig().block_size == 16 and EngineConfig().num_blocks == 1024
     with pytest.raises(ValueError):

@@ -573,6 +573,66 @@ def test_graph_replays_equal_eager_steps_with_eager_work_between(tmp_path, dtype
         runner.cache.check()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "D", "E"])
+def test_small_steps_with_portions_are_recorded_by_bucket_and_replayed_with_other_divisions(tmp_path, name, dtype):
+    """Steps of a few tokens that are not single tokens only (a prompt's portion beside decoded
+    tokens, two short prompts, a portion alone) are recorded once per (tokens, requests) bucket and
+    replayed with whatever division of the tokens among the requests the next step has: the
+    boundaries live on the device only.  Every wanted row is compared with the plain model; the
+    same bucket is replayed with four different divisions, a recorded single-token step and eager
+    work of another kind run in between, and a request that ends frees pages that a later
+    request's portion then uses."""
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+
+    cfg, block, weights, folder = _folder(tmp_path, name, 81)
+    lengths = {"a": 40, "b": 23, "c": 31, "d": 12, "e": 50}
+    requests = {rid: tiny.random_tokens(cfg, n, seed=30 + n) for rid, n in lengths.items()}
+    expected = {rid: ru.oracle(cfg, weights, t) for rid, t in requests.items()}
+    runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=-(-100 // block) + 4, block_size=block, max_concurrent=4)
+    fed = {rid: 0 for rid in requests}
+
+    def step(*parts):
+        """parts: (request, tokens to feed, whether the last of them wants logits)"""
+        entries, wanted = [], []
+        for rid, count, wants in parts:
+            tokens = requests[rid][fed[rid] : fed[rid] + count]
+            assert len(tokens) == count
+            entries.append(StepEntry(rid, tokens, [count - 1] if wants else []))
+            fed[rid] += count
+            if wants:
+                wanted.append((rid, fed[rid] - 1))
+        logits = runner.step(entries).cpu().numpy()
+        assert logits.shape[0] == len(wanted)
+        for row, (rid, position) in enumerate(wanted):
+            ru.assert_close(logits[row : row + 1], expected[rid][position : position + 1], dtype, f"{name} {rid}[{position}]")
+
+    graphs = runner.decode_graphs
+    step(("a", 10, False), ("b", 7, True))  # 17 tokens, 2 requests: bucket (32, 4)
+    assert list(graphs.graphs) == [(32, 4, 16)] and graphs.mixed_replays == 1
+    step(("a", 1, True), ("b", 1, True), ("c", 9, True))  # 11 tokens, 3 requests: bucket (16, 4)
+    step(("a", 1, True), ("c", 11, False), ("d", 3, True))  # the same bucket, another division
+    step(("a", 1, True), ("b", 1, True), ("c", 1, True), ("d", 1, True))  # single tokens: their own recorded step
+    torch.randn(64, 64, device=DEV) @ torch.randn(64, 64, device=DEV)  # eager work of another kind
+    step(("b", 1, True), ("c", 5, True), ("d", 1, False))  # (16, 4) again: one request wants nothing
+    step(("d", 7, True))  # a portion alone, 7 tokens, 1 request: bucket (16, 2)
+    assert fed["d"] == lengths["d"]
+    runner.free_request("d")
+    step(("e", 16, False), ("a", 1, True))  # 17 tokens: (32, 4) again, the new request on d's pages
+    step(("e", 14, True), ("a", 2, True), ("b", 2, True), ("c", 2, True))  # 20 tokens, 4 requests, none to spare: (32, 8)
+    step(("e", 16, True))  # exactly the bucket's tokens: (16, 1)
+    assert set(graphs.graphs) == {(32, 4, 16), (16, 4, 16), (4, 16), (16, 2, 16), (32, 8, 16), (16, 1, 16)}
+    assert graphs.mixed_replays == 8 and graphs.replays == 1
+    # a step of more tokens than the largest bucket, or one that wants two rows of a request, is launched kernel by kernel
+    before = graphs.mixed_replays
+    runner.step([StepEntry("a", requests["a"][fed["a"] : fed["a"] + 3], [0, 2])])
+    assert graphs.mixed_replays == before
+    for rid in ("a", "b", "c", "e"):
+        runner.free_request(rid)
+    runner.cache.check()
+    assert runner.num_free_blocks() == runner.num_blocks
+
+
 @pytest.mark.parametrize("cuda_graph", [True, False])
 def test_tokens_left_on_the_device_give_the_steps_of_tokens_from_the_host(tmp_path, cuda_graph):
     """A decode step whose tokens are still on the device (`device_row`) equals the step fed
@@ -991,7 +1051,7 @@ def test_toy_state_mixer_on_device_tensors_alone_is_recorded_and_replayed(tmp_pa
             logits = runner.step(entries).cpu().numpy()
             for row, rid in enumerate(requests):
                 got[rid].append(logits[row : row + 1])
-        assert runner.decode_graphs.replays == decoded and list(runner.decode_graphs.graphs) == [(4, 16)]
+        assert runner.decode_graphs.replays == decoded and [key for key in runner.decode_graphs.graphs if len(key) == 2] == [(4, 16)]
         ru.assert_close(np.concatenate(got["d0"]), expected["d0"][5:], dtype, "toy on device d0")
         ru.assert_close(np.concatenate(got["d1"]), expected["d1"][5:], dtype, "toy on device d1")
         ru.assert_close(np.concatenate(got["d2"]), expected["d2"][8:], dtype, "toy on device d2")
@@ -1646,7 +1706,7 @@ def test_a_whole_architecture_with_config_keys_and_tensor_names_of_its_own(tmp_p
         return ModelSpec(
             vocab_size=cfg.n_vocab, hidden_size=cfg.d_model, embedding_name="wte.weight", layers=layers,
             order=[LayerCall(i) for _ in range(cfg.loops) for i in range(cfg.n_layer)],
-            final_norm=norm, final_norm_prefix="ln_f.", head_name="unused.weight", tie_word_embeddings=True,
+            final_norm=norm, final_norm_prefix="ln_f.", tie_word_embeddings=True,
         )
 
     raw = {"architectures": ["TinyToyLM"], "n_layer": 2, "d_model": 96, "n_head": 6, "n_kv_head": 3, "d_head": 16,
@@ -1701,6 +1761,90 @@ def test_a_whole_architecture_with_config_keys_and_tensor_names_of_its_own(tmp_p
         assert runner.decode_graphs.replays == 6
     finally:
         ARCHITECTURES.unregister("TinyToyLM")
+
+
+def test_an_architecture_of_another_overall_shape_brings_a_model_object_of_its_own(tmp_path):
+    """Not embedding -> blocks -> one norm -> one head: a model with two heads whose logits are
+    added, built by the architecture's own `build_model` from the package's parts.  Loader,
+    random-weights mode, runner, scheduler and `LLM` work from the model contract alone."""
+    import dataclasses
+
+    from safetensors.torch import load_file
+
+    from mini_infer_amd.engine.llm import LLM
+    from mini_infer_amd.models.spec import Architecture
+    from mini_infer_amd.parts.embedding import OutputHead, TokenEmbedding
+    from mini_infer_amd.parts.norm import RMSNorm
+    from mini_infer_amd.registry import ARCHITECTURES
+    from mini_infer_amd.weights import write_random_model
+
+    @dataclasses.dataclass(frozen=True)
+    class TwoHeadConfig:
+        width: int
+        vocab: int
+        eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(int(raw["width"]), int(raw["vocab"]), float(raw["eps"]))
+
+    class TwoHeadModel:
+        graph_safe = True
+        max_position_embeddings = None
+
+        def __init__(self, config, dtype, device):
+            self.dtype, self.device, self.vocab_size = dtype, torch.device(device), config.vocab
+            self.embedding = TokenEmbedding(config.vocab, config.width, "table", dtype, device)
+            self.norm = RMSNorm(config.width, config.eps, dtype, device)
+            self.heads = [OutputHead(config.width, config.vocab, f"head_{n}", dtype, device) for n in "ab"]
+
+        def param_specs(self):
+            specs = {**self.embedding.param_specs(""), **self.norm.param_specs("norm.")}
+            for head in self.heads:
+                specs.update(head.param_specs(""))
+            return specs
+
+        def optional_names(self):
+            return set()
+
+        def load_params(self, get):
+            self.embedding.load_params("", get)
+            self.norm.load_params("norm.", get)
+            for head in self.heads:
+                head.load_params("", get)
+
+        def cache_needs(self, page_size):
+            return []
+
+        def forward(self, ctx, caches):
+            h = self.norm.forward(None, self.embedding.forward(ctx), rows=ctx.logit_rows)
+            return self.heads[0].forward(h, ctx) + self.heads[1].forward(h, ctx)
+
+    raw = {"architectures": ["TwoHeadTestLM"], "width": 64, "vocab": 97, "eps": 1e-5}
+    ARCHITECTURES.register("TwoHeadTestLM", Architecture("TwoHeadTestLM", TwoHeadConfig.from_dict, build_model=TwoHeadModel))
+    try:
+        with pytest.raises(ValueError, match="one of the two"):
+            Architecture("Neither", TwoHeadConfig.from_dict)
+        folder = write_random_model(raw, seed=3, out_dir=tmp_path / "two_heads", std=0.5, norm_jitter=0.2, dtype="float32")
+        weights = {k: v.double().numpy() for k, v in load_file(str(folder / "model.safetensors")).items()}
+        assert sorted(weights) == ["head_a", "head_b", "norm.weight", "table"]
+
+        def plain_next(token):
+            h = pl.rms_norm(weights["table"][[token]], weights["norm.weight"], raw["eps"])
+            return int(np.argmax(h @ (weights["head_a"] + weights["head_b"]).T))
+
+        llm = LLM(folder, dtype="float32", num_blocks=1, block_size=4, max_concurrent=2)
+        assert not llm.runner.cache.has_pages and not llm.runner.cache.states.has_state
+        prompts = [[5, 9, 33], [96], [1, 2]]
+        for prompt, result in zip(prompts, llm.generate(prompts, max_tokens=5)):
+            expected, last = [], prompt[-1]
+            for _ in range(5):
+                last = plain_next(last)
+                expected.append(last)
+            assert result.tokens == expected and result.finish_reason == "length"
+        assert llm.runner.decode_graphs.replays > 0
+    finally:
+        ARCHITECTURES.unregister("TwoHeadTestLM")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

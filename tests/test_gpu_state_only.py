@@ -136,7 +136,7 @@ def test_logits_of_a_state_only_model_under_a_mixed_schedule_with_recorded_steps
         logits = runner.step([StepEntry(rid, [requests[rid][n + k]], [0]) for rid, n in zip(requests, prompts)]).cpu().numpy()
         for row, rid in enumerate(requests):
             got[rid].append(logits[row : row + 1])
-    assert runner.decode_graphs.replays == decoded and list(runner.decode_graphs.graphs) == [(4, 16)]
+    assert runner.decode_graphs.replays == decoded and [key for key in runner.decode_graphs.graphs if len(key) == 2] == [(4, 16)]
     for rid, first in zip(requests, (5, 5, 8)):
         ru.assert_close(np.concatenate(got[rid]), expected[rid][first:], dtype, f"state only {rid}")
     for rid in requests:
@@ -199,9 +199,11 @@ def test_a_failing_step_leaves_every_state_row_and_the_slot_table_bit_equal(stat
         raise KernelShapeError("a kernel refuses this size")
 
     monkeypatch.setattr(feed_forward, "forward", refuse)
-    portion = 1 if recorded else 3  # (a recorded step raises only while it is being recorded: force an eager one)
+    # (a recorded step runs none of the model's Python when it is replayed: two wanted rows of one
+    # request make this step one that is launched kernel by kernel)
+    portion = 1 if recorded else 3
     failing = [StepEntry("a", tokens["a"][fed["a"] : fed["a"] + portion], [portion - 1]),
-               StepEntry("b", tokens["b"][fed["b"] : fed["b"] + 2], [1]), StepEntry("new", [1, 2, 3], [2])]
+               StepEntry("b", tokens["b"][fed["b"] : fed["b"] + 2], [0, 1]), StepEntry("new", [1, 2, 3], [2])]
     with pytest.raises(KernelShapeError):
         runner.step(failing)
     torch.cuda.synchronize()
