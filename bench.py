@@ -69,7 +69,11 @@ LLAMA_32_3B = {
 LLAMA_31_70B = dict(
     LLAMA_31_8B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64, intermediate_size=28672
 )
-SIZES = {"8b": ("Llama-3.1-8B", LLAMA_31_8B), "3b": ("Llama-3.2-3B", LLAMA_32_3B), "70b": ("Llama-3.1-70B", LLAMA_31_70B)}
+LLAMA_32_1B = dict(
+    LLAMA_32_3B, num_hidden_layers=16, hidden_size=2048, num_attention_heads=32, head_dim=64, intermediate_size=8192
+)
+SIZES = {"8b": ("Llama-3.1-8B", LLAMA_31_8B), "3b": ("Llama-3.2-3B", LLAMA_32_3B), "70b": ("Llama-3.1-70B", LLAMA_31_70B),
+         "1b": ("Llama-3.2-1B", LLAMA_32_1B)}
 PROMPT_LEN = 2048
 BLOCK_SIZE = 16
 
@@ -99,7 +103,7 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
     return linear + attention + head
 
 
-def measure_serving(dtype: str) -> dict:
+def measure_serving(dtype: str, mixed_graphs: bool = True) -> dict:
     """Continuous batching through the scheduler: 32 concurrent requests, prompt lengths
     uniform in [128, 4096] of uniform-random ids, 256 greedy tokens each, a 2,048-token
     budget per step, at Llama-3.2-3B layer sizes with random weights."""
@@ -115,6 +119,7 @@ def measure_serving(dtype: str) -> dict:
     )
     import os
 
+    runner.decode_graphs.mixed = mixed_graphs
     scheduler = ContinuousScheduler(
         runner, max_concurrent=requests_n, chunk_size=2048, max_num_batched_tokens=2048, trace_out=os.devnull
     )
@@ -162,7 +167,7 @@ def measure_serving(dtype: str) -> dict:
     }
 
 
-def measure_reference_workload(dtype: str) -> dict:
+def measure_reference_workload(dtype: str, mixed_graphs: bool = True, sizes: str = "8b") -> dict:
     """The workload the reference publishes numbers for (docs/benchmarks/
     2026-11-05-model-metrics.md:19-41; scripts/bench/modal_model_metrics.py:58-62, :239-252):
     1,024-token prompts, 128 greedy tokens, 2,048 pages of 16, 16 seats.  Time to the first
@@ -170,7 +175,8 @@ def measure_reference_workload(dtype: str) -> dict:
     start together.  Here: Llama-3.1-8B layer sizes with random weights, prompts of random
     ids (no request stops early), and up to 4,096 tokens a step, which is what a step of the
     reference can carry in this setting (16 requests x its chunk of 256 each; it has no
-    budget over all requests)."""
+    budget over all requests).  Then short prompts, where the host's share of a step shows:
+    16 requests of 16 tokens each that start together, 64 tokens each."""
     import statistics
 
     import numpy as np
@@ -179,15 +185,17 @@ def measure_reference_workload(dtype: str) -> dict:
     from mini_infer_amd import ContinuousScheduler, ModelRunner, Request, SamplingParams
 
     prompt_len, new_tokens, concurrency = 1024, 128, 16
+    model_name, model = SIZES[sizes]
     runner = ModelRunner.from_random(
-        LLAMA_31_8B, seed=0, dtype=dtype, num_blocks=2048, block_size=BLOCK_SIZE, max_concurrent=concurrency
+        model, seed=0, dtype=dtype, num_blocks=2048, block_size=BLOCK_SIZE, max_concurrent=concurrency
     )
+    runner.decode_graphs.mixed = mixed_graphs
     scheduler = ContinuousScheduler(runner, max_concurrent=concurrency, chunk_size=4096, max_num_batched_tokens=4096)
     rng = np.random.default_rng(5)
 
-    def request() -> Request:
-        ids = rng.integers(0, LLAMA_31_8B["vocab_size"], size=prompt_len).tolist()
-        return Request(ids, SamplingParams(ignore_eos=True), new_tokens)
+    def request(length: int = prompt_len, tokens: int = new_tokens) -> Request:
+        ids = rng.integers(0, model["vocab_size"], size=length).tolist()
+        return Request(ids, SamplingParams(ignore_eos=True), tokens)
 
     def timed(requests: list) -> list[dict]:
         """Drive the engine from here; per request: submit, first token and last token times, tokens."""
@@ -213,7 +221,39 @@ def measure_reference_workload(dtype: str) -> dict:
     batch = timed([request() for _ in range(concurrency)])
     torch.cuda.synchronize()
     seconds = max(m["last"] for m in batch) - min(m["submit"] for m in batch)
+    # short prompts: requests arrive one step apart (1, 2, 3, ... live), so that steps of a few
+    # tokens with a prompt among single tokens are what runs, then all 16 at once
+    def staggered() -> list[dict]:
+        handles, marks = [], []
+        while len(handles) < concurrency or not all(h.done() for h in handles):
+            if len(handles) < concurrency:
+                marks.append({"submit": time.perf_counter(), "first": None, "last": None, "tokens": 0})
+                handles.append(scheduler.submit(request(16, 64)))
+            scheduler.step()
+            now = time.perf_counter()
+            for h, mark in zip(handles, marks):
+                tokens = sum(1 for step in h.steps() if step.finish_reason is None)
+                if tokens > mark["tokens"]:
+                    mark["tokens"], mark["last"] = tokens, now
+                    if mark["first"] is None:
+                        mark["first"] = now
+        return marks
+
+    staggered()  # warm-up
+    timed([request(16, 64) for _ in range(concurrency)])
+    torch.cuda.synchronize()
+    short = timed([request(16, 64) for _ in range(concurrency)])
+    short_seconds = max(m["last"] for m in short) - min(m["submit"] for m in short)
+    torch.cuda.synchronize()
+    arriving = staggered()
+    arriving_seconds = max(m["last"] for m in arriving) - min(m["submit"] for m in arriving)
     return {
+        "model": model_name + " layer sizes",
+        "mixed_steps_recorded": mixed_graphs,
+        "short_prompts_16x16_tok_s": round(sum(m["tokens"] for m in short) / short_seconds, 1),
+        "short_prompts_16x16_ttft_ms": round(statistics.median((m["first"] - m["submit"]) * 1e3 for m in short), 2),
+        "short_prompts_arriving_tok_s": round(sum(m["tokens"] for m in arriving) / arriving_seconds, 1),
+        "short_prompts_arriving_ttft_ms": round(statistics.median((m["first"] - m["submit"]) * 1e3 for m in arriving), 2),
         "prompt_tokens": prompt_len,
         "new_tokens": new_tokens,
         "tokens_per_step": 4096,
@@ -405,6 +445,9 @@ def main() -> int:
         help="instead of the default run: for each context length C, prompts of C-40 tokens prefilled in portions "
         "of 8,192 and decoded to C positions, at batch 1 and at --batch; prints one JSON line and exits",
     )
+    parser.add_argument("--no-mixed-graphs", action="store_true",
+                        help="with --serving / --reference-workload: launch steps that have portions of prompts in them kernel "
+                        "by kernel, however few their tokens (recorded steps of single tokens stay)")
     parser.add_argument("--attention-batch", type=int, default=0)
     parser.add_argument("--attention-repeats", type=int, default=20)
     args = parser.parse_args()
@@ -592,11 +635,11 @@ def main() -> int:
     if args.serving:
         del runner
         torch.cuda.empty_cache()
-        line["serving"] = measure_serving(args.dtype)
+        line["serving"] = measure_serving(args.dtype, not args.no_mixed_graphs)
     if args.reference_workload:
         runner = None
         torch.cuda.empty_cache()
-        line["reference_workload"] = measure_reference_workload(args.dtype)
+        line["reference_workload"] = measure_reference_workload(args.dtype, not args.no_mixed_graphs, args.sizes)
     print(json.dumps(line), flush=True)
     return 0
 

@@ -27,6 +27,10 @@ from mini_infer_amd.weights import load_checkpoint
 from mini_infer_amd.weights.random_init import fill_random_on_device
 
 _DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+# Steps of single tokens are recorded up to this many requests (in buckets of powers of two).  At
+# the widths of a 3B model a step of 128 single tokens keeps the device busy for about as long as
+# the host needs to launch it kernel by kernel; beyond 256 the device is the slower of the two.
+MAX_RECORDED_BATCH = 256
 
 
 def resolve_dtype(dtype: str | torch.dtype | None) -> torch.dtype:
@@ -85,7 +89,7 @@ class ModelRunner:
         self.last_row_slots: torch.Tensor | None = None
         # small steps (single tokens, and few tokens with portions among them) are replayed as HIP
         # graphs where every part of the model allows it
-        self.decode_graphs = DecodeGraphs(self, max_batch=64) if cuda_graph and model.graph_safe else None
+        self.decode_graphs = DecodeGraphs(self, max_batch=MAX_RECORDED_BATCH) if cuda_graph and model.graph_safe else None
 
     # -- construction -----------------------------------------------------------
 

@@ -359,23 +359,27 @@ def test_sixty_four_requests_past_two_thousand_tokens_in_recorded_steps(wide):
     runner.cache.check()
 
 
+@pytest.mark.parametrize("recorded", [False, True])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_hundred_single_tokens_in_one_step(wide, dtype):
-    """100 requests bring one token each to the same step: more rows than any recorded decode
-    step takes, so the step is launched kernel by kernel (o and down in partial sums up to 128
-    rows, the vendor library's products for the rest, decode attention over 100 requests)."""
+def test_a_hundred_single_tokens_in_one_step(wide, dtype, recorded):
+    """100 requests bring one token each to the same step (o and down in partial sums up to 128
+    rows, the vendor library's products for the rest, decode attention over 100 requests): once
+    launched kernel by kernel, once as the recorded step of 128 rows with 28 padding rows."""
     from mini_infer_amd.engine import ModelRunner, StepEntry
 
     folder, oracle = wide
     lengths = [17 + (13 * i) % 181 for i in range(100)]
     requests = {f"h{i}": tiny.random_tokens(WIDE, n + 1, seed=700 + i) for i, n in enumerate(lengths)}
-    runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=100 * 13, block_size=16, max_concurrent=100)
+    runner = ModelRunner.from_pretrained(folder, dtype=dtype, num_blocks=100 * 13, block_size=16, max_concurrent=100,
+                                         cuda_graph=recorded)
     ids = list(requests)
     for first in range(0, 100, 10):
         runner.step([StepEntry(rid, requests[rid][: lengths[ids.index(rid)]], []) for rid in ids[first : first + 10]])
-    replays = runner.decode_graphs.replays
     got = runner.step([StepEntry(rid, [requests[rid][n]], [0]) for rid, n in zip(ids, lengths)]).cpu().numpy()
-    assert runner.decode_graphs.replays == replays  # not a recorded step
+    if recorded:
+        assert runner.decode_graphs.replays == 1 and [key for key in runner.decode_graphs.graphs if len(key) == 2] == [(128, 16)]
+    else:
+        assert runner.decode_graphs is None
     for row, (rid, n) in enumerate(zip(ids, lengths)):
         expected = oracle(requests[rid], rows=[n])
         ru.assert_close(got[row : row + 1], expected, dtype, f"8B widths, 100 rows, {rid} ({n} tokens)")
