@@ -255,11 +255,11 @@ class DecodeGraphs:
         )
 
     def takes_mixed(self, index, wants: list, device_tokens: torch.Tensor | None = None) -> bool:
-        """Whether a step with a portion in it is replayed: few tokens, at most one wanted row a request."""
+        """Whether a step that is not one of single tokens with every row wanted is replayed: few
+        tokens, at most one wanted row a request."""
         total = int(index.cu_seqlens_q[-1])
         return (
             self.mixed
-            and index.max_q_len > 1
             and total <= MIXED_MAX_TOKENS
             and all(len(w) <= 1 for w in wants)
             and (device_tokens is None or device_tokens.numel() <= self.max_batch)

@@ -621,8 +621,9 @@ def test_small_steps_with_portions_are_recorded_by_bucket_and_replayed_with_othe
     step(("e", 16, False), ("a", 1, True))  # 17 tokens: (32, 4) again, the new request on d's pages
     step(("e", 14, True), ("a", 2, True), ("b", 2, True), ("c", 2, True))  # 20 tokens, 4 requests, none to spare: (32, 8)
     step(("e", 16, True))  # exactly the bucket's tokens: (16, 1)
+    step(("a", 1, True), ("b", 1, False))  # single tokens, but one of them wants nothing: (16, 4) once more
     assert set(graphs.graphs) == {(32, 4, 16), (16, 4, 16), (4, 16), (16, 2, 16), (32, 8, 16), (16, 1, 16)}
-    assert graphs.mixed_replays == 8 and graphs.replays == 1
+    assert graphs.mixed_replays == 9 and graphs.replays == 1
     # a step of more tokens than the largest bucket, or one that wants two rows of a request, is launched kernel by kernel
     before = graphs.mixed_replays
     runner.step([StepEntry("a", requests["a"][fed["a"] : fed["a"] + 3], [0, 2])])
