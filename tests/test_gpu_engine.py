@@ -849,6 +849,21 @@ def test_layers_with_and_without_a_window_have_page_groups_of_their_own(tmp_path
         ru.assert_close(got["y"], expected["y"], dtype, "windowed y")
         runner.cache.check()
         assert all(g.pool.num_free == 10 for g in runner.cache.groups)
+        if dtype == "float32":
+            # through the scheduler: portions under a small budget beside single tokens (recorded
+            # steps with portions in them), pages the window has passed given back on the way
+            from mini_infer_amd.engine.llm import LLM
+
+            llm = LLM(folder, dtype=dtype, num_blocks=24, block_size=4, max_num_batched_tokens=24, chunk_size=16, max_concurrent=3)
+            prompts = [tiny.random_tokens(cfg, n, seed=90 + n) for n in (21, 5, 34, 12)]
+            for prompt, result in zip(prompts, llm.generate(prompts, max_tokens=7)):
+                sequence = list(prompt)
+                for _ in range(7):
+                    sequence.append(pl.greedy(pl.llama_logits(cfg, weights, np.array(sequence), window=[6, None, 6])[-1]))
+                assert result.tokens == sequence[len(prompt):] and result.finish_reason == "length"
+            assert llm.runner.decode_graphs.mixed_replays > 0 and llm.runner.decode_graphs.replays > 0
+            llm.runner.cache.check()
+            assert all(g.pool.num_free == 24 for g in llm.runner.cache.groups)
     finally:
         ARCHITECTURES.unregister("WindowedTestLM")
 
