@@ -607,6 +607,29 @@ def test_float32_product_is_rounded_once():
     assert torch.equal(ops.gemm_f32(a[:7], w), ops.gemm_f32(a, w)[:7])  # a row's bits do not depend on its company
 
 
+@pytest.mark.parametrize("mode,dtype", ATTENTION_MODES)
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,window", [(8, 2, 64, None), (32, 8, 128, 50), (6, 3, 96, None)])
+def test_paged_attention_with_request_boundaries_known_on_the_device_only(mode, dtype, q_heads, kv_heads, head_dim, window):
+    """What a recorded step with portions in it asks of the attention: `host_cu_seqlens_q=None`,
+    the launch shaped by the number of tokens and requests alone; requests that bring no token
+    (here two, at the end, as the padding of a bucket leaves them) are passed over."""
+    from mini_infer_amd import ops
+
+    page_size = 16
+    lengths, q_lens = [300, 41, 1500, 90, 64], [70, 1, 1, 33, 2]
+    case = _paged_case(dtype, q_heads, kv_heads, head_dim, page_size, lengths, q_lens, seed=21, v_transposed=mode == "mfma")
+    tokens = case["q"].shape[0]
+    cu = torch.tensor(case["host_cu"] + [tokens, tokens], dtype=torch.int32, device=DEV)
+    table = torch.cat([case["block_table"], torch.zeros((2, case["block_table"].shape[1]), dtype=torch.int32, device=DEV)])
+    scale = 1.0 / math.sqrt(head_dim)
+    out = ops.paged_attention(
+        case["q"], case["k_pages"], case["v_pages"], table, case["token_request"], case["positions"], cu, None,
+        q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, scale=scale, window=window, max_seq_len=2048,
+        v_transposed=case["v_transposed"])
+    expected = _attention_expected(case, scale, window)
+    assert np.abs(out.double().cpu().numpy() - expected).max() < _tol(dtype, 2)
+
+
 @pytest.mark.parametrize("window", [None, 700])
 def test_paged_attention_whole_long_prompts_many_tiles(window):
     """Whole prompts of a few thousand tokens beside a short one: dozens of tiles per head,
